@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Benchmark of the GPTQ 3-bit matvec (K=4096, N=11008, fp32 activations) on one
+MI355X: achieved HBM GB/s (algorithmic bytes / time per call) and microseconds per
+call, with weights rotated over more than 512 MB of distinct buffers so that no
+call is served from the 256 MB Infinity Cache.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
+
+Prints ONE JSON line.  A step is one hq_q3_matvec call (one kernel launch)."""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, vendor figure
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+K, N = 4096, 11008
+ROWS = 3 * K // 32
+ALGO_BYTES = ROWS * N * 4 + 2 * N * 4 + K * 4 + N * 4   # weights + scale/zero + x + y = 17,056,768
+
+
+def _time_loop(fn, n_buffers, steps, warmup):
+    """Event-timed back-to-back launches on torch's current stream (the stream the
+    kernels are enqueued on).  Returns seconds for `steps` calls."""
+    import torch
+    for i in range(warmup):
+        fn(i % n_buffers)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(steps):
+        fn(i % n_buffers)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3
+
+
+def bench_q3(steps, warmup, hot=False):
+    import torch
+    import hecbench_amd as hq
+    from hecbench_amd import _lib
+    dev = torch.device("cuda:0")
+    lib = _lib.load()
+    n_buf = 1 if hot else 34           # 34 x 16.9 MB = 575 MB of distinct weights
+    g = torch.Generator(device=dev)
+    g.manual_seed(1234)
+    # any 32-bit pattern is a valid string of 3-bit codes: uniform random words = uniform codes
+    mats = [torch.randint(-2 ** 31, 2 ** 31 - 1, (ROWS, N), dtype=torch.int32, device=dev, generator=g)
+            for _ in range(n_buf)]
+    scales = torch.empty(N, device=dev).uniform_(0.005, 0.02, generator=g)
+    zeros = scales * torch.randint(3, 5, (N,), device=dev, generator=g).float()
+    x = torch.randn(K, device=dev, generator=g)
+    y = torch.empty(N, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    px, ps, pz, py = (ctypes.c_void_p(t.data_ptr()) for t in (x, scales, zeros, y))
+    pm = [ctypes.c_void_p(m.data_ptr()) for m in mats]
+
+    def call(i):
+        rc = lib.hq_q3_matvec(px, 0, pm[i], ps, pz, py, K, N, 1, 0, stream)
+        if rc:
+            raise RuntimeError(lib.hq_strerror(rc).decode())
+
+    secs = _time_loop(call, n_buf, steps, warmup)
+    return secs, dict(x=x, scales=scales, zeros=zeros, mat0=mats[0], y=y, call=call)
+
+
+def cpu_baseline_q3(state, budget_s=12.0):
+    """The oracle's serial restatement of the reference fp32 kernel on one host core,
+    on weight buffer 0; doubles as the correctness check of the timed GPU buffers."""
+    import numpy as np
+    import torch
+    from tests import oracle_api as oa
+    from tests.tol import rel_err
+    o = oa.load_oracle()
+    mat = state["mat0"].cpu().numpy()
+    x = state["x"].cpu().numpy()
+    s = state["scales"].cpu().numpy()
+    z = state["zeros"].cpu().numpy()
+    state["call"](0)
+    torch.cuda.synchronize()
+    got = state["y"].cpu().numpy()
+    t0 = time.perf_counter()
+    ref = o.q3_matvec_f32(x, mat, s, z)
+    one = time.perf_counter() - t0
+    err = rel_err(got, ref)
+    reps = max(3, int(budget_s / max(one, 1e-3)))
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        o.q3_matvec_f32(x, mat, s, z)
+    per = (time.perf_counter() - t0) / reps
+    return {"value": round(ALGO_BYTES / per / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "us_per_call": round(per * 1e6, 1),
+            "sample": f"{reps} serial calls of the oracle's fp32 restatement (4096x11008, one weight buffer)",
+            "gpu_vs_oracle_max_rel_err": err}
+
+
+def bench_others(steps, warmup):
+    """Microseconds per call and algorithmic GB/s of the other configurations."""
+    import numpy as np
+    import torch
+    import hecbench_amd as hq
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(99)
+    out = {}
+    # config 0: NF4 dequant 4096x4096, blocksize 64 (rotate 14 x 43 MB)
+    n = 4096 * 4096
+    nb = 14
+    packed = [torch.randint(0, 256, (n // 2,), dtype=torch.uint8, device=dev, generator=g) for _ in range(nb)]
+    absmax = [torch.empty(n // 64, device=dev).uniform_(0.5, 2.0, generator=g) for _ in range(nb)]
+    outs = [torch.empty(n, dtype=torch.float16, device=dev) for _ in range(nb)]
+    secs = _time_loop(lambda i: hq.dequant_4bit(packed[i], absmax[i], n, 64, 0, out=outs[i]), nb, steps, warmup)
+    b = n // 2 + n // 64 * 4 + 64 + n * 2
+    out["nf4_dequant_4096x4096"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
+                                    "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
+    del packed, absmax, outs
+    # config 2: LUT-GEMM K=4096 N=16384 q=3 G=128 (rotate 20 x 29 MB)
+    Kl, Nl = 4096, 16384
+    nb = 20
+    bW = [torch.randint(-2 ** 31, 2 ** 31 - 1, (Kl // 32, 3, Nl), dtype=torch.int32, device=dev, generator=g)
+          for _ in range(nb)]
+    alpha = [(torch.randn(Kl // 128, 3, Nl, device=dev, generator=g) * 0.02).abs().half() for _ in range(nb)]
+    qb = torch.zeros(Kl // 128, Nl, dtype=torch.float16, device=dev)
+    xl = torch.randn(Kl, device=dev, generator=g).half()
+    yl = torch.empty(Nl, dtype=torch.float16, device=dev)
+    secs = _time_loop(lambda i: hq.lut_matmul(xl, bW[i], alpha[i], qb, 128, out=yl), nb, steps, warmup)
+    b = Kl // 32 * 3 * Nl * 4 + Kl // 128 * 3 * Nl * 2 + Kl // 128 * Nl * 2 + Kl * 2 + Nl * 2
+    out["lut_gemv_4096x16384_q3"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
+                                     "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
+    del bW, alpha
+    # config 3: AQLM 4096x4096 (rotate 128 x 4 MB of codes; the 1 MB code book is shared)
+    Ma, Ka = 4096, 4096
+    nb = 128
+    codes = [torch.randint(-32768, 32768, (Ma, Ka // 8), dtype=torch.int16, device=dev, generator=g)
+             for _ in range(nb)]
+    cb = (torch.randn(65536, 8, device=dev, generator=g) * 0.05).half()
+    sc = torch.empty(Ma, device=dev).uniform_(0.5, 1.5, generator=g).half()
+    xa = torch.randn(Ka, device=dev, generator=g).half()
+    ya = torch.empty(Ma, dtype=torch.float16, device=dev)
+    secs = _time_loop(lambda i: hq.code1x16_matvec(codes[i], xa, cb, (Ma, 0, 0, 0), 65536, scales=sc, out=ya),
+                      nb, steps, warmup)
+    b = Ma * Ka // 8 * 2 + 65536 * 16 + 3 * Ka * 2
+    out["aqlm_4096x4096"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
+                             "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS,
+                             "gather_GBps": (Ma * Ka // 8 * 16) * steps / secs / 1e9}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--all", action="store_true", help="also time the other configurations")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this path has no collective and every box here has one GPU; "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (no CPU path exists for the product kernels)", file=sys.stderr)
+        sys.exit(2)
+    import hecbench_amd as hq
+    hq.init()
+    info = hq.device_info()
+
+    secs, state = bench_q3(args.steps, args.warmup)
+    us = secs / args.steps * 1e6
+    gbs = ALGO_BYTES / (secs / args.steps) / 1e9
+    hot_secs, _ = bench_q3(args.steps, args.warmup, hot=True)
+    result = {
+        "metric": "achieved HBM GB/s: GPTQ-3bit matvec 4096x11008 (algorithmic bytes / time per call)",
+        "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us * 1e-3, 6), "us_per_call": round(us, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "GPTQ 3-bit matvec K=4096 N=11008 batch 1, fp32 x, weights rotated over 34 "
+                               "distinct 16.9 MB buffers (575 MB)", "algorithmic_bytes_per_call": ALGO_BYTES},
+        "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
+        "effective_fp16_weight_GBps": round(K * N * 2 / (secs / args.steps) / 1e9, 1),
+        "hot_cache_us_per_call": round(hot_secs / args.steps * 1e6, 3),
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+        "device": info,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline_q3(state)
+    if args.all:
+        result["other_configs"] = bench_others(max(200, args.steps // 8), 50)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

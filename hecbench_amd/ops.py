@@ -1,0 +1,130 @@
+"""Operator-level wrappers: same names, argument meaning and error behaviour as
+the reference launch wrappers, over the C ABI.  No arithmetic happens here."""
+import ctypes
+
+import torch
+
+from . import _lib
+
+NF4 = 0
+FP4 = 1
+_F32, _F16 = 0, 1
+_ACCUMULATE = 1
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise ValueError("hecbench_amd operators take device tensors only (no CPU path)")
+        if t is not None and not t.is_contiguous():
+            raise ValueError("hecbench_amd operators take contiguous tensors")
+
+
+def init():
+    _lib.check(_lib.load().hq_init(), "hq_init")
+
+
+def device_info():
+    lib = _lib.load()
+    v = [ctypes.c_int() for _ in range(5)]
+    name = ctypes.create_string_buffer(256)
+    _lib.check(lib.hq_device_info(*[ctypes.byref(x) for x in v], name, 256), "hq_device_info")
+    return {"compute_units": v[0].value, "wavefront_size": v[1].value, "lds_bytes_per_cu": v[2].value,
+            "memory_clock_khz": v[3].value, "memory_bus_bits": v[4].value, "name": name.value.decode()}
+
+
+def q3_matvec(x, qweight, scales, zeros, out=None, accumulate=False):
+    """y[n] = sum_k x[k]*(scales[n]*q[k][n] - zeros[n]); x fp32 or fp16 [K]."""
+    _dev(x, qweight, scales, zeros, out)
+    K = x.numel()
+    N = qweight.shape[1]
+    if qweight.shape[0] * 32 != 3 * K:
+        raise ValueError("qweight must have 3*K/32 packed rows")
+    if out is None:
+        out = torch.empty(N, dtype=torch.float32, device=x.device)
+    dt = _F16 if x.dtype == torch.float16 else _F32
+    if x.dtype not in (torch.float16, torch.float32):
+        raise ValueError("x must be fp32 or fp16")
+    rc = _lib.load().hq_q3_matvec(_ptr(x), dt, _ptr(qweight), _ptr(scales), _ptr(zeros), _ptr(out), K, N, 1,
+                                  _ACCUMULATE if accumulate else 0, _stream())
+    _lib.check(rc, "hq_q3_matvec")
+    return out
+
+
+def vecquant3matmul(vec, mat, mul, scales, zeros, height=None, width=None):
+    """Reference signature (src/quant3MatMul-hip/kernels.h:171-190): mul += vec @ W."""
+    q3_matvec(vec.reshape(-1), mat, scales, zeros, out=mul.reshape(-1), accumulate=True)
+
+
+def vecquant3matmul_faster(vec, mat, mul, scales, zeros, height=None, width=None):
+    """Reference signature (src/quant3MatMul-hip/kernels.h:193-217): fp16 vec, mul += vec @ W."""
+    if vec.dtype != torch.float16:
+        raise ValueError("vecquant3matmul_faster takes an fp16 vector")
+    q3_matvec(vec.reshape(-1), mat, scales, zeros, out=mul.reshape(-1), accumulate=True)
+
+
+def q3_gemm(A, qweight, scales, zeros, out=None):
+    """out[m][n] = sum_k A[m][k]*(scales[n]*q[k][n] - zeros[n]); A fp16 [M][K]."""
+    _dev(A, qweight, scales, zeros, out)
+    M, K = A.shape
+    N = qweight.shape[1]
+    if out is None:
+        out = torch.empty(M, N, dtype=torch.float32, device=A.device)
+    rc = _lib.load().hq_q3_matvec(_ptr(A), _F16, _ptr(qweight), _ptr(scales), _ptr(zeros), _ptr(out), K, N, M,
+                                  0, _stream())
+    _lib.check(rc, "hq_q3_matvec(batch)")
+    return out
+
+
+def dequant_4bit(packed, absmax, n_elems, blocksize, table=NF4, out=None):
+    _dev(packed, absmax, out)
+    if out is None:
+        out = torch.empty(n_elems, dtype=torch.float16, device=packed.device)
+    rc = _lib.load().hq_dequant_nf4(_ptr(packed), _ptr(absmax), _ptr(out), n_elems, blocksize, table, _stream())
+    _lib.check(rc, "hq_dequant_nf4")
+    return out
+
+
+def quantize_dynamic8(code, A, out=None):
+    _dev(code, A, out)
+    if out is None:
+        out = torch.empty(A.numel(), dtype=torch.uint8, device=A.device)
+    rc = _lib.load().hq_quantize_dynamic8(_ptr(code), _ptr(A), _ptr(out), A.numel(), _stream())
+    _lib.check(rc, "hq_quantize_dynamic8")
+    return out
+
+
+def lut_matmul(x, bW, alpha, q_bias, group_size, out=None):
+    """matmul(output, input, nqW, m) of src/lut-gemm-hip/kernels.cu:27-31.
+    bW uint32/int32 [K/32][nb][N], alpha fp16 [K/G][nb][N], q_bias fp16 [K/G][N] or None."""
+    _dev(x, bW, alpha, q_bias, out)
+    K = x.numel()
+    nb, N = bW.shape[1], bW.shape[2]
+    if out is None:
+        out = torch.empty(N, dtype=torch.float16, device=x.device)
+    rc = _lib.load().hq_lut_gemv(_ptr(bW), _ptr(alpha), _ptr(q_bias), _ptr(x), _ptr(out), K, N, nb, group_size,
+                                 _stream())
+    _lib.check(rc, "hq_lut_gemv")
+    return out
+
+
+def code1x16_matvec(codes, x, codebooks, codebook_a_sizes, codebook_stride_int4, scales=None, out=None):
+    """code1x16_matvec of src/quantAQLM-hip/main.cu:103-139 (plus the optional row scale)."""
+    _dev(codes, x, codebooks, scales, out)
+    M = codes.shape[0]
+    K = x.numel()
+    if out is None:
+        out = torch.empty(M, dtype=torch.float16, device=x.device)
+    sizes = (ctypes.c_int * 4)(*codebook_a_sizes)
+    rc = _lib.load().hq_aqlm_matvec(_ptr(codes), _ptr(codebooks), _ptr(scales), _ptr(x), _ptr(out), M, K, sizes,
+                                    codebook_stride_int4, _stream())
+    _lib.check(rc, "hq_aqlm_matvec")
+    return out

@@ -1,0 +1,142 @@
+/*
+ * hq.h — C ABI of libhq: weight-only quantized-inference kernels for AMD
+ * Instinct MI355X (gfx950 / CDNA4).
+ *
+ * The entry points replace the host launch wrappers of the HeCBench benchmarks
+ * quant3MatMul, lut-gemm, quantAQLM and quantBnB (citations are relative to the
+ * HeCBench tree).  Conventions shared by every entry point:
+ *
+ *   - all data pointers are DEVICE pointers owned by the caller;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     calls are asynchronous on that stream and never synchronise;
+ *   - outputs are OVERWRITTEN unless HQ_FLAG_ACCUMULATE is given, so no
+ *     pre-zeroing memset is needed (the reference wrappers accumulate with
+ *     atomics and make the caller memset first);
+ *   - return value: 0 on success, a negative HQ_ERR_* code for a rejected
+ *     argument (nothing is launched), or a positive hipError_t value;
+ *   - nothing is printed; hq_strerror() turns a code into text;
+ *   - the library keeps one small per-device workspace (split-K partial sums
+ *     and arrival counters, allocated by hq_init() or by the first call on a
+ *     device); calls that share a device must not overlap in time on different
+ *     streams unless stated otherwise below.
+ */
+#ifndef HQ_H
+#define HQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HQ_OK 0
+#define HQ_ERR_NULL_POINTER (-1)
+#define HQ_ERR_BAD_SHAPE (-2)
+#define HQ_ERR_BAD_ENUM (-3)
+#define HQ_ERR_MISALIGNED (-4)
+#define HQ_ERR_UNSUPPORTED_DEVICE (-5)
+#define HQ_ERR_TOO_LARGE (-6)
+
+/* element types of the activation vector / matrix */
+#define HQ_DTYPE_F32 0
+#define HQ_DTYPE_F16 1
+
+/* flags */
+#define HQ_FLAG_ACCUMULATE 1u /* y += result (reference wrapper semantics) */
+
+/* 4-bit code books of hq_dequant_4bit */
+#define HQ_TABLE_NF4 0
+#define HQ_TABLE_FP4 1
+
+/* Version of this ABI (bumped on incompatible change). */
+int hq_abi_version(void);
+
+/* Text for a return code of this library (HQ_ERR_* or a hipError_t value). */
+const char* hq_strerror(int code);
+
+/* Prepare the current HIP device: checks that it is a gfx950 part, allocates
+ * the per-device workspace.  Optional (the first compute call does the same),
+ * but calling it keeps the allocation out of the first timed call.
+ * Mirrors the device query of the AQLM launcher, src/quantAQLM-hip/main.cu:108-121. */
+int hq_init(void);
+
+/* Device facts the benchmark drivers print next to the roofline numbers.
+ * Any pointer may be NULL. */
+int hq_device_info(int* compute_units, int* wavefront_size, int* lds_bytes_per_cu,
+                   int* memory_clock_khz, int* memory_bus_bits, char* name, int name_len);
+
+/*
+ * Blockwise 4-bit dequantisation to fp16 (NF4 or FP4 code book).
+ *   out[2i]   = fp16_rn(table[packed[i] >> 4]  * absmax[(2i)   / blocksize])
+ *   out[2i+1] = fp16_rn(table[packed[i] & 15]  * absmax[(2i+1) / blocksize])
+ * fp32 multiply, one round-to-nearest-even to fp16 (bit-exact contract).
+ * n_elems >= 0; blocksize > 0 and even.  Stands in the place of the quantBnB
+ * benchmark's kernel launch, src/quantBnB-hip/main.cu:176 (the reference
+ * benchmark itself holds the 8-bit quantiser, see hq_quantize_dynamic8).
+ */
+int hq_dequant_nf4(const uint8_t* packed, const float* absmax, void* out_fp16,
+                   int64_t n_elems, int blocksize, int table, void* stream);
+
+/*
+ * bitsandbytes dynamic-map 8-bit quantisation: out[i] = index of the entry of
+ * the sorted 256-entry table `code` nearest to A[i], with the reference's
+ * search and tie rules.  Replaces kQuantize<256,256><<<...>>>(code, A, out, n),
+ * src/quantBnB-hip/main.cu:90-130,176.  Bit-exact contract.
+ */
+int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_t n,
+                         void* stream);
+
+/*
+ * GPTQ 3-bit matvec / batched GEMM:
+ *   y[m][n] = sum_k x[m][k] * (scales[n] * q[k][n] - zeros[n]),  m < batch_M
+ * qweight is int32[3*K/32][N] row-major: the 32 codes of k-group g of column n
+ * form a 96-bit little-endian string in words qweight[(3g+j)*N + n], j=0..2,
+ * code i at bits 3i..3i+2 (src/quant3MatMul-hip/kernels.h:42-86).  zeros holds
+ * the pre-multiplied scale*zero_point.
+ *   x        : [batch_M][K] row-major, fp32 (HQ_DTYPE_F32) or fp16 (HQ_DTYPE_F16)
+ *   y        : fp32 [batch_M][N]
+ *   K % 32 == 0, N % 4 == 0, batch_M >= 1; qweight 16-byte aligned.
+ * Products are accumulated in fp32 for both dtypes (the reference's fp16
+ * variant accumulates 16 terms in fp16; this library is never less accurate).
+ * batch_M == 1 replaces vecquant3matmul / vecquant3matmul_faster
+ * (src/quant3MatMul-hip/kernels.h:171-217) — pass HQ_FLAG_ACCUMULATE for their
+ * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 and runs the
+ * MFMA GEMM path (no counterpart in the reference).
+ */
+int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float* scales,
+                 const float* zeros, float* y, int K, int N, int batch_M, unsigned flags,
+                 void* stream);
+
+/*
+ * LUT-GEMM binary-coded-quantisation matvec (fp16 in, fp16 out):
+ *   y[n] = sum_k x[k] * ( q_bias[k/G][n] + sum_b alpha[k/G][b][n] * s(k,b,n) ),
+ *   s = +1 if bit (k%32) of bW[k/32][b][n] is set, else -1
+ * Layouts (src/lut-gemm-hip/nQWeight_fp16.h:24-26): bW uint32[K/32][nbits][N],
+ * alpha fp16[K/G][nbits][N], q_bias fp16[K/G][N] or NULL, x fp16[K], y fp16[N].
+ * K % 32 == 0, G % 32 == 0, K % G == 0, 1 <= nbits <= 8.
+ * Sums are kept in fp32 and rounded to fp16 once.  Replaces
+ * matmul(output, input, nqW, m), src/lut-gemm-hip/kernels.cu:27-31.
+ */
+int hq_lut_gemv(const uint32_t* bW, const void* alpha_fp16, const void* q_bias_fp16,
+                const void* x_fp16, void* y_fp16, int K, int N, int nbits, int group_size,
+                void* stream);
+
+/*
+ * AQLM 1x16 code-book matvec (fp16 in, fp16 out):
+ *   y[m] = fp16_rn( scale[m] * sum_g dot8(codebook[cb(m)][u16(codes[m][g])], x[8g..8g+7]) )
+ * codes int16[M][K/8] (read as unsigned), codebooks fp16[..][65536][8] with
+ * consecutive code books codebook_stride_int4*16 bytes apart, cb(m) = first j
+ * with m < codebook_a_sizes[j].  scales_fp16 may be NULL (the reference kernel
+ * applies no scale).  K % 8 == 0.  fp32 accumulation, one rounding.  Replaces
+ * code1x16_matvec, src/quantAQLM-hip/main.cu:103-139 (without its internal
+ * synchronisation, timing and printing).
+ */
+int hq_aqlm_matvec(const int16_t* codes, const void* codebooks_fp16, const void* scales_fp16,
+                   const void* x_fp16, void* y_fp16, int M, int K,
+                   const int codebook_a_sizes[4], int codebook_stride_int4, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HQ_H */

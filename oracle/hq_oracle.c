@@ -1,0 +1,464 @@
+/*
+ * hq_oracle.c — CPU restatement of the reference arithmetic.  TEST
+ * INFRASTRUCTURE ONLY (see hq_oracle.h): never linked into the product library.
+ *
+ * Build: gcc -O2 -ffp-contract=off -fPIC -shared hq_oracle.c -o libhq_oracle.so -lm
+ * (-ffp-contract=off matters: the fp32 restatements round after every multiply
+ * and add, which is what the functions below document).
+ */
+#include "hq_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------ fp16 */
+
+static double round_to_f16_grid(double d) {
+  /* Round a double to the nearest binary16 value (ties to even); the result is
+   * returned as a double that binary16 represents exactly (or +-inf). */
+  if (d != d || isinf(d)) return d;
+  double a = fabs(d);
+  if (a == 0.0) return d;
+  int e;
+  (void)frexp(a, &e); /* a = m * 2^e, m in [0.5,1) => floor(log2 a) = e-1 */
+  int q = e - 1 - 10; /* exponent of the last kept bit (11-bit significand) */
+  if (q < -24) q = -24; /* subnormal quantum */
+  double quantum = ldexp(1.0, q);
+  double r = rint(a / quantum) * quantum; /* rint: ties-to-even by default */
+  if (r >= 65520.0) r = INFINITY;        /* overflow threshold of binary16 */
+  return d < 0 ? -r : r;
+}
+
+uint16_t hqo_f64_to_f16(double d) {
+  if (d != d) return 0x7e00;
+  double r = round_to_f16_grid(d);
+  uint16_t sign = signbit(r) ? 0x8000 : 0;
+  double a = fabs(r);
+  if (isinf(a)) return sign | 0x7c00;
+  if (a == 0.0) return sign;
+  int e;
+  double m = frexp(a, &e); /* a = m*2^e, m in [0.5,1) */
+  int E = e - 1;           /* unbiased exponent */
+  if (E < -14) {           /* subnormal: a = frac * 2^-24 */
+    return sign | (uint16_t)(a * 16777216.0);
+  }
+  uint16_t frac = (uint16_t)((m * 2.0 - 1.0) * 1024.0);
+  return sign | (uint16_t)((E + 15) << 10) | frac;
+}
+
+uint16_t hqo_f32_to_f16(float f) { return hqo_f64_to_f16((double)f); }
+
+float hqo_f16_to_f32(uint16_t h) {
+  int s = h >> 15, e = (h >> 10) & 31, m = h & 1023;
+  double v;
+  if (e == 31) v = m ? NAN : INFINITY;
+  else if (e == 0) v = ldexp((double)m, -24);
+  else v = ldexp(1.0 + m / 1024.0, e - 15);
+  return (float)(s ? -v : v);
+}
+
+/* Sum p + c rounded to odd in double, so that a second rounding to binary16 is
+ * the correctly rounded result of the exact sum. */
+static double add_round_to_odd(double p, double c) {
+  double s = p + c;
+  if (s != s || isinf(s)) return s;
+  double bb = s - p;
+  double err = (p - (s - bb)) + (c - bb); /* TwoSum: p + c = s + err exactly */
+  if (err != 0.0) {
+    uint64_t bits;
+    memcpy(&bits, &s, 8);
+    if (!(bits & 1)) s = nextafter(s, err > 0 ? INFINITY : -INFINITY);
+  }
+  return s;
+}
+
+uint16_t hqo_hfma(uint16_t a, uint16_t b, uint16_t c) {
+  double p = (double)hqo_f16_to_f32(a) * (double)hqo_f16_to_f32(b); /* exact */
+  return hqo_f64_to_f16(add_round_to_odd(p, (double)hqo_f16_to_f32(c)));
+}
+uint16_t hqo_hadd(uint16_t a, uint16_t b) {
+  return hqo_f64_to_f16((double)hqo_f16_to_f32(a) + (double)hqo_f16_to_f32(b));
+}
+uint16_t hqo_hmul(uint16_t a, uint16_t b) {
+  return hqo_f64_to_f16((double)hqo_f16_to_f32(a) * (double)hqo_f16_to_f32(b));
+}
+
+/* ------------------------------------------------------------- GPTQ 3bit */
+
+/* Value i (0..31) of a 32-value group lives at bit 3*i of the 96-bit string
+ * formed by the group's three words (word 0 lowest); values 10 and 21 straddle
+ * word boundaries (src/quant3MatMul-hip/kernels.h:55,71). */
+static inline unsigned q3_get(const uint32_t w[3], int i) {
+  int bit = 3 * i, wd = bit >> 5, sh = bit & 31;
+  uint32_t v = w[wd] >> sh;
+  if (sh > 29) v |= w[wd + 1] << (32 - sh);
+  return v & 7u;
+}
+
+void hqo_q3_pack(const uint8_t* codes, int K, int N, int32_t* mat) {
+  int G = K / 32;
+  for (int g = 0; g < G; ++g)
+    for (int n = 0; n < N; ++n) {
+      uint32_t w[3] = {0, 0, 0};
+      for (int i = 0; i < 32; ++i) {
+        uint32_t q = codes[(size_t)(32 * g + i) * N + n] & 7u;
+        int bit = 3 * i, wd = bit >> 5, sh = bit & 31;
+        w[wd] |= q << sh;
+        if (sh > 29) w[wd + 1] |= q >> (32 - sh);
+      }
+      for (int j = 0; j < 3; ++j) mat[(size_t)(3 * g + j) * N + n] = (int32_t)w[j];
+    }
+}
+
+void hqo_q3_unpack(const int32_t* mat, int K, int N, uint8_t* codes) {
+  int G = K / 32;
+  for (int g = 0; g < G; ++g)
+    for (int n = 0; n < N; ++n) {
+      uint32_t w[3];
+      for (int j = 0; j < 3; ++j) w[j] = (uint32_t)mat[(size_t)(3 * g + j) * N + n];
+      for (int i = 0; i < 32; ++i) codes[(size_t)(32 * g + i) * N + n] = (uint8_t)q3_get(w, i);
+    }
+}
+
+void hqo_q3_matvec_f32(const float* x, const int32_t* mat, float* mul,
+                       const float* scales, const float* zeros, int K, int N) {
+  /* One 256-row block (8 groups) at a time, as the reference grid does
+   * (BLOCKWIDTH=256, BLOCKHEIGHT=24, kernels.h:5-6,22-23). */
+  float* res = (float*)malloc(sizeof(float) * (size_t)N);
+  int G = K / 32;
+  for (int g0 = 0; g0 < G; g0 += 8) {
+    for (int n = 0; n < N; ++n) res[n] = 0.f;
+    int g1 = g0 + 8 < G ? g0 + 8 : G;
+    for (int g = g0; g < g1; ++g) {
+      const uint32_t* r0 = (const uint32_t*)mat + (size_t)(3 * g) * N;
+      const uint32_t* r1 = r0 + N;
+      const uint32_t* r2 = r1 + N;
+      for (int i = 0; i < 32; ++i) {
+        float xv = x[32 * g + i];
+        int bit = 3 * i, wd = bit >> 5, sh = bit & 31;
+        const uint32_t* ra = wd == 0 ? r0 : (wd == 1 ? r1 : r2);
+        const uint32_t* rb = wd == 0 ? r1 : r2;
+        if (sh <= 29) {
+          for (int n = 0; n < N; ++n) {
+            float q = (float)((ra[n] >> sh) & 7u);
+            res[n] += (scales[n] * q - zeros[n]) * xv; /* kernels.h:43-84 */
+          }
+        } else {
+          for (int n = 0; n < N; ++n) {
+            float q = (float)(((ra[n] >> sh) | (rb[n] << (32 - sh))) & 7u);
+            res[n] += (scales[n] * q - zeros[n]) * xv;
+          }
+        }
+      }
+    }
+    for (int n = 0; n < N; ++n) mul[n] += res[n]; /* atomicAdd, kernels.h:89 */
+  }
+  free(res);
+}
+
+void hqo_q3_matvec_f64(const double* x, const int32_t* mat, double* y,
+                       const float* scales, const float* zeros, int K, int N) {
+  int G = K / 32;
+  for (int n = 0; n < N; ++n) y[n] = 0.0;
+  for (int g = 0; g < G; ++g)
+    for (int n = 0; n < N; ++n) {
+      uint32_t w[3];
+      for (int j = 0; j < 3; ++j) w[j] = (uint32_t)mat[(size_t)(3 * g + j) * N + n];
+      double s = scales[n], z = zeros[n], acc = 0.0;
+      for (int i = 0; i < 32; ++i) acc += (s * (double)q3_get(w, i) - z) * x[32 * g + i];
+      y[n] += acc;
+    }
+}
+
+void hqo_q3_matvec_f16(const uint16_t* x, const int32_t* mat, float* mul,
+                       const float* scales, const float* zeros, int K, int N) {
+  int G = K / 32;
+  uint16_t qh[8];
+  for (int q = 0; q < 8; ++q) qh[q] = hqo_f32_to_f16((float)q); /* deq2, kernels.h:112-119 */
+  for (int n = 0; n < N; ++n) {
+    uint16_t s16 = hqo_f32_to_f16(scales[n]);  /* kernels.h:121 */
+    uint16_t z16 = hqo_f32_to_f16(-zeros[n]);  /* kernels.h:122 */
+    for (int g0 = 0; g0 < G; g0 += 8) {
+      float res = 0.f;
+      int g1 = g0 + 8 < G ? g0 + 8 : G;
+      for (int g = g0; g < g1; ++g) {
+        uint32_t w[3];
+        for (int j = 0; j < 3; ++j) w[j] = (uint32_t)mat[(size_t)(3 * g + j) * N + n];
+        uint16_t ax = 0, ay = 0; /* res2 = half2(0), kernels.h:135 */
+        for (int p = 0; p < 16; ++p) {
+          uint16_t wl = hqo_hfma(qh[q3_get(w, 2 * p)], s16, z16);
+          uint16_t wh = hqo_hfma(qh[q3_get(w, 2 * p + 1)], s16, z16);
+          ax = hqo_hfma(wl, x[32 * g + 2 * p], ax);
+          ay = hqo_hfma(wh, x[32 * g + 2 * p + 1], ay);
+        }
+        res += hqo_f16_to_f32(ax) + hqo_f16_to_f32(ay); /* kernels.h:165 */
+      }
+      mul[n] += res; /* kernels.h:168 */
+    }
+  }
+}
+
+void hqo_q3_gemm(const uint16_t* A, const int32_t* mat, double* out,
+                 const float* scales, const float* zeros, int M, int K, int N,
+                 int mode) {
+  int G = K / 32;
+  double* Ad = (double*)malloc(sizeof(double) * (size_t)M * K);
+  for (size_t i = 0; i < (size_t)M * K; ++i) Ad[i] = hqo_f16_to_f32(A[i]);
+  double* wcol = (double*)malloc(sizeof(double) * (size_t)K);
+  for (int n = 0; n < N; ++n) {
+    for (int g = 0; g < G; ++g) {
+      uint32_t w[3];
+      for (int j = 0; j < 3; ++j) w[j] = (uint32_t)mat[(size_t)(3 * g + j) * N + n];
+      for (int i = 0; i < 32; ++i) {
+        unsigned q = q3_get(w, i);
+        if (mode == 0) wcol[32 * g + i] = (double)scales[n] * q - (double)zeros[n];
+        else wcol[32 * g + i] = hqo_f16_to_f32(hqo_f32_to_f16(scales[n] * (float)q - zeros[n]));
+      }
+    }
+    for (int m = 0; m < M; ++m) {
+      const double* a = Ad + (size_t)m * K;
+      double acc = 0.0;
+      for (int k = 0; k < K; ++k) acc += a[k] * wcol[k];
+      out[(size_t)m * N + n] = acc;
+    }
+  }
+  free(wcol);
+  free(Ad);
+}
+
+/* --------------------------------------------------------------- NF4/FP4 */
+
+/* bitsandbytes NF4 code book (fp32 literals of the upstream library; the
+ * reference tree holds no NF4 table). */
+const float hqo_nf4_table[16] = {
+    -1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39491748809814453f,
+    -0.28444138169288635f, -0.18477343022823334f, -0.09105003625154495f, 0.0f,
+    0.07958029955625534f, 0.16093020141124725f, 0.24611230194568634f,
+    0.33791524171829224f, 0.44070982933044434f, 0.5626170039176941f,
+    0.7229568362236023f, 1.0f};
+
+/* bitsandbytes FP4 decode tree: bit 3 = sign, low three bits select
+ * {0, 1/192, 2/3, 1, 1/3, 1/2, 1/6, 1/4}. */
+const float hqo_fp4_table[16] = {
+    0.0f, 0.005208333333f, 0.66666667f, 1.0f, 0.33333333f, 0.5f, 0.16666667f, 0.25f,
+    -0.0f, -0.005208333333f, -0.66666667f, -1.0f, -0.33333333f, -0.5f, -0.16666667f, -0.25f};
+
+void hqo_dequant_4bit(const uint8_t* packed, const float* absmax, uint16_t* out,
+                      int64_t n, int blocksize, int table) {
+  const float* T = table ? hqo_fp4_table : hqo_nf4_table;
+  for (int64_t e = 0; e < n; ++e) {
+    uint8_t b = packed[e >> 1];
+    unsigned c = (e & 1) ? (b & 15u) : (b >> 4); /* high nibble first */
+    float v = T[c] * absmax[e / blocksize];      /* one fp32 multiply */
+    out[e] = hqo_f32_to_f16(v);                  /* one rounding to fp16 */
+  }
+}
+
+/* ------------------------------------------------ dynamic 8-bit quantize */
+
+uint8_t hqo_dquantize(const float* code, float x) {
+  /* src/quantBnB-hip/main.cu:17-66 */
+  int pivot = 127, upper_pivot = 255, lower_pivot = 0;
+  float lower = -1.0f, upper = 1.0f;
+  float val = code[pivot];
+  for (int i = 64; i > 0; i >>= 1) {
+    if (x > val) { lower_pivot = pivot; lower = val; pivot += i; }
+    else         { upper_pivot = pivot; upper = val; pivot -= i; }
+    val = code[pivot];
+  }
+  if (upper_pivot == 255) upper = code[upper_pivot];
+  if (lower_pivot == 0) lower = code[lower_pivot];
+  if (x > val) {
+    float midpoint = (upper + val) * 0.5f;
+    return (uint8_t)(x > midpoint ? upper_pivot : pivot);
+  } else {
+    float midpoint = (lower + val) * 0.5f;
+    return (uint8_t)(x < midpoint ? lower_pivot : pivot);
+  }
+}
+
+void hqo_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) out[i] = hqo_dquantize(code, A[i]);
+}
+
+static int cmp_float(const void* a, const void* b) {
+  float x = *(const float*)a, y = *(const float*)b;
+  return (x > y) - (x < y);
+}
+
+static void linspace_f32(float start, float end, int steps, float* o) {
+  /* symmetric float32 linspace: lower half counts up from start, upper half
+   * counts down from end */
+  if (steps == 1) { o[0] = start; return; }
+  float step = (end - start) / (float)(steps - 1);
+  int half = steps / 2;
+  for (int i = 0; i < steps; ++i)
+    o[i] = i < half ? start + step * (float)i : end - step * (float)(steps - 1 - i);
+}
+
+void hqo_dynamic_map(float* code) {
+  /* signed dynamic map, 7 exponent bits, 8 total bits */
+  int cnt = 0;
+  float b[65];
+  for (int i = 0; i < 7; ++i) {
+    int items = (1 << i) + 1;
+    linspace_f32(0.1f, 1.0f, items, b);
+    float sc = (float)pow(10.0, -6 + i);
+    for (int j = 0; j + 1 < items; ++j) {
+      float mean = (b[j] + b[j + 1]) / 2.0f;
+      code[cnt++] = sc * mean;
+      code[cnt++] = -sc * mean;
+    }
+  }
+  code[cnt++] = 0.0f;
+  code[cnt++] = 1.0f;
+  qsort(code, 256, sizeof(float), cmp_float);
+}
+
+/* -------------------------------------------------------------- LUT-GEMM */
+
+void hqo_bcq_pack(const int8_t* signs, int K, int N, int nb, uint32_t* bW) {
+  for (int k0 = 0; k0 < K; k0 += 32)
+    for (int b = 0; b < nb; ++b)
+      for (int n = 0; n < N; ++n) {
+        uint32_t s = 0;
+        for (int t = 0; t < 32; ++t)
+          if (signs[((size_t)(k0 + t) * nb + b) * N + n] > 0) s |= 1u << t;
+        bW[((size_t)(k0 / 32) * nb + b) * N + n] = s;
+      }
+}
+
+void hqo_bcq_dequant(const uint32_t* bW, const uint16_t* alpha, const uint16_t* qbias,
+                     int K, int N, int nb, int group, double* W) {
+  for (int k = 0; k < K; ++k)
+    for (int n = 0; n < N; ++n) {
+      int g = k / group;
+      double w = qbias ? hqo_f16_to_f32(qbias[(size_t)g * N + n]) : 0.0;
+      for (int b = 0; b < nb; ++b) {
+        uint32_t word = bW[((size_t)(k / 32) * nb + b) * N + n];
+        double s = (word >> (k & 31)) & 1u ? 1.0 : -1.0;
+        w += hqo_f16_to_f32(alpha[((size_t)g * nb + b) * N + n]) * s;
+      }
+      W[(size_t)k * N + n] = w;
+    }
+}
+
+void hqo_lut_gemv_f64(const uint32_t* bW, const uint16_t* alpha, const uint16_t* qbias,
+                      const uint16_t* x, double* y, int K, int N, int nb, int group) {
+  int NG = K / group;
+  double* xs = (double*)malloc(sizeof(double) * (size_t)K);
+  for (int k = 0; k < K; ++k) xs[k] = hqo_f16_to_f32(x[k]);
+  for (int n = 0; n < N; ++n) y[n] = 0.0;
+  for (int g = 0; g < NG; ++g) {
+    double xsum = 0.0;
+    for (int k = g * group; k < (g + 1) * group; ++k) xsum += xs[k];
+    for (int b = 0; b < nb; ++b)
+      for (int kw = g * group / 32; kw < (g + 1) * group / 32; ++kw) {
+        const uint32_t* row = bW + ((size_t)kw * nb + b) * N;
+        const uint16_t* al = alpha + ((size_t)g * nb + b) * N;
+        for (int n = 0; n < N; ++n) {
+          uint32_t w = row[n];
+          double s = 0.0;
+          for (int t = 0; t < 32; ++t) s += (w >> t) & 1u ? xs[kw * 32 + t] : -xs[kw * 32 + t];
+          y[n] += (double)hqo_f16_to_f32(al[n]) * s;
+        }
+      }
+    if (qbias)
+      for (int n = 0; n < N; ++n) y[n] += (double)hqo_f16_to_f32(qbias[(size_t)g * N + n]) * xsum;
+  }
+  free(xs);
+}
+
+void hqo_lut_gemv_f16(const uint32_t* bW, const uint16_t* alpha, const uint16_t* qbias,
+                      const uint16_t* x, uint16_t* y, int K, int N, int nb, int group) {
+  /* K tile of 32 (the bias path of the reference, mv_fp16.h:252-258) */
+  const uint16_t ONE = 0x3c00, MONE = 0xbc00, TWO = 0x4000;
+  for (int n = 0; n < N; ++n) y[n] = 0; /* hipMemset in matmul(), kernels.cu:28 */
+  uint16_t lut[4][256];
+  for (int kt = 0; kt < K / 32; ++kt) {
+    for (int t = 0; t < 4; ++t) {
+      const uint16_t* inp = x + kt * 32 + t * 8;
+      for (int lx = 0; lx < 64; ++lx) { /* mv_fp16.h:144-153 */
+        uint16_t acc = hqo_hmul((lx & 1) ? ONE : MONE, inp[0]);
+        for (int j = 1; j < 8; ++j)
+          acc = hqo_hadd(acc, hqo_hmul(((lx >> j) & 1) ? ONE : MONE, inp[j]));
+        lut[t][lx] = acc;
+      }
+      for (int s = 6; s < 8; ++s) { /* mv_fp16.h:165-170 */
+        uint16_t iv = hqo_hmul(TWO, inp[s]);
+        for (int i = 1 << s; i < (1 << (s + 1)); ++i) lut[t][i] = hqo_hadd(lut[t][i - (1 << s)], iv);
+      }
+    }
+    int g = (kt * 32) / group;
+    for (int n = 0; n < N; ++n) {
+      uint16_t o = 0;
+      if (qbias) { /* mv_fp16.h:183-201 */
+        uint16_t to = 0;
+        for (int t = 0; t < 4; ++t) to = hqo_hadd(to, lut[t][255]);
+        o = hqo_hadd(o, hqo_hmul(qbias[(size_t)g * N + n], to));
+      }
+      for (int b = 0; b < nb; ++b) { /* mv_fp16.h:203-224 */
+        uint32_t w = bW[((size_t)kt * nb + b) * N + n];
+        uint16_t to = 0;
+        for (int t = 0; t < 4; ++t) to = hqo_hadd(to, lut[t][(w >> (8 * t)) & 255u]);
+        o = hqo_hadd(o, hqo_hmul(alpha[((size_t)g * nb + b) * N + n], to));
+      }
+      y[n] = hqo_hadd(y[n], o); /* unsafeAtomicAdd, mv_fp16.h:225 */
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ AQLM */
+
+void hqo_aqlm_matvec(const int16_t* codes, const uint16_t* codebooks,
+                     const uint16_t* scales, const uint16_t* x, uint16_t* y16,
+                     double* y64, int M, int K, const int cb_a_sizes[4],
+                     int cb_stride_int4, int mode) {
+  int ncodes = K / 8;
+  for (int m = 0; m < M; ++m) {
+    const uint16_t* cb = codebooks;
+    for (int j = 0; j < 4 && m >= cb_a_sizes[j]; ++j)
+      cb += (size_t)cb_stride_int4 * 8; /* main.cu:45-50 */
+    const int16_t* row = codes + (size_t)m * ncodes;
+    double acc = 0.0;
+    if (mode == 0) {
+      for (int c = 0; c < ncodes; ++c) {
+        const uint16_t* e = cb + (size_t)(uint16_t)row[c] * 8; /* main.cu:72 */
+        for (int j = 0; j < 8; ++j)
+          acc += (double)hqo_f16_to_f32(e[j]) * (double)hqo_f16_to_f32(x[8 * c + j]);
+      }
+    } else {
+      float lane[64];
+      for (int l = 0; l < 64; ++l) lane[l] = 0.f;
+      /* lane l, trip it: int4 index l + 64*it of the row = codes 8*(l+64*it).. */
+      for (int it = 0; it * 512 < ncodes; ++it)
+        for (int l = 0; l < 64; ++l) {
+          int c0 = 8 * (l + 64 * it);
+          if (c0 >= ncodes) continue;
+          for (int i = 0; i < 8; ++i) {
+            const uint16_t* e = cb + (size_t)(uint16_t)row[c0 + i] * 8;
+            const uint16_t* xv = x + 8 * (c0 + i);
+            uint16_t rx = 0, ry = 0;
+            for (int j = 0; j < 4; ++j) { /* main.cu:84-86 */
+              rx = hqo_hfma(e[2 * j], xv[2 * j], rx);
+              ry = hqo_hfma(e[2 * j + 1], xv[2 * j + 1], ry);
+            }
+            lane[l] += hqo_f16_to_f32(rx) + hqo_f16_to_f32(ry); /* main.cu:87 */
+          }
+        }
+      for (int i = 32; i > 0; i /= 2) { /* __shfl_down tree, main.cu:95-97 */
+        float nw[64];
+        for (int l = 0; l < 64; ++l) nw[l] = lane[l] + (l + i < 64 ? lane[l + i] : lane[l]);
+        memcpy(lane, nw, sizeof(nw));
+      }
+      acc = lane[0];
+    }
+    if (y64) y64[m] = scales ? acc * (double)hqo_f16_to_f32(scales[m]) : acc;
+    if (y16) {
+      float r = (float)acc;
+      if (scales) r = r * hqo_f16_to_f32(scales[m]); /* fp32 multiply, one rounding */
+      y16[m] = hqo_f32_to_f16(r);
+    }
+  }
+}

@@ -1,0 +1,126 @@
+/*
+ * hq_oracle.h — CPU restatement of the HeCBench weight-only quantized-inference
+ * kernels (quant3MatMul, lut-gemm, quantAQLM, quantBnB) plus the NF4/FP4
+ * blockwise dequant.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  Only the test-suite, the
+ * smoke check and the benchmark's cpu_baseline leg may call it, and only as the
+ * checker / reported baseline.  The shipped library (libhq.so) never links or
+ * calls anything declared here.
+ *
+ * Every function cites the reference lines (relative to the HeCBench tree) whose
+ * arithmetic it restates.  Functions marked PARITY UNPINNED have no counterpart
+ * or no check in the reference; they are pinned only by closed forms and brute
+ * force in tests/.
+ *
+ *   q3 unpack / fp32 matvec : pinned by the reference known answer -49152.f
+ *                             (src/quant3MatMul-hip/main.cu:36-53,84-105)
+ *   q3 fp16 ("faster")      : pinned by the same known answer
+ *   q3 batched GEMM         : PARITY UNPINNED (no batched kernel in the reference)
+ *   NF4 / FP4 dequant       : PARITY UNPINNED (no NF4/FP4 code in the reference)
+ *   dynamic 8-bit quantize  : pinned by the reference host function compiled
+ *                             into oracle/_ref (src/quantBnB-omp/main.cpp)
+ *   LUT-GEMM                : bit packing + dequant formula pinned by the
+ *                             reference host loops compiled into oracle/_ref
+ *                             (src/lut-gemm-hip/main.cu:118-146)
+ *   AQLM                    : PARITY UNPINNED (the reference checks nothing)
+ */
+#ifndef HQ_ORACLE_H
+#define HQ_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- IEEE binary16 helpers (round-to-nearest-even, subnormals kept) ---- */
+uint16_t hqo_f32_to_f16(float f);
+float    hqo_f16_to_f32(uint16_t h);
+uint16_t hqo_f64_to_f16(double d);
+/* fp16 fused multiply-add a*b+c with a single rounding (device __hfma). */
+uint16_t hqo_hfma(uint16_t a, uint16_t b, uint16_t c);
+uint16_t hqo_hadd(uint16_t a, uint16_t b);
+uint16_t hqo_hmul(uint16_t a, uint16_t b);
+
+/* ---- GPTQ 3-bit (quant3MatMul) ---------------------------------------- */
+/* codes[k*N+n] in 0..7  <->  mat[(3*(k/32)+j)*N + n], j=0..2.
+ * Layout derived from src/quant3MatMul-hip/kernels.h:42-86. */
+void hqo_q3_pack(const uint8_t* codes, int K, int N, int32_t* mat);
+void hqo_q3_unpack(const int32_t* mat, int K, int N, uint8_t* codes);
+
+/* fp32 kernel, src/quant3MatMul-hip/kernels.h:12-90: per 256-row block
+ * res += (scale*float(q) - zero) * x  sequentially in fp32 (no FMA
+ * contraction), block partials added to mul[] in block order.  mul is
+ * accumulated into (the reference caller zeroes it, main.cu:80). */
+void hqo_q3_matvec_f32(const float* x, const int32_t* mat, float* mul,
+                       const float* scales, const float* zeros, int K, int N);
+
+/* Same sum in double precision, written to y (overwrites). */
+void hqo_q3_matvec_f64(const double* x, const int32_t* mat, double* y,
+                       const float* scales, const float* zeros, int K, int N);
+
+/* "faster" kernel, src/quant3MatMul-hip/kernels.h:93-169: scale/zero rounded
+ * to fp16, per 32-value group a fresh half2 accumulator collects 16
+ * hfma2(hfma2(q, scale, -zero), x, acc) terms, widened and added in fp32. */
+void hqo_q3_matvec_f16(const uint16_t* x_f16, const int32_t* mat, float* mul,
+                       const float* scales, const float* zeros, int K, int N);
+
+/* Batched GEMM, PARITY UNPINNED: out[m][n] = sum_k A[m][k]*(s[n]*q[k][n]-z[n]).
+ * mode 0: exact in double; mode 1: weight rounded once to fp16
+ * (w16 = fp16_rn(s*q - z) in fp32), products accumulated in double. */
+void hqo_q3_gemm(const uint16_t* A_f16, const int32_t* mat, double* out,
+                 const float* scales, const float* zeros, int M, int K, int N,
+                 int mode);
+
+/* ---- NF4 / FP4 blockwise dequant (PARITY UNPINNED) --------------------- */
+extern const float hqo_nf4_table[16];
+extern const float hqo_fp4_table[16];
+/* out[2i] = f16(table[byte>>4]*absmax[2i/bs]); out[2i+1] = f16(table[byte&15]*...) */
+void hqo_dequant_4bit(const uint8_t* packed, const float* absmax,
+                      uint16_t* out_f16, int64_t n_elems, int blocksize,
+                      int table /*0=NF4, 1=FP4*/);
+
+/* ---- bitsandbytes dynamic 8-bit quantize (quantBnB) -------------------- */
+/* src/quantBnB-hip/main.cu:13-66 with STOCHASTIC=0. */
+uint8_t hqo_dquantize(const float* code256, float x);
+void    hqo_quantize_dynamic8(const float* code256, const float* A, uint8_t* out,
+                              int64_t n);
+/* The signed dynamic map bitsandbytes builds (256 sorted fp32 values). */
+void    hqo_dynamic_map(float* code256);
+
+/* ---- LUT-GEMM (BCQ) ----------------------------------------------------- */
+/* bit packing of src/lut-gemm-hip/main.cu:118-134:
+ * signs[(k*nb + b)*N + n] in {-1,+1} -> bW[((k/32)*nb + b)*N + n] bit (k%32). */
+void hqo_bcq_pack(const int8_t* signs, int K, int N, int nb, uint32_t* bW);
+/* dense weights, src/lut-gemm-hip/main.cu:136-146 (W[k*N+n], double). */
+void hqo_bcq_dequant(const uint32_t* bW, const uint16_t* alpha_f16,
+                     const uint16_t* qbias_f16 /*nullable*/, int K, int N, int nb,
+                     int group, double* W);
+/* y[n] = sum_k x[k]*W[k][n] in double (x, alpha, bias are fp16 inputs). */
+void hqo_lut_gemv_f64(const uint32_t* bW, const uint16_t* alpha_f16,
+                      const uint16_t* qbias_f16, const uint16_t* x_f16, double* y,
+                      int K, int N, int nb, int group);
+/* Reference evaluation order, src/lut-gemm-hip/mv_fp16.h:133-227: fp16 LUT
+ * built by the doubling chain, fp16 partial sums, fp16 alpha multiply, and the
+ * per-K-tile fp16 results added to the output in tile order (the GPU's atomic
+ * order is arbitrary; tile order is one admissible outcome). */
+void hqo_lut_gemv_f16(const uint32_t* bW, const uint16_t* alpha_f16,
+                      const uint16_t* qbias_f16, const uint16_t* x_f16,
+                      uint16_t* y_f16, int K, int N, int nb, int group);
+
+/* ---- AQLM 1x16 (PARITY UNPINNED) ---------------------------------------- */
+/* src/quantAQLM-hip/main.cu:29-101.  mode 0: double accumulation;
+ * mode 1: the reference's arithmetic (4 chained hfma2 per code, halves widened
+ * and summed in fp32 in lane order, fp32 shuffle-down tree over 64 lanes).
+ * scales_f16 NULL => no scale (reference behaviour); else y = f16(scale*acc). */
+void hqo_aqlm_matvec(const int16_t* codes, const uint16_t* codebooks_f16,
+                     const uint16_t* scales_f16, const uint16_t* x_f16,
+                     uint16_t* y_f16, double* y_f64 /*nullable*/, int M, int K,
+                     const int cb_a_sizes[4], int cb_stride_int4, int mode);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,171 @@
+"""Parity of hq_q3_matvec (batch 1) with the CPU oracle, through the C ABI."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from tests import oracle_api as oa
+from tests.tol import TOL_F16_ACC, TOL_F32_ACC, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(hq, x, mat, scales, zeros, out=None, accumulate=False):
+    import torch
+    dev = torch.device("cuda:0")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    o = None if out is None else t(out)
+    y = hq.q3_matvec(t(x), t(mat), t(scales), t(zeros), out=o, accumulate=accumulate)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def _reference_pattern(K, N):
+    """Weights of the reference's own check: every code is 1 (main.cu:35-43)."""
+    p1 = 0b01001001001001001001001001001001
+    mat = np.zeros((3 * K // 32, N), np.uint32)
+    mat[0::3] = p1
+    mat[1::3] = (p1 << 1) & 0xFFFFFFFF
+    mat[2::3] = (p1 << 2) & 0xFFFFFFFF
+    return mat.view(np.int32)
+
+
+def test_known_answer_minus_49152(hq):
+    """The reference's verification: x=1, scale=-1, zero=0, all codes 1, K=49152 ->
+    every output is exactly -49152 (src/quant3MatMul-hip/main.cu:84-105), fp32 and fp16 input."""
+    K, N = 49152, 12288
+    mat = _reference_pattern(K, N)
+    s = -np.ones(N, np.float32)
+    z = np.zeros(N, np.float32)
+    y = _run(hq, np.ones(K, np.float32), mat, s, z)
+    assert (y == -49152.0).all()
+    y = _run(hq, np.ones(K, np.float16), mat, s, z)
+    assert (y == -49152.0).all()
+    # the reference wrappers accumulate into mul: start from 1000 -> -48152
+    y = _run(hq, np.ones(K, np.float32), mat, s, z, out=np.full(N, 1000, np.float32), accumulate=True)
+    assert (y == -48152.0).all()
+
+
+@pytest.mark.parametrize("K,N,seed", [(4096, 11008, 11), (256, 256, 12), (1024, 64, 13), (32, 4, 14),
+                                      (4096, 1000, 15), (8192, 4096, 16), (6144, 320, 17), (160, 132, 18)])
+def test_matvec_f32_vs_oracle(hq, oracle, K, N, seed):
+    codes, scales, zeros, x = oa.make_q3_problem(seed, K, N)
+    mat = oracle.q3_pack(codes)
+    y = _run(hq, x, mat, scales, zeros)
+    ref64 = oracle.q3_matvec_f64(x, mat, scales, zeros)
+    ref32 = oracle.q3_matvec_f32(x, mat, scales, zeros)
+    assert rel_err(y, ref32) <= TOL_F32_ACC
+    # fp32-accumulate accuracy: as close to the exact sum as the reference's own fp32 order
+    assert rel_err(y, ref64) <= 1e-4
+
+
+@pytest.mark.parametrize("K,N,seed", [(4096, 11008, 21), (512, 256, 22)])
+def test_matvec_f16_vs_oracle(hq, oracle, K, N, seed):
+    codes, scales, zeros, x = oa.make_q3_problem(seed, K, N, x_dtype=np.float16)
+    mat = oracle.q3_pack(codes)
+    y = _run(hq, x, mat, scales, zeros)
+    ref16 = oracle.q3_matvec_f16(x, mat, scales, zeros)          # the reference's fp16 arithmetic
+    ref64 = oracle.q3_matvec_f64(x.astype(np.float64), mat, scales, zeros)
+    assert rel_err(y, ref16) <= TOL_F16_ACC
+    assert rel_err(y, ref64) <= 1e-4   # fp32 accumulation: far tighter than the fp16 contract
+
+
+def test_integer_exact(hq, oracle):
+    """scale=1, zero=0, small integer x: the result is an exact integer matvec."""
+    K, N = 2048, 512
+    rng = np.random.default_rng(5)
+    codes = rng.integers(0, 8, size=(K, N), dtype=np.uint8)
+    x = rng.integers(-8, 9, size=K).astype(np.float32)
+    mat = oracle.q3_pack(codes)
+    y = _run(hq, x, mat, np.ones(N, np.float32), np.zeros(N, np.float32))
+    want = x.astype(np.int64) @ codes.astype(np.int64)
+    assert (y.astype(np.int64) == want).all() and (y == np.round(y)).all()
+
+
+def test_each_code_position(hq, oracle):
+    """One non-zero code at every position of a k-group: catches a wrong field
+    mask, a wrong power-of-two slot scale or a swapped activation slot."""
+    K, N = 64, 64
+    for k in range(K):
+        codes = np.zeros((K, N), np.uint8)
+        codes[k, :] = np.arange(N) % 8
+        x = np.zeros(K, np.float32)
+        x[k] = 1.0 + k / 64.0
+        x[(k + 1) % K] = 100.0  # must not leak in
+        mat = oracle.q3_pack(codes)
+        y = _run(hq, x, mat, np.ones(N, np.float32), np.zeros(N, np.float32))
+        assert np.array_equal(y, (np.arange(N) % 8) * np.float32(1.0 + k / 64.0)), k
+
+
+def test_wide_dynamic_range_and_zero_vector(hq, oracle):
+    K, N = 1024, 256
+    codes, scales, zeros, x = oa.make_q3_problem(31, K, N)
+    mat = oracle.q3_pack(codes)
+    for scale in (1e-30, 1e-6, 1e6, 1e30):
+        xs = (x * np.float32(scale)).astype(np.float32)
+        y = _run(hq, xs, mat, scales, zeros)
+        ref = oracle.q3_matvec_f64(xs, mat, scales, zeros)
+        assert rel_err(y, ref) <= 1e-4, scale
+    y = _run(hq, np.zeros(K, np.float32), mat, scales, zeros)
+    assert (y == 0).all()
+
+
+def test_split_k_env_matches(hq, oracle, monkeypatch):
+    """Launch shapes with and without split-K give the same answer (tolerance)."""
+    K, N = 4096, 1024
+    codes, scales, zeros, x = oa.make_q3_problem(41, K, N)
+    mat = oracle.q3_pack(codes)
+    ref = oracle.q3_matvec_f64(x, mat, scales, zeros)
+    for waves, steps, ks in [(16, 2, 1), (8, 2, 2), (4, 2, 4), (4, 1, 8), (16, 1, 2), (8, 4, 1), (4, 4, 2)]:
+        monkeypatch.setenv("HQ_Q3_WAVES", str(waves))
+        monkeypatch.setenv("HQ_Q3_STEPS", str(steps))
+        monkeypatch.setenv("HQ_Q3_KSPLIT", str(ks))
+        for _ in range(2):  # twice: the arrival counters must reset themselves
+            y = _run(hq, x, mat, scales, zeros)
+            assert rel_err(y, ref) <= 1e-4, (waves, steps, ks)
+
+
+def test_rejects_bad_arguments(hq):
+    import torch
+    dev = torch.device("cuda:0")
+    x = torch.zeros(64, device=dev)
+    w = torch.zeros((6, 8), dtype=torch.int32, device=dev)
+    s = torch.zeros(8, device=dev)
+    with pytest.raises(hq.HqError):
+        hq.q3_matvec(x, torch.zeros((6, 6), dtype=torch.int32, device=dev), s[:6], s[:6])  # N % 4
+    with pytest.raises(ValueError):
+        hq.q3_matvec(x, w[:3], s, s)  # wrong packed height
+    with pytest.raises(ValueError):
+        hq.q3_matvec(x.cpu(), w, s, s)  # no CPU path
+
+
+def test_vs_reference_kernels(hq, oracle):
+    """Where the reference's own HIP kernels were compiled into oracle/_ref, run
+    them on the same device buffers: fp32 kernel and fp16 'faster' kernel."""
+    import torch
+    ref = oa.load_ref_hip()
+    if ref is None:
+        pytest.skip("oracle/_ref/libhecref_hip.so not built")
+    dev = torch.device("cuda:0")
+    K, N = 4096, 11008  # both multiples of 256, as the reference grid requires
+    codes, scales, zeros, x = oa.make_q3_problem(51, K, N)
+    mat = oracle.q3_pack(codes)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    dx, dm, ds, dz = t(x), t(mat), t(scales), t(zeros)
+    dx16 = t(x.astype(np.float16))
+    vp = lambda a: ctypes.c_void_p(a.data_ptr())
+    mul = torch.zeros(N, device=dev)
+    ref.ref_vecquant3matmul_f32(vp(dx), vp(dm), vp(mul), vp(ds), vp(dz), 3 * K // 32, N)
+    torch.cuda.synchronize()
+    y = hq.q3_matvec(dx, dm, ds, dz)
+    torch.cuda.synchronize()
+    assert rel_err(y.cpu().numpy(), mul.cpu().numpy()) <= TOL_F32_ACC
+    mul16 = torch.zeros(N, device=dev)
+    ref.ref_vecquant3matmul_faster(vp(dx16), vp(dm), vp(mul16), vp(ds), vp(dz), 3 * K // 32, N)
+    torch.cuda.synchronize()
+    y16 = hq.q3_matvec(dx16, dm, ds, dz)
+    torch.cuda.synchronize()
+    assert rel_err(y16.cpu().numpy(), mul16.cpu().numpy()) <= TOL_F16_ACC
+    # and the oracle's restatement of the fp16 kernel agrees with the real one
+    o16 = oracle.q3_matvec_f16(x.astype(np.float16), mat, scales, zeros)
+    assert rel_err(o16, mul16.cpu().numpy()) <= 2e-3
