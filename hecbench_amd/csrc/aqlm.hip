@@ -31,11 +31,17 @@ struct AqlmArgs {
   int cb_stride;  // in 16-byte units
 };
 
+__device__ __forceinline__ h2v as_h2(uint32_t v) { return __builtin_bit_cast(h2v, v); }
+
 __device__ __forceinline__ float dot8(u4v e, u4v xv, float acc) {
-  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2v, e.x), __builtin_bit_cast(h2v, xv.x), acc, false);
-  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2v, e.y), __builtin_bit_cast(h2v, xv.y), acc, false);
-  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2v, e.z), __builtin_bit_cast(h2v, xv.z), acc, false);
-  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2v, e.w), __builtin_bit_cast(h2v, xv.w), acc, false);
+  // components are copied to scalars first: bit-casting a vector element in place
+  // makes the compiler read element 0 for every component
+  const uint32_t e0 = e.x, e1 = e.y, e2 = e.z, e3 = e.w;
+  const uint32_t x0 = xv.x, x1 = xv.y, x2 = xv.z, x3 = xv.w;
+  acc = __builtin_amdgcn_fdot2(as_h2(e0), as_h2(x0), acc, false);
+  acc = __builtin_amdgcn_fdot2(as_h2(e1), as_h2(x1), acc, false);
+  acc = __builtin_amdgcn_fdot2(as_h2(e2), as_h2(x2), acc, false);
+  acc = __builtin_amdgcn_fdot2(as_h2(e3), as_h2(x3), acc, false);
   return acc;
 }
 

@@ -3,8 +3,7 @@
 //   out[2i]   = fp16_rn(table[packed[i] >> 4] * absmax[(2i)   / blocksize])
 //   out[2i+1] = fp16_rn(table[packed[i] & 15] * absmax[(2i+1) / blocksize])
 //
-// Pure streaming, write-dominated (4 bytes out per packed nibble pair... 64 B out
-// per 16 B in).  A lane owns 16 packed bytes (one 128-bit load, 32 codes) and
+// Pure streaming, write-dominated (64 bytes out per 16 bytes in).  A lane owns 16 packed bytes (one 128-bit load, 32 codes) and
 // writes 64 contiguous bytes as four 128-bit nontemporal stores.  The 16-entry
 // code book sits in LDS: 16 entries occupy 16 distinct banks, so lanes that hit
 // the same bank always hit the same address (broadcast) and the lookups are
@@ -29,10 +28,19 @@ __constant__ float c_fp4[16] = {
     0.0f, 0.005208333333f, 0.66666667f, 1.0f, 0.33333333f, 0.5f, 0.16666667f, 0.25f,
     -0.0f, -0.005208333333f, -0.66666667f, -1.0f, -0.33333333f, -0.5f, -0.16666667f, -0.25f};
 
+// The contract is two roundings: an fp32 product, then fp32 -> fp16.  The empty asm
+// pins the fp32 product in a register so that the compiler cannot merge multiply and
+// conversion into one mixed-precision instruction, which rounds only once.
+__device__ __forceinline__ float mul_rounded_f32(float a, float b) {
+  float v = a * b;
+  asm volatile("" : "+v"(v));
+  return v;
+}
+
 __device__ __forceinline__ uint32_t deq_pair(const float* tab, uint32_t byte, float a_hi, float a_lo) {
   // high nibble is the earlier element
-  const float v0 = tab[byte >> 4] * a_hi;
-  const float v1 = tab[byte & 15u] * a_lo;
+  const float v0 = mul_rounded_f32(tab[byte >> 4], a_hi);
+  const float v1 = mul_rounded_f32(tab[byte & 15u], a_lo);
   h2v h = {(_Float16)v0, (_Float16)v1};
   return __builtin_bit_cast(uint32_t, h);
 }
@@ -84,7 +92,7 @@ __global__ __launch_bounds__(256) void dequant4_tail_kernel(const uint8_t* __res
   const float* tab = table ? c_fp4 : c_nf4;
   const uint32_t byte = packed[e >> 1];
   const uint32_t code = (e & 1) ? (byte & 15u) : (byte >> 4);
-  out[e] = (_Float16)(tab[code] * absmax[e / blocksize]);
+  out[e] = (_Float16)mul_rounded_f32(tab[code], absmax[e / blocksize]);
 }
 
 }  // namespace

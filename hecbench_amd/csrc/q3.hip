@@ -10,9 +10,10 @@
 // the integer codes are never converted one by one: each 32-bit window of the
 // packed string is ANDed into two subnormal-fp16 fields (see q3_recipe.h) and the
 // multiply-accumulate runs on the matrix cores as a 16x16x32 fp16 MFMA whose
-// "batch" dimension carries the three fp16 pieces (hi/mid/lo, 11 bits each) of
-// the fp32 activation vector.  All products are exact in fp32 and accumulation is
-// fp32, so the result has fp32-accumulate accuracy.
+// "batch" dimension carries three fixed-point digits (11 bits each, 33 bits below
+// the largest |x|) of the fp32 activation vector.  Products and partial sums are
+// integers in units of one quantum, so the accumulation is exact; the only
+// roundings are the handful of fp32 operations of the epilogue.
 //
 // Work split: a workgroup owns a 64-column tile and a contiguous range of
 // k-groups; a wave's 16-lane quarter `kb` streams one k-group as three
@@ -145,12 +146,18 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
                        : reinterpret_cast<const float*>(a.x)[k_begin + k];
     const int gl = k >> 5, ki = k & 31;
     const int slot = c_slots.slot[ki], pos = c_slots.pos[ki];
-    const float v = xv * scaleE * pow2f(-pos);
-    const _Float16 h0 = (_Float16)v;
-    const float r1 = (v - (float)h0) * 2048.f;
-    const _Float16 h1 = (_Float16)r1;
-    const float r2 = (r1 - (float)h1) * 2048.f;
-    const _Float16 h2 = (_Float16)r2;
+    // Fixed-point split of u = x*2^E (|u| < 2^15) into three signed 11-bit digits
+    // with quanta 2^5, 2^-6, 2^-17.  Every MFMA product is then an integer multiple
+    // of one quantum and a wave's partial sums stay below 2^24 quanta, so the matrix
+    // core accumulation is exact whatever its internal rounding is.
+    const float u = xv * scaleE;
+    const float p0 = rintf(u * 0.03125f);
+    const float r1 = u - p0 * 32.f;        // exact
+    const float p1 = rintf(r1 * 64.f);
+    const float r2 = r1 - p1 * 0.015625f;  // exact
+    const float p2 = rintf(r2 * 131072.f);
+    const float sl = pow2f(4 - pos);       // digit * 2^(4-pos) fits fp16 exactly
+    const _Float16 h0 = (_Float16)(p0 * sl), h1 = (_Float16)(p1 * sl), h2 = (_Float16)(p2 * sl);
     _Float16* dst = xs_h + ((size_t)(gl * 4 + (slot >> 3)) * 4) * 8 + (slot & 7);
     dst[0] = h0; dst[8] = h1; dst[16] = h2;
   }
@@ -205,7 +212,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     }
     const float inv11 = 1.f / 2048.f;
     float S = fmaf(fmaf(c2, inv11, c1), inv11, c0);
-    float qx = S * 16777216.f * pow2f(-E);
+    float qx = S * 33554432.f * pow2f(-E);  // 2^20 (operand scale) * 2^5 (digit 0 quantum)
     val = a.scales[n] * qx - a.zeros[n] * xsum;
     if (a.nsplit == 1) {
       a.y[n] = (a.flags & HQ_FLAG_ACCUMULATE) ? a.y[n] + val : val;

@@ -1,0 +1,79 @@
+"""Parity of hq_lut_gemv with the CPU oracle (and, where built, the reference's
+own kernel), through the C ABI."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from tests import oracle_api as oa
+from tests.tol import FLOOR_F16, TOL_F16_ACC, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(hq, bW, alpha, qbias, x, group):
+    import torch
+    dev = torch.device("cuda:0")
+    t = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    y = hq.lut_matmul(t(x), t(bW.view(np.int32)), t(alpha), t(qbias), group)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("K,N,nb,group,zero_bias,seed", [
+    (4096, 16384, 3, 128, True, 1), (4096, 16384, 3, 128, False, 2), (1024, 4096, 8, 128, False, 3),
+    (1024, 4096, 4, 128, False, 4), (512, 130, 3, 64, False, 5), (96, 64, 1, 32, False, 6),
+    (2048, 1001, 2, 2048, False, 7), (1536, 256, 3, 512, False, 8)])
+def test_vs_oracle(hq, oracle, K, N, nb, group, zero_bias, seed):
+    bW, alpha, qbias, x = oa.make_lut_problem(seed, K, N, nb, group, zero_bias)
+    y = _run(hq, bW, alpha, qbias, x, group)
+    ref = oracle.lut_gemv_f64(bW, alpha, qbias, x, group)
+    # fp32 sums rounded once to fp16: half an fp16 ulp of the result, far inside the fp16-accumulate bound
+    assert rel_err(y, ref) <= 2e-3
+    assert rel_err(y, ref) <= TOL_F16_ACC
+
+
+def test_no_bias_pointer(hq, oracle):
+    bW, alpha, _, x = oa.make_lut_problem(9, 1024, 512, 3, 128)
+    y = _run(hq, bW, alpha, None, x, 128)
+    ref = oracle.lut_gemv_f64(bW, alpha, None, x, 128)
+    assert rel_err(y, ref) <= 2e-3
+
+
+def test_closed_forms(hq, oracle):
+    """alpha = 0 -> y = sum_g bias[g] * sum_{k in g} x;  nb=1, alpha=1, bias=0 -> y = sum +-x."""
+    K, N, G = 512, 128, 128
+    rng = np.random.default_rng(3)
+    x = rng.integers(-4, 5, size=K).astype(np.float16)
+    bW = rng.integers(0, 2 ** 32, size=(K // 32, 1, N), dtype=np.uint64).astype(np.uint32)
+    qb = rng.integers(-2, 3, size=(K // G, N)).astype(np.float16)
+    y = _run(hq, bW, np.zeros((K // G, 1, N), np.float16), qb, x, G)
+    want = (qb.astype(np.float64) * x.astype(np.float64).reshape(K // G, G).sum(1)[:, None]).sum(0)
+    assert np.array_equal(y.astype(np.float64), want)
+    y = _run(hq, bW, np.ones((K // G, 1, N), np.float16), np.zeros((K // G, N), np.float16), x, G)
+    bits = ((bW[:, 0, :, None] >> np.arange(32, dtype=np.uint32)) & 1).transpose(0, 2, 1).reshape(K, N)
+    want = ((2.0 * bits - 1.0) * x.astype(np.float64)[:, None]).sum(0)
+    assert np.array_equal(y.astype(np.float64), want)
+
+
+def test_vs_reference_kernel(hq, oracle):
+    import torch
+    ref = oa.load_ref_hip()
+    if ref is None:
+        pytest.skip("oracle/_ref/libhecref_hip.so not built")
+    dev = torch.device("cuda:0")
+    K, N, nb, G = 4096, 16384, 3, 128
+    bW, alpha, qbias, x = oa.make_lut_problem(21, K, N, nb, G, zero_bias=False)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    dW, da, dq, dx = t(bW.view(np.int32)), t(alpha), t(qbias), t(x)
+    out = torch.zeros(N, dtype=torch.float16, device=dev)
+    vp = lambda a: ctypes.c_void_p(a.data_ptr())
+    ref.ref_lut_matmul(vp(out), vp(dx), vp(dW), vp(da), vp(dq), K, N, nb, K // G)
+    torch.cuda.synchronize()
+    y = hq.lut_matmul(dx, dW, da, dq, G)
+    torch.cuda.synchronize()
+    r = out.cpu().numpy()
+    exact = oracle.lut_gemv_f64(bW, alpha, qbias, x, G)
+    # the reference accumulates everything in fp16 (and across 128 K tiles with fp16 atomics)
+    assert rel_err(y.cpu().numpy(), r, FLOOR_F16) <= TOL_F16_ACC
+    assert rel_err(y.cpu().numpy(), exact) <= rel_err(r, exact)

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from tests import oracle_api as oa
-from tests.tol import TOL_F16_ACC, TOL_F32_ACC, rel_err
+from tests.tol import FLOOR_F16, TOL_F16_ACC, TOL_F32_ACC, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -66,7 +66,7 @@ def test_matvec_f16_vs_oracle(hq, oracle, K, N, seed):
     y = _run(hq, x, mat, scales, zeros)
     ref16 = oracle.q3_matvec_f16(x, mat, scales, zeros)          # the reference's fp16 arithmetic
     ref64 = oracle.q3_matvec_f64(x.astype(np.float64), mat, scales, zeros)
-    assert rel_err(y, ref16) <= TOL_F16_ACC
+    assert rel_err(y, ref16, FLOOR_F16) <= TOL_F16_ACC
     assert rel_err(y, ref64) <= 1e-4   # fp32 accumulation: far tighter than the fp16 contract
 
 
@@ -165,7 +165,7 @@ def test_vs_reference_kernels(hq, oracle):
     torch.cuda.synchronize()
     y16 = hq.q3_matvec(dx16, dm, ds, dz)
     torch.cuda.synchronize()
-    assert rel_err(y16.cpu().numpy(), mul16.cpu().numpy()) <= TOL_F16_ACC
+    assert rel_err(y16.cpu().numpy(), mul16.cpu().numpy(), FLOOR_F16) <= TOL_F16_ACC
     # and the oracle's restatement of the fp16 kernel agrees with the real one
     o16 = oracle.q3_matvec_f16(x.astype(np.float16), mat, scales, zeros)
-    assert rel_err(o16, mul16.cpu().numpy()) <= 2e-3
+    assert rel_err(o16, mul16.cpu().numpy(), FLOOR_F16) <= 2e-3
