@@ -3,8 +3,7 @@
 //   out[2i]   = fp16_rn(table[packed[i] >> 4] * absmax[(2i)   / blocksize])
 //   out[2i+1] = fp16_rn(table[packed[i] & 15] * absmax[(2i+1) / blocksize])
 //
-// Pure streaming, write-dominated (64 bytes out per 16 bytes in).  A lane owns 16 packed bytes (one 128-bit load, 32 codes) and
-// writes 64 contiguous bytes as four 128-bit nontemporal stores.  The 16-entry
+// Pure streaming, write-dominated (64 bytes out per 16 bytes in).  The 16-entry
 // code book sits in LDS: 16 entries occupy 16 distinct banks, so lanes that hit
 // the same bank always hit the same address (broadcast) and the lookups are
 // conflict-free.  The multiply is a single fp32 operation followed by one
@@ -45,40 +44,54 @@ __device__ __forceinline__ uint32_t deq_pair(const float* tab, uint32_t byte, fl
   return __builtin_bit_cast(uint32_t, h);
 }
 
-// Fast path: n_elems % 32 == 0 handled in 32-element lane chunks; blocksize a
-// multiple of 32 means one absmax per lane chunk, otherwise (blocksize 2..16 or
-// not dividing 32) absmax is looked up per element.
-template <bool ONE_ABSMAX>
-__global__ __launch_bounds__(256) void dequant4_kernel(const u4v* __restrict__ packed,
+// Main path.  A lane turns one packed 32-bit word (8 codes) into one 128-bit store,
+// so every load instruction of a wave reads 256 contiguous bytes and every store
+// instruction writes 1 KB of contiguous, fully covered cache lines (a lane that
+// writes its own 64 contiguous bytes instead leaves every line partially written per
+// instruction and runs 3-4x slower).  A workgroup covers 256*U consecutive words and
+// issues its U loads before the first store.
+//   MODE 0: blocksize == 1 << shift and blocksize % 8 == 0 (one absmax per word)
+//   MODE 1: blocksize % 8 == 0, not a power of two (one absmax per word, division)
+//   MODE 2: any even blocksize (absmax looked up per element)
+template <int U, int MODE>
+__global__ __launch_bounds__(256) void dequant4_kernel(const uint32_t* __restrict__ packed,
                                                       const float* __restrict__ absmax,
-                                                      u4v* __restrict__ out, int64_t nchunks,
-                                                      int blocksize, int table) {
+                                                      u4v* __restrict__ out, int64_t nwords,
+                                                      int blocksize, int shift, int table) {
   __shared__ float tab[16];
   if (threadIdx.x < 16) tab[threadIdx.x] = table ? c_fp4[threadIdx.x] : c_nf4[threadIdx.x];
-  __syncthreads();
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nchunks; i += stride) {
-    const u4v p = __builtin_nontemporal_load(packed + i);
-    const int64_t e0 = i * 32;
-    float am = 0.f;
-    if (ONE_ABSMAX) am = absmax[e0 / blocksize];
-    const uint32_t words[4] = {p.x, p.y, p.z, p.w};
+  const int64_t base = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  uint32_t w[U];
+  float am[U];
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      uint32_t o[4];
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const uint32_t byte = (words[w] >> (8 * b)) & 255u;
-        if (ONE_ABSMAX) {
-          o[b] = deq_pair(tab, byte, am, am);
-        } else {
-          const int64_t e = e0 + (w * 4 + b) * 2;
-          o[b] = deq_pair(tab, byte, absmax[e / blocksize], absmax[(e + 1) / blocksize]);
-        }
-      }
-      u4v ov = {o[0], o[1], o[2], o[3]};
-      __builtin_nontemporal_store(ov, out + i * 4 + w);
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * 256;
+    w[u] = 0u;
+    am[u] = 0.f;
+    if (i < nwords) {
+      w[u] = __builtin_nontemporal_load(packed + i);
+      if (MODE == 0) am[u] = absmax[(i * 8) >> shift];
+      if (MODE == 1) am[u] = absmax[(i * 8) / blocksize];
     }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t i = base + u * 256;
+    if (i >= nwords) continue;
+    uint32_t o[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const uint32_t byte = (w[u] >> (8 * b)) & 255u;
+      if (MODE == 2) {
+        const int64_t e = i * 8 + 2 * b;
+        o[b] = deq_pair(tab, byte, absmax[e / blocksize], absmax[(e + 1) / blocksize]);
+      } else {
+        o[b] = deq_pair(tab, byte, am[u], am[u]);
+      }
+    }
+    u4v ov = {o[0], o[1], o[2], o[3]};
+    __builtin_nontemporal_store(ov, out + i);
   }
 }
 
@@ -109,22 +122,29 @@ extern "C" int hq_dequant_nf4(const uint8_t* packed, const float* absmax, void* 
   int rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
 
-  const bool wide = !((uintptr_t)packed & 15) && !((uintptr_t)out_fp16 & 15);
-  const int64_t nchunks = wide ? n_elems / 32 : 0;
-  if (nchunks > 0) {
-    int64_t blocks = (nchunks + 255) / 256;
-    const int64_t cap = (int64_t)dev->cus * hq_env_int("HQ_NF4_BLOCKS_PER_CU", 16);
-    if (blocks > cap) blocks = cap;
-    if (blocksize % 32 == 0)
-      hipLaunchKernelGGL(dequant4_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                         (const u4v*)packed, absmax, (u4v*)out_fp16, nchunks, blocksize, table);
+  const bool wide = !((uintptr_t)packed & 3) && !((uintptr_t)out_fp16 & 15);
+  const int64_t nwords = wide ? n_elems / 8 : 0;
+  if (nwords > 0) {
+    constexpr int U = 8;
+    const int64_t blocks = (nwords + 256 * U - 1) / (256 * U);
+    if (blocks > 0x7fffffff) return HQ_ERR_TOO_LARGE;
+    const bool pow2 = (blocksize & (blocksize - 1)) == 0;
+    int shift = 0;
+    while ((1 << shift) < blocksize) ++shift;
+    const uint32_t* pw = reinterpret_cast<const uint32_t*>(packed);
+    if (blocksize % 8 == 0 && pow2)
+      hipLaunchKernelGGL((dequant4_kernel<U, 0>), dim3((unsigned)blocks), dim3(256), 0, stream, pw, absmax,
+                         (u4v*)out_fp16, nwords, blocksize, shift, table);
+    else if (blocksize % 8 == 0)
+      hipLaunchKernelGGL((dequant4_kernel<U, 1>), dim3((unsigned)blocks), dim3(256), 0, stream, pw, absmax,
+                         (u4v*)out_fp16, nwords, blocksize, shift, table);
     else
-      hipLaunchKernelGGL(dequant4_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                         (const u4v*)packed, absmax, (u4v*)out_fp16, nchunks, blocksize, table);
+      hipLaunchKernelGGL((dequant4_kernel<U, 2>), dim3((unsigned)blocks), dim3(256), 0, stream, pw, absmax,
+                         (u4v*)out_fp16, nwords, blocksize, shift, table);
     rc = hq_launch_status();
     if (rc != HQ_OK) return rc;
   }
-  const int64_t e_begin = nchunks * 32;
+  const int64_t e_begin = nwords * 8;
   if (e_begin < n_elems) {
     const int64_t rest = n_elems - e_begin;
     if ((rest + 255) / 256 > 0x7fffffff) return HQ_ERR_TOO_LARGE;

@@ -15,12 +15,15 @@
 // integers in units of one quantum, so the accumulation is exact; the only
 // roundings are the handful of fp32 operations of the epilogue.
 //
-// Work split: a workgroup owns a 64-column tile and a contiguous range of
-// k-groups; a wave's 16-lane quarter `kb` streams one k-group as three
+// Work split: a workgroup owns a 64-column tile and WAVES*4*STEPS consecutive
+// k-groups; a wave's 16-lane quarter `kb` streams one k-group per step as three
 // uint4 loads (4 adjacent columns x 3 packed rows), i.e. 256 contiguous bytes
-// per packed row per quarter.  With one workgroup per tile no cross-workgroup
-// reduction is needed; with split-K the partial sums go to a workspace and the
-// last workgroup to arrive at a tile adds them in a fixed order.
+// per packed row per quarter.  A wave issues all its global loads first, stages
+// its own activations in LDS without a workgroup barrier, and meets the other
+// waves only in the final reduction.  When one workgroup covers all of K no
+// cross-workgroup reduction is needed; otherwise (split-K) the partial sums go to
+// a workspace and the last workgroup to arrive at a tile adds them in a fixed
+// order, so results do not depend on arrival order.
 #include "hq_internal.h"
 #include "q3_recipe.h"
 
@@ -29,8 +32,7 @@ namespace {
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
-
-__constant__ hq_q3::SlotTable c_slots = hq_q3::make_slot_table();
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 
 struct Q3Args {
   const void* x;
@@ -49,15 +51,28 @@ struct Q3Args {
 
 __device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t)(e + 127) << 23); }
 
+// Cross-lane reductions without LDS traffic: four DPP butterfly steps inside each
+// 16-lane row, then the four row results are read into scalars.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_f(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int m = 32; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m));
-  return v;
+  v = fmaxf(v, dpp_f<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, dpp_f<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, dpp_f<0x141>(v));  // row_half_mirror
+  v = fmaxf(v, dpp_f<0x140>(v));  // row_mirror
+  return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
 }
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int m = 32; m > 0; m >>= 1) v += __shfl_xor(v, m);
-  return v;
+  v += dpp_f<0xB1>(v);
+  v += dpp_f<0x4E>(v);
+  v += dpp_f<0x141>(v);
+  v += dpp_f<0x140>(v);
+  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
 }
 
 // Sixteen two-field registers of one column's k-group.
@@ -74,148 +89,172 @@ __device__ __forceinline__ void unpack16(uint32_t w0, uint32_t w1, uint32_t w2, 
   for (int r = 0; r < 16; ++r) a[r] = win[kRecipe[r].window] & mask_of(r);
 }
 
-template <int WAVES, int STEPS>
+template <int WAVES, int STEPS, bool XF16>
 __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
-  constexpr int T = WAVES * 64;
-  constexpr int GROUPS_PER_ROUND = WAVES * 4 * STEPS;
+  // One round per workgroup: the host sizes gpw <= WAVES*4*STEPS.
+  // LDS: xs[WAVES][STEPS*4 groups][4 mfma][4 piece slots] uint4 | red[WAVES][3][64] | desc[WAVES] | xsum[WAVES]
   extern __shared__ uint4 smem[];
-  // layout: xs[gpw_pad][4 mfma][4 pieces] uint4 | red[WAVES][3][64] float | misc
-  const int gpw_pad = (a.gpw + GROUPS_PER_ROUND - 1) / GROUPS_PER_ROUND * GROUPS_PER_ROUND;
   uint4* xs = smem;
-  float* red = reinterpret_cast<float*>(smem + (size_t)gpw_pad * 16);
-  float* misc = red + WAVES * 3 * 64;  // [0..WAVES) max, [WAVES..2*WAVES) sum
+  float* red = reinterpret_cast<float*>(smem + WAVES * STEPS * 64);
+  float* desc = red + WAVES * 3 * 64;
+  float* wsum = desc + WAVES;
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int c = lane & 15, kb = lane >> 4;
-  const int ntiles = (a.N + 63) >> 6;
-  const int tile = blockIdx.x % ntiles, split = blockIdx.x / ntiles;
+  const int tile = blockIdx.x, split = blockIdx.y;
   const int G = a.K >> 5;
   const int g_begin = split * a.gpw;
   const int g_count = min(a.gpw, G - g_begin);
-  const int col = tile * 64 + 4 * c;
-  const bool col_ok = col < a.N;
-  const int rounds = gpw_pad / GROUPS_PER_ROUND;
   const size_t row_stride = (size_t)a.N;
+  const int n = tile * 64 + tid;
 
-  uint32_t wreg[STEPS][3][4];
-  auto issue = [&](int round) {
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const int gl = (round * STEPS + s) * (WAVES * 4) + wv * 4 + kb;
-      if (col_ok && gl < g_count) {
-        const uint32_t* p = a.w + (size_t)(3 * (g_begin + gl)) * row_stride + col;
-#pragma unroll
-        for (int j = 0; j < 3; ++j) {
-          u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(p + j * row_stride));
-          wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < 3; ++j)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) wreg[s][j][q] = 0u;
-      }
-    }
-  };
-  issue(0);  // weights are in flight while the activations are staged
-
-  // ---- stage the activation pieces in operand-slot order -------------------
-  for (int i = tid; i < gpw_pad * 16; i += T) xs[i] = make_uint4(0, 0, 0, 0);
-  const int k_begin = g_begin * 32, k_count = g_count * 32;
-  float amax = 0.f, asum = 0.f;
-  for (int k = tid; k < k_count; k += T) {
-    float v = a.x_f16 ? (float)reinterpret_cast<const _Float16*>(a.x)[k_begin + k]
-                      : reinterpret_cast<const float*>(a.x)[k_begin + k];
-    amax = fmaxf(amax, fabsf(v));
-    asum += v;
+  // ---- issue every global load of this wave up front -------------------------------
+  // No load sits under a branch (addresses are clamped instead), so the compiler can
+  // count them and the wait for the activations does not wait for the weights.
+  float sc_n = 0.f, zr_n = 0.f, y_old = 0.f;
+  if (tid < 64) {
+    const int nc = min(n, a.N - 1);
+    sc_n = a.scales[nc];
+    zr_n = a.zeros[nc];
+    y_old = ((a.flags & HQ_FLAG_ACCUMULATE) && a.nsplit == 1) ? a.y[nc] : 0.f;
   }
-  amax = wave_max(amax);
-  asum = wave_sum(asum);
-  if (lane == 0) { misc[wv] = amax; misc[WAVES + wv] = asum; }
-  __syncthreads();
-  float xmax = 0.f, xsum = 0.f;
+  // activations: lane (c, kb) owns the two codes that unpack16() leaves in register c
+  // of k-group kb (element k_lo in the low half, k_hi in the high half)
+  const uint64_t tw = c < 8 ? (c < 4 ? hq_q3::packed_entries(0) : hq_q3::packed_entries(1))
+                            : (c < 12 ? hq_q3::packed_entries(2) : hq_q3::packed_entries(3));
+  const uint32_t te = (uint32_t)(tw >> (16 * (c & 3))) & 0xffffu;
+  const int k_lo = te & 31, k_hi = (te >> 5) & 31, p_lo = (te >> 10) & 7, p_hi = (te >> 13) & 7;
+  float xr[STEPS][2];
+  int gclamp[STEPS];
 #pragma unroll
-  for (int i = 0; i < WAVES; ++i) { xmax = fmaxf(xmax, misc[i]); xsum += misc[WAVES + i]; }
-  // 2^E * max|x| lies in [2^14, 2^15): the hi piece never overflows fp16.
+  for (int s = 0; s < STEPS; ++s) {
+    const int gl = s * (WAVES * 4) + wv * 4 + kb;
+    gclamp[s] = g_begin + min(gl, g_count - 1);
+    const size_t k = (size_t)gclamp[s] * 32;
+    if (XF16) {
+      const _Float16* xp = reinterpret_cast<const _Float16*>(a.x) + k;
+      xr[s][0] = (float)xp[k_lo]; xr[s][1] = (float)xp[k_hi];
+    } else {
+      const float* xp = reinterpret_cast<const float*>(a.x) + k;
+      xr[s][0] = xp[k_lo]; xr[s][1] = xp[k_hi];
+    }
+  }
+  // weights: out-of-range columns read the last valid quad (their results are never
+  // stored), out-of-range k-groups read a valid group and get zero activations below
+  const int col = min(tile * 64 + 4 * c, a.N - 4);
+  uint32_t wreg[STEPS][3][4];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const uint32_t* p = a.w + (size_t)(3 * gclamp[s]) * row_stride + col;
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(p + j * row_stride));
+      wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    if (s * (WAVES * 4) + wv * 4 + kb >= g_count) { xr[s][0] = 0.f; xr[s][1] = 0.f; }
+  }
+
+  // ---- stage this wave's activation digits in operand-slot order (wave-local) ----------
+  float amax = 0.f, asum = 0.f;
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    amax = fmaxf(amax, fmaxf(fabsf(xr[s][0]), fabsf(xr[s][1])));
+    asum += xr[s][0] + xr[s][1];
+  }
+  const float xmax = wave_max(amax);
+  asum = wave_sum(asum);
+  // 2^E * max|x| lies in [2^14, 2^15): digit 0 never overflows fp16.
   int E = 14 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
   E = xmax > 0.f ? max(-100, min(100, E)) : 0;
   const float scaleE = pow2f(E);
-  _Float16* xs_h = reinterpret_cast<_Float16*>(xs);
-  for (int k = tid; k < k_count; k += T) {
-    float xv = a.x_f16 ? (float)reinterpret_cast<const _Float16*>(a.x)[k_begin + k]
-                       : reinterpret_cast<const float*>(a.x)[k_begin + k];
-    const int gl = k >> 5, ki = k & 31;
-    const int slot = c_slots.slot[ki], pos = c_slots.pos[ki];
-    // Fixed-point split of u = x*2^E (|u| < 2^15) into three signed 11-bit digits
-    // with quanta 2^5, 2^-6, 2^-17.  Every MFMA product is then an integer multiple
-    // of one quantum and a wave's partial sums stay below 2^24 quanta, so the matrix
-    // core accumulation is exact whatever its internal rounding is.
-    const float u = xv * scaleE;
-    const float p0 = rintf(u * 0.03125f);
-    const float r1 = u - p0 * 32.f;        // exact
-    const float p1 = rintf(r1 * 64.f);
-    const float r2 = r1 - p1 * 0.015625f;  // exact
-    const float p2 = rintf(r2 * 131072.f);
-    const float sl = pow2f(4 - pos);       // digit * 2^(4-pos) fits fp16 exactly
-    const _Float16 h0 = (_Float16)(p0 * sl), h1 = (_Float16)(p1 * sl), h2 = (_Float16)(p2 * sl);
-    _Float16* dst = xs_h + ((size_t)(gl * 4 + (slot >> 3)) * 4) * 8 + (slot & 7);
-    dst[0] = h0; dst[8] = h1; dst[16] = h2;
+  uint4* xs_w = xs + wv * (STEPS * 64);
+  const float sl_lo = pow2f(4 - p_lo), sl_hi = pow2f(4 - p_hi);  // digit * 2^(4-pos) fits fp16 exactly
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    // Fixed-point split of u = x*2^E (|u| < 2^15) into three signed 11-bit digits with
+    // quanta 2^5, 2^-6, 2^-17.  Every MFMA product is then an integer multiple of one
+    // quantum and a wave's partial sums stay below 2^24 quanta, so the matrix-core
+    // accumulation is exact whatever its internal rounding is.
+    float d[2][3];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const float u = xr[s][e] * scaleE;
+      d[e][0] = rintf(u * 0.03125f);
+      const float r1 = u - d[e][0] * 32.f;        // exact
+      d[e][1] = rintf(r1 * 64.f);
+      const float r2 = r1 - d[e][1] * 0.015625f;  // exact
+      d[e][2] = rintf(r2 * 131072.f);
+    }
+    // register c of MFMA j = c/4 of this k-group: dword c%4 of the 16-byte operand chunk
+    uint32_t* dst = reinterpret_cast<uint32_t*>(xs_w + ((s * 4 + kb) * 4 + (c >> 2)) * 4) + (c & 3);
+#pragma unroll
+    for (int p = 0; p < 3; ++p) {
+      const h2v pair = {(_Float16)(d[0][p] * sl_lo), (_Float16)(d[1][p] * sl_hi)};
+      dst[4 * p] = __builtin_bit_cast(uint32_t, pair);
+    }
   }
-  __syncthreads();
+  // The digits are read back by other lanes of this wave only: order the LDS writes
+  // before the reads without a workgroup barrier.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 
-  // ---- main loop ---------------------------------------------------------------
+  // ---- unpack + MFMA -----------------------------------------------------------------------
   f4 acc[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
-  const int piece = c < 3 ? c : 3;
-  for (int round = 0; round < rounds; ++round) {
-    if (round > 0) issue(round);
+  const int piece = c < 3 ? c : 2;  // columns 3..15 of the MFMA are never read
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const int gl_base = (round * STEPS + s) * (WAVES * 4) + wv * 4;
-      if (gl_base >= g_count) continue;  // wave-uniform
-      const uint4* xb = xs + (size_t)(gl_base + kb) * 16 + piece;
-      h8 B[4];
+  for (int s = 0; s < STEPS; ++s) {
+    if (s * (WAVES * 4) + wv * 4 >= g_count) continue;  // wave-uniform
+    const uint4* xb = xs_w + (size_t)(s * 4 + kb) * 16 + piece;
+    h8 B[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) B[j] = __builtin_bit_cast(h8, xb[j * 4]);
+    for (int j = 0; j < 4; ++j) B[j] = __builtin_bit_cast(h8, xb[j * 4]);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        uint32_t f[16];
-        unpack16(wreg[s][0][q], wreg[s][1][q], wreg[s][2][q], f);
+    for (int q = 0; q < 4; ++q) {
+      uint32_t f[16];
+      unpack16(wreg[s][0][q], wreg[s][1][q], wreg[s][2][q], f);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          u4v av = {f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]};
-          acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), B[j], acc[q], 0, 0, 0);
-        }
+      for (int j = 0; j < 4; ++j) {
+        u4v av = {f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]};
+        acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), B[j], acc[q], 0, 0, 0);
       }
     }
   }
 
-  // ---- combine waves, pieces, scale/zero ------------------------------------------
-  // D[row = 4*kb + i][col = c]: row is the weight column (quarter-major), col the piece.
+  // ---- combine waves, digits, scale/zero --------------------------------------------------
+  // D[row = 4*kb + i][col = c]: row is the weight column (quarter-major), col the digit.
   if (c < 3) {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
       for (int i = 0; i < 4; ++i) red[(wv * 3 + c) * 64 + 4 * (4 * kb + i) + q] = acc[q][i];
   }
+  if (lane == 0) {
+    desc[wv] = pow2f(-E);
+    wsum[wv] = asum;
+  }
   __syncthreads();
-  const int n = tile * 64 + tid;
   float val = 0.f;
   if (tid < 64 && n < a.N) {
-    float c0 = 0.f, c1 = 0.f, c2 = 0.f;
+    const float inv11 = 1.f / 2048.f;
+    float qx = 0.f, xsum = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      c0 += red[(w * 3 + 0) * 64 + tid];
-      c1 += red[(w * 3 + 1) * 64 + tid];
-      c2 += red[(w * 3 + 2) * 64 + tid];
+      const float c0 = red[(w * 3 + 0) * 64 + tid];
+      const float c1 = red[(w * 3 + 1) * 64 + tid];
+      const float c2 = red[(w * 3 + 2) * 64 + tid];
+      // 2^20 (operand scale) * 2^5 (digit-0 quantum) / 2^E
+      qx += fmaf(fmaf(c2, inv11, c1), inv11, c0) * 33554432.f * desc[w];
+      xsum += wsum[w];
     }
-    const float inv11 = 1.f / 2048.f;
-    float S = fmaf(fmaf(c2, inv11, c1), inv11, c0);
-    float qx = S * 33554432.f * pow2f(-E);  // 2^20 (operand scale) * 2^5 (digit 0 quantum)
-    val = a.scales[n] * qx - a.zeros[n] * xsum;
+    val = sc_n * qx - zr_n * xsum;
     if (a.nsplit == 1) {
-      a.y[n] = (a.flags & HQ_FLAG_ACCUMULATE) ? a.y[n] + val : val;
+      a.y[n] = y_old + val;
     } else {
       a.partial[((size_t)tile * a.nsplit + split) * 64 + tid] = val;
     }
@@ -243,18 +282,21 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   }
 }
 
-template <int WAVES, int STEPS>
-int launch_matvec(const Q3Args& a, int ntiles, hipStream_t stream) {
-  constexpr int GPR = WAVES * 4 * STEPS;
-  const int gpw_pad = (a.gpw + GPR - 1) / GPR * GPR;
-  const size_t smem = (size_t)gpw_pad * 256 + (size_t)WAVES * 3 * 64 * 4 + (size_t)WAVES * 2 * 4;
+template <int WAVES, int STEPS, bool XF16>
+int launch_matvec_t(const Q3Args& a, int ntiles, hipStream_t stream) {
+  const size_t smem = (size_t)WAVES * STEPS * 1024 + (size_t)WAVES * 3 * 64 * 4 + (size_t)WAVES * 2 * 4;
   static const hipError_t attr =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_matvec_kernel<WAVES, STEPS>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_matvec_kernel<WAVES, STEPS, XF16>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
   if (attr != hipSuccess) return (int)attr;
-  hipLaunchKernelGGL((q3_matvec_kernel<WAVES, STEPS>), dim3(ntiles * a.nsplit), dim3(WAVES * 64), smem,
+  hipLaunchKernelGGL((q3_matvec_kernel<WAVES, STEPS, XF16>), dim3(ntiles, a.nsplit), dim3(WAVES * 64), smem,
                      stream, a);
   return hq_launch_status();
+}
+template <int WAVES, int STEPS>
+int launch_matvec(const Q3Args& a, int ntiles, hipStream_t stream) {
+  return a.x_f16 ? launch_matvec_t<WAVES, STEPS, true>(a, ntiles, stream)
+                 : launch_matvec_t<WAVES, STEPS, false>(a, ntiles, stream);
 }
 
 }  // namespace
@@ -270,7 +312,7 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   if (x_dtype != HQ_DTYPE_F32 && x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
   if (flags & ~HQ_FLAG_ACCUMULATE) return HQ_ERR_BAD_ENUM;
   if (K <= 0 || N <= 0 || batch_M <= 0 || (K & 31) || (N & 3)) return HQ_ERR_BAD_SHAPE;
-  if (((uintptr_t)qweight & 15) || ((uintptr_t)x & (x_dtype == HQ_DTYPE_F16 ? 1 : 3)) ||
+  if (((uintptr_t)qweight & 15) || ((uintptr_t)x & (x_dtype == HQ_DTYPE_F16 ? 3 : 7)) ||
       ((uintptr_t)y & 3) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
     return HQ_ERR_MISALIGNED;
   const HqDevice* dev = nullptr;
@@ -284,22 +326,16 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   const int G = K / 32;
   const int ntiles = (N + 63) / 64;
   // Launch shape: WAVES waves per workgroup, each streaming STEPS k-groups per
-  // 16-lane quarter per round; split K so that a workgroup runs one round and the
-  // grid covers the CU count a few times over.
+  // 16-lane quarter; K is split over ceil(G / (WAVES*4*STEPS)) workgroups per tile.
   int waves = hq_env_int("HQ_Q3_WAVES", 16);
   int steps = hq_env_int("HQ_Q3_STEPS", 2);
-  int nsplit = hq_env_int("HQ_Q3_KSPLIT", 0);
+  int nsplit = 0;
   if (waves != 4 && waves != 8 && waves != 16) waves = 16;
   if (steps != 1 && steps != 2 && steps != 4) steps = 2;
-  const int gpr = waves * 4 * steps;
-  if (nsplit <= 0) nsplit = (G + gpr - 1) / gpr;
-  if (nsplit > G) nsplit = G;
-  int gpw = (G + nsplit - 1) / nsplit;
-  if (gpw > 192) {  // activation pieces of a workgroup must fit its LDS budget
-    nsplit = (G + 191) / 192;
-    gpw = (G + nsplit - 1) / nsplit;
-  }
-  nsplit = (G + gpw - 1) / gpw;
+  const int gpr = waves * 4 * steps;  // k-groups one workgroup covers
+  (void)nsplit;
+  nsplit = (G + gpr - 1) / gpr;
+  const int gpw = gpr;
 
   Q3Args a;
   a.x = x; a.w = reinterpret_cast<const uint32_t*>(qweight); a.scales = scales; a.zeros = zeros;

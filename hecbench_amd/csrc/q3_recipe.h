@@ -79,6 +79,19 @@ constexpr bool recipe_is_consistent() {
 }
 static_assert(recipe_is_consistent(), "every code must be covered once, inside the fp16 mantissa");
 
+// Per-register facts packed for in-register lookup: entry r (16 bits) holds
+// k_lo | k_hi << 5 | p_lo << 10 | p_hi << 13; four entries per 64-bit word.
+constexpr uint64_t packed_entries(int word) {
+  uint64_t v = 0;
+  for (int i = 0; i < 4; ++i) {
+    const Field2& f = kRecipe[4 * word + i];
+    const uint64_t e = (uint64_t)f.k_lo | ((uint64_t)f.k_hi << 5) | ((uint64_t)f.p_lo << 10) |
+                       ((uint64_t)f.p_hi << 13);
+    v |= e << (16 * i);
+  }
+  return v;
+}
+
 struct SlotTable {
   uint8_t slot[32];
   uint8_t pos[32];
