@@ -256,20 +256,28 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     if (a.nsplit == 1) {
       a.y[n] = y_old + val;
     } else {
-      a.partial[((size_t)tile * a.nsplit + split) * 64 + tid] = val;
+      // Device-coherent (write-through) store: visible to the other XCDs' workgroups
+      // without flushing or invalidating this XCD's L2.
+      __hip_atomic_store(&a.partial[((size_t)tile * a.nsplit + split) * 64 + tid], val, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
     }
   }
   if (a.nsplit > 1) {
+    // Arrival counting with relaxed device-scope atomics only.  The barrier waits for
+    // this workgroup's partial-sum stores to be acknowledged (they are write-through,
+    // so acknowledged means visible device-wide) before the counter is bumped; the last
+    // workgroup to arrive reads every partial with device-coherent loads and adds them
+    // in split order, so the result does not depend on the arrival order.  Full
+    // release/acquire fences are avoided on purpose: on this multi-XCD part they write
+    // back and invalidate the whole L2 and cost tens of microseconds per call.
     __shared__ unsigned s_last;
-    __threadfence();
     __syncthreads();
     if (tid == 0) {
-      unsigned old = atomicAdd(&a.counters[tile], 1u);
+      const unsigned old = __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       s_last = (old == (unsigned)(a.nsplit - 1));
     }
     __syncthreads();
     if (s_last) {
-      __threadfence();
       if (tid < 64 && n < a.N) {
         float sum = 0.f;
         for (int s = 0; s < a.nsplit; ++s)
@@ -277,7 +285,8 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         a.y[n] = (a.flags & HQ_FLAG_ACCUMULATE) ? a.y[n] + sum : sum;
       }
-      if (tid == 0) a.counters[tile] = 0u;  // ready for the next call
+      if (tid == 0)  // ready for the next call
+        __hip_atomic_store(&a.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
