@@ -151,6 +151,23 @@ def bench_others(steps, warmup):
     out["aqlm_4096x4096"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
                              "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS,
                              "gather_GBps": (Ma * Ka // 8 * 16) * steps / secs / 1e9}
+    # config 4: batched GPTQ 3-bit GEMM M=64 K=8192 N=28672 (rotate 7 x 88 MB)
+    Mg, Kg, Ng = 64, 8192, 28672
+    nb = 7
+    mats = [torch.randint(-2 ** 31, 2 ** 31 - 1, (3 * Kg // 32, Ng), dtype=torch.int32, device=dev, generator=g)
+            for _ in range(nb)]
+    sg = torch.empty(Ng, device=dev).uniform_(0.005, 0.02, generator=g)
+    zg = sg * torch.randint(3, 5, (Ng,), device=dev, generator=g).float()
+    Ag = torch.randn(Mg, Kg, device=dev, generator=g).half()
+    og = torch.empty(Mg, Ng, device=dev)
+    st = max(50, steps // 4)
+    secs = _time_loop(lambda i: hq.q3_gemm(Ag, mats[i], sg, zg, out=og), nb, st, 10)
+    b = 3 * Kg // 32 * Ng * 4 + 2 * Ng * 4 + Mg * Kg * 2 + Mg * Ng * 4
+    fl = 2.0 * Mg * Kg * Ng
+    out["q3_gemm_64x8192x28672"] = {"us": secs / st * 1e6, "GBps": b * st / secs / 1e9,
+                                    "frac_hbm": b * st / secs / 1e9 / HBM_PEAK_GBS,
+                                    "TFLOPs": fl * st / secs / 1e12,
+                                    "frac_mfma_f16": fl * st / secs / 1e12 / MFMA_F16_PEAK_TFLOPS}
     return out
 
 

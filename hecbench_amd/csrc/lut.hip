@@ -153,16 +153,23 @@ __global__ __launch_bounds__(256) void lut_gemv_kernel(LutArgs a) {
   if (tid < 64 * CPL && n < a.N) {
     float v = (red[tid] + red[64 * CPL + tid]) + (red[2 * 64 * CPL + tid] + red[3 * 64 * CPL + tid]);
     if (a.nsplit == 1) a.y[n] = (_Float16)v;
-    else a.partial[((size_t)tile * a.nsplit + split) * (64 * CPL) + tid] = v;
+    else  // device-coherent (write-through) store, see the arrival protocol below
+      __hip_atomic_store(&a.partial[((size_t)tile * a.nsplit + split) * (64 * CPL) + tid], v, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
   }
   if (a.nsplit > 1) {
+    // Split-K arrival counting with relaxed device-scope atomics only: the barrier
+    // waits for this workgroup's write-through partial stores to be acknowledged
+    // before the counter is bumped; the last workgroup to arrive adds the partials in
+    // split order.  Full release/acquire fences would write back and invalidate the
+    // whole L2 of the XCD on every workgroup and cost tens of microseconds per call.
     unsigned* s_last = reinterpret_cast<unsigned*>(lds + kTables * 256);
-    __threadfence();
     __syncthreads();
-    if (tid == 0) *s_last = (atomicAdd(&a.counters[tile], 1u) == (unsigned)(a.nsplit - 1));
+    if (tid == 0)
+      *s_last = (__hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                 (unsigned)(a.nsplit - 1));
     __syncthreads();
     if (*s_last) {
-      __threadfence();
       if (tid < 64 * CPL && n < a.N) {
         float sum = 0.f;
         for (int s = 0; s < a.nsplit; ++s)
@@ -170,7 +177,7 @@ __global__ __launch_bounds__(256) void lut_gemv_kernel(LutArgs a) {
                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         a.y[n] = (_Float16)sum;
       }
-      if (tid == 0) a.counters[tile] = 0u;
+      if (tid == 0) __hip_atomic_store(&a.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
