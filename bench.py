@@ -24,6 +24,9 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 K, N = 4096, 11008
 ROWS = 3 * K // 32
 ALGO_BYTES = ROWS * N * 4 + 2 * N * 4 + K * 4 + N * 4   # weights + scale/zero + x + y = 17,056,768
+# HBM bytes per launch of the matvec kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what
+# the same counter reads for a plain 256 MiB device copy (profiles/q3_matvec_4096x11008.txt).
+Q3_TRAFFIC_BYTES = 17257991
 
 
 def _time_loop(fn, n_buffers, steps, warmup):
@@ -178,6 +181,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all", action="store_true", help="also time the other configurations")
+    ap.add_argument("--no-hot", action="store_true", help="skip the hot-cache (single buffer) timing")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run 20 plain device copies of 256 MiB (reference point for rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this path has no collective and every box here has one GPU; "
@@ -191,10 +198,18 @@ def main():
     hq.init()
     info = hq.device_info()
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_()
+        dst = torch.empty_like(src)
+        for _ in range(20):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     secs, state = bench_q3(args.steps, args.warmup)
     us = secs / args.steps * 1e6
     gbs = ALGO_BYTES / (secs / args.steps) / 1e9
-    hot_secs, _ = bench_q3(args.steps, args.warmup, hot=True)
+    hot_secs = None if args.no_hot else bench_q3(args.steps, args.warmup, hot=True)[0]
     result = {
         "metric": "achieved HBM GB/s: GPTQ-3bit matvec 4096x11008 (algorithmic bytes / time per call)",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -204,9 +219,9 @@ def main():
                                "distinct 16.9 MB buffers (575 MB)", "algorithmic_bytes_per_call": ALGO_BYTES},
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
         "effective_fp16_weight_GBps": round(K * N * 2 / (secs / args.steps) / 1e9, 1),
-        "hot_cache_us_per_call": round(hot_secs / args.steps * 1e6, 3),
+        "hot_cache_us_per_call": None if hot_secs is None else round(hot_secs / args.steps * 1e6, 3),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": Q3_TRAFFIC_BYTES},
         "device": info,
     }
     if not args.no_cpu:
