@@ -182,6 +182,201 @@ __global__ __launch_bounds__(256) void lut_gemv_kernel(LutArgs a) {
   }
 }
 
+
+// ======================================================================================
+// Matrix-core path (group size a multiple of 128, N a multiple of 64).
+//
+// sum_k s*x = 2*sum_k bit*x - sum_k x.  A single bit left in place at bit p (p <= 9) of
+// an otherwise zero 16-bit half is the subnormal fp16 number 2^(p-24), so sixteen ANDs
+// (and one shift) turn a packed 32-bit word into the sixteen operand registers of four
+// 16x16x32 fp16 MFMAs; the factor 2^p is folded into the activation of that slot.  No
+// table, no LDS lookup, no bank conflicts.  Lane quarter kb streams k-word 4*quad + kb,
+// so one MFMA chain sums a whole 128-element quad of one bit plane for 64 columns (four
+// adjacent columns per lane, one 128-bit load per plane and quad); alpha is applied to the
+// chain's result in fp32.  Every B column holds the same activations, so the result is
+// replicated across the 16 lanes of a row group and each lane applies alpha to its own
+// four columns.
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+
+// register r of a word: (bit in the low half, bit in the high half); both sit at
+// position p = r (r < 10) of their half, or r - 10 after a shift by 10 (r >= 10)
+__device__ __forceinline__ void unpack_bits(uint32_t w, uint32_t (&a)[16]) {
+  const uint32_t w10 = w >> 10;
+#pragma unroll
+  for (int r = 0; r < 10; ++r) a[r] = w & (0x00010001u << r);
+#pragma unroll
+  for (int r = 10; r < 16; ++r) a[r] = w10 & (0x00010001u << (r - 10));
+}
+
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_f(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+// Sum over the 64 lanes: four DPP butterfly steps per 16-lane row, then the row sums.
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f<0x141>(v);  // row_half_mirror
+  v += dpp_f<0x140>(v);  // row_mirror
+  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
+}
+
+struct Half16 {  // sixteen fp16 values as two 128-bit loads
+  u4v lo, hi;
+  __device__ __forceinline__ float get(int i) const {
+    const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    const uint32_t d = w[i >> 1];
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)((i & 1) ? (d >> 16) : (d & 0xffffu)));
+  }
+};
+__device__ __forceinline__ Half16 load_half16(const _Float16* p) {
+  Half16 h;
+  h.lo = reinterpret_cast<const u4v*>(p)[0];
+  h.hi = reinterpret_cast<const u4v*>(p)[1];
+  return h;
+}
+
+// NB bit planes, QUADS 128-element quads per wave per round.
+template <int NB, int QUADS, int WAVES, bool BIAS>
+__global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
+  constexpr int kMfmaWaves = WAVES;
+  extern __shared__ float lds[];
+  u4v* xs = reinterpret_cast<u4v*>(lds);                 // [waves][QUADS][4 kb][4 j]
+  float* red = lds + kMfmaWaves * QUADS * 16 * 4;        // [waves][64]
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int c = lane & 15, kb = lane >> 4;
+  const int tile = blockIdx.x;
+  const int nquads = a.K >> 7;
+  const size_t n0 = (size_t)tile * 64;
+  const uint32_t col_off = 4u * c;   // first of the lane's 4 columns (N % 64 == 0: no partial tiles)
+  const uint32_t acol = 16u * kb;    // first of the 16 columns this lane applies alpha to
+  // register c of a word holds bit c (low half) and bit c + 16 (high half), both at
+  // position p of their half
+  const int p = c < 10 ? c : c - 10;
+  const float slot_scale = __uint_as_float((uint32_t)(127 - p) << 23);  // 2^-p
+  u4v* xs_w = xs + wv * (QUADS * 16);
+
+  float run[4][4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) run[q][i] = 0.f;
+
+  for (int q0 = wv * QUADS; q0 < nquads; q0 += kMfmaWaves * QUADS) {
+    // ---- loads of this round (unconditional, clamped): activations, then packed words -------
+    float xlo[QUADS], xhi[QUADS];
+    u4v wq[QUADS][NB];
+#pragma unroll
+    for (int t = 0; t < QUADS; ++t) {
+      const int quad = min(q0 + t, nquads - 1);
+      const _Float16* xp = a.x + (size_t)quad * 128 + 32 * kb;
+      xlo[t] = (float)xp[c];
+      xhi[t] = (float)xp[c + 16];
+    }
+#pragma unroll
+    for (int t = 0; t < QUADS; ++t) {
+      const int quad = min(q0 + t, nquads - 1);
+      const uint32_t* wp = a.bW + ((size_t)(4 * quad + kb) * NB) * a.N + n0 + col_off;
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+        wq[t][b] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wp + (size_t)b * a.N));
+    }
+    // ---- stage the activations in operand-slot order (wave-local) ---------------------------
+    float xsum[QUADS];
+#pragma unroll
+    for (int t = 0; t < QUADS; ++t) {
+      if (q0 + t >= nquads) { xlo[t] = 0.f; xhi[t] = 0.f; }
+      const h2v pair = {(_Float16)(xlo[t] * slot_scale), (_Float16)(xhi[t] * slot_scale)};
+      reinterpret_cast<uint32_t*>(xs_w + (t * 4 + kb) * 4 + (c >> 2))[c & 3] = __builtin_bit_cast(uint32_t, pair);
+      xsum[t] = wave_sum(xlo[t] + xhi[t]);  // sum of the quad's 128 activations
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    // ---- MFMA chains --------------------------------------------------------------------------
+#pragma unroll
+    for (int t = 0; t < QUADS; ++t) {
+      if (q0 + t >= nquads) break;  // wave-uniform
+      const int quad = q0 + t;
+      const int g = (quad * 128) / a.G;
+      Half16 al[NB];
+#pragma unroll
+      for (int b = 0; b < NB; ++b) al[b] = load_half16(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
+      h8 B[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) B[j] = __builtin_bit_cast(h8, xs_w[(t * 4 + kb) * 4 + j]);
+      const float half_x = xsum[t] * -2.98023223876953125e-8f;  // -(sum x)/2 in operand units (2^-24)
+      if (BIAS) {
+        const Half16 bi = load_half16(a.qbias + (size_t)g * a.N + n0 + acol);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) run[q][i] = fmaf(bi.get(4 * i + q), -half_x, run[q][i]);
+      }
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const uint32_t words[4] = {wq[t][b].x, wq[t][b].y, wq[t][b].z, wq[t][b].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          uint32_t f[16];
+          unpack_bits(words[q], f);
+          f4 acc = {half_x, half_x, half_x, half_x};  // chain result = sum bit*x - (sum x)/2
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const u4v av = {f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]};
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), B[j], acc, 0, 0, 0);
+          }
+          // rows 4*kb + i of the tile's 16-column block q: column 16*kb + 4*i + q
+#pragma unroll
+          for (int i = 0; i < 4; ++i) run[q][i] = fmaf(al[b].get(4 * i + q), acc[i], run[q][i]);
+        }
+      }
+    }
+  }
+  // ---- combine the waves -------------------------------------------------------------------------
+  if (c == 0) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[wv * 64 + 16 * kb + 4 * i + q] = run[q][i];
+  }
+  __syncthreads();
+  const int n = tile * 64 + tid;
+  if (tid < 64 && n < a.N) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < kMfmaWaves; ++w) v += red[w * 64 + tid];
+    // operand scale 2^-24, and the chains hold half of sum s*x
+    a.y[n] = (_Float16)(v * 33554432.f);
+  }
+}
+
+template <int NB, int QUADS, int WAVES>
+int launch_bcq_mfma_w(const LutArgs& a, hipStream_t stream) {
+  const size_t smem = (size_t)WAVES * QUADS * 16 * 16 + (size_t)WAVES * 64 * 4;
+  const int ntiles = a.N / 64;
+  if (a.qbias)
+    hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, true>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
+  else
+    hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, false>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
+  return hq_launch_status();
+}
+// Waves per workgroup: 16 when K offers at least 16*QUADS quads (four waves per SIMD hide
+// the matrix-core latency of the dependent chains), otherwise 8.
+template <int NB, int QUADS>
+int launch_bcq_mfma(const LutArgs& a, hipStream_t stream) {
+  const int want = hq_env_int("HQ_LUT_WAVES", 0);
+  if (want == 8 || (want != 16 && (a.K >> 7) < 16 * QUADS)) return launch_bcq_mfma_w<NB, QUADS, 8>(a, stream);
+  return launch_bcq_mfma_w<NB, QUADS, 16>(a, stream);
+}
+
 }  // namespace
 
 extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_bias, const void* x,
@@ -197,6 +392,23 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
   int rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
 
+  if (group_size % 128 == 0 && N % 64 == 0 && !((uintptr_t)bW & 15) && !((uintptr_t)alpha & 15) &&
+      !((uintptr_t)q_bias & 15) && hq_env_int("HQ_LUT_PATH", 1) == 1) {
+    LutArgs a;
+    a.bW = bW; a.alpha = (const _Float16*)alpha; a.qbias = (const _Float16*)q_bias;
+    a.x = (const _Float16*)x; a.y = (_Float16*)y; a.partial = nullptr; a.counters = nullptr;
+    a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = K; a.nsplit = 1;
+    switch (nbits) {
+      case 1: return launch_bcq_mfma<1, 2>(a, stream);
+      case 2: return launch_bcq_mfma<2, 2>(a, stream);
+      case 3: return launch_bcq_mfma<3, 2>(a, stream);
+      case 4: return launch_bcq_mfma<4, 2>(a, stream);
+      case 5: return launch_bcq_mfma<5, 1>(a, stream);
+      case 6: return launch_bcq_mfma<6, 1>(a, stream);
+      case 7: return launch_bcq_mfma<7, 1>(a, stream);
+      default: return launch_bcq_mfma<8, 1>(a, stream);
+    }
+  }
   const bool pair = (N % 2 == 0) && !((uintptr_t)bW & 7);
   const int cpl = pair ? 2 : 1;
   const int ntiles = (N + 64 * cpl - 1) / (64 * cpl);

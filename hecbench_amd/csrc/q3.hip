@@ -124,31 +124,34 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
                             : (c < 12 ? hq_q3::packed_entries(2) : hq_q3::packed_entries(3));
   const uint32_t te = (uint32_t)(tw >> (16 * (c & 3))) & 0xffffu;
   const int k_lo = te & 31, k_hi = (te >> 5) & 31, p_lo = (te >> 10) & 7, p_hi = (te >> 13) & 7;
+  // Scalar base pointers of this workgroup's slice plus 32-bit per-lane byte offsets.
+  const char* xbase = reinterpret_cast<const char*>(a.x) + (size_t)g_begin * 32 * (XF16 ? 2 : 4);
   float xr[STEPS][2];
-  int gclamp[STEPS];
+  uint32_t glc[STEPS];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
-    const int gl = s * (WAVES * 4) + wv * 4 + kb;
-    gclamp[s] = g_begin + min(gl, g_count - 1);
-    const size_t k = (size_t)gclamp[s] * 32;
+    glc[s] = (uint32_t)min(s * (WAVES * 4) + wv * 4 + kb, g_count - 1);
     if (XF16) {
-      const _Float16* xp = reinterpret_cast<const _Float16*>(a.x) + k;
-      xr[s][0] = (float)xp[k_lo]; xr[s][1] = (float)xp[k_hi];
+      xr[s][0] = (float)*reinterpret_cast<const _Float16*>(xbase + (glc[s] * 32u + (uint32_t)k_lo) * 2u);
+      xr[s][1] = (float)*reinterpret_cast<const _Float16*>(xbase + (glc[s] * 32u + (uint32_t)k_hi) * 2u);
     } else {
-      const float* xp = reinterpret_cast<const float*>(a.x) + k;
-      xr[s][0] = xp[k_lo]; xr[s][1] = xp[k_hi];
+      xr[s][0] = *reinterpret_cast<const float*>(xbase + (glc[s] * 32u + (uint32_t)k_lo) * 4u);
+      xr[s][1] = *reinterpret_cast<const float*>(xbase + (glc[s] * 32u + (uint32_t)k_hi) * 4u);
     }
   }
   // weights: out-of-range columns read the last valid quad (their results are never
   // stored), out-of-range k-groups read a valid group and get zero activations below
-  const int col = min(tile * 64 + 4 * c, a.N - 4);
+  const int tile_cols = min(64, a.N - tile * 64);           // multiple of 4
+  const uint32_t col_off = (uint32_t)min(4 * c, tile_cols - 4) * 4u;
+  const uint32_t row_bytes = (uint32_t)a.N * 4u;
+  const char* wbase = reinterpret_cast<const char*>(a.w) + ((size_t)(3 * g_begin) * row_stride + (size_t)tile * 64) * 4;
   uint32_t wreg[STEPS][3][4];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
-    const uint32_t* p = a.w + (size_t)(3 * gclamp[s]) * row_stride + col;
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
-      u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(p + j * row_stride));
+      const uint32_t off = (glc[s] * 3u + (uint32_t)j) * row_bytes + col_off;
+      u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wbase + off));
       wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
     }
   }
@@ -168,31 +171,32 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   asum = wave_sum(asum);
   // 2^E * max|x| lies in [2^14, 2^15): digit 0 never overflows fp16.
   int E = 14 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
-  E = xmax > 0.f ? max(-100, min(100, E)) : 0;
+  E = xmax > 0.f ? max(-120, min(120, E)) : 0;
   const float scaleE = pow2f(E);
   uint4* xs_w = xs + wv * (STEPS * 64);
-  const float sl_lo = pow2f(4 - p_lo), sl_hi = pow2f(4 - p_hi);  // digit * 2^(4-pos) fits fp16 exactly
+  // Fixed-point split of v = x * 2^(E + 4 - pos) (|v| < 2^(19-pos)) into three signed
+  // 11-bit digits with quanta 2^9, 2^-2, 2^-13, stored as plain fp16 integers.  With the
+  // operand value code*2^(pos-24) every digit-0 product is an integer below 2^13 in units
+  // of 2^-24, so a wave's digit-0 chain (at most 512 slots) is exact in the matrix core
+  // whatever its internal rounding is; digits 1 and 2 carry 2^-11 and 2^-22 of the weight.
+  const float sE_lo = scaleE * pow2f(4 - p_lo), sE_hi = scaleE * pow2f(4 - p_hi);
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
-    // Fixed-point split of u = x*2^E (|u| < 2^15) into three signed 11-bit digits with
-    // quanta 2^5, 2^-6, 2^-17.  Every MFMA product is then an integer multiple of one
-    // quantum and a wave's partial sums stay below 2^24 quanta, so the matrix-core
-    // accumulation is exact whatever its internal rounding is.
     float d[2][3];
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
-      const float u = xr[s][e] * scaleE;
-      d[e][0] = rintf(u * 0.03125f);
-      const float r1 = u - d[e][0] * 32.f;        // exact
-      d[e][1] = rintf(r1 * 64.f);
-      const float r2 = r1 - d[e][1] * 0.015625f;  // exact
-      d[e][2] = rintf(r2 * 131072.f);
+      const float v = xr[s][e] * (e ? sE_hi : sE_lo);
+      d[e][0] = rintf(v * 0.001953125f);
+      const float r1 = v - d[e][0] * 512.f;   // exact
+      d[e][1] = rintf(r1 * 4.f);
+      const float r2 = r1 - d[e][1] * 0.25f;  // exact
+      d[e][2] = rintf(r2 * 8192.f);
     }
     // register c of MFMA j = c/4 of this k-group: dword c%4 of the 16-byte operand chunk
     uint32_t* dst = reinterpret_cast<uint32_t*>(xs_w + ((s * 4 + kb) * 4 + (c >> 2)) * 4) + (c & 3);
 #pragma unroll
     for (int p = 0; p < 3; ++p) {
-      const h2v pair = {(_Float16)(d[0][p] * sl_lo), (_Float16)(d[1][p] * sl_hi)};
+      const h2v pair = {(_Float16)d[0][p], (_Float16)d[1][p]};
       dst[4 * p] = __builtin_bit_cast(uint32_t, pair);
     }
   }
@@ -214,16 +218,18 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     h8 B[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) B[j] = __builtin_bit_cast(h8, xb[j * 4]);
+    // the four columns' chains are independent: issue them round-robin so that no MFMA
+    // waits for the one before it
+    uint32_t f[4][16];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      uint32_t f[16];
-      unpack16(wreg[s][0][q], wreg[s][1][q], wreg[s][2][q], f);
+    for (int q = 0; q < 4; ++q) unpack16(wreg[s][0][q], wreg[s][1][q], wreg[s][2][q], f[q]);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        u4v av = {f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]};
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        u4v av = {f[q][4 * j], f[q][4 * j + 1], f[q][4 * j + 2], f[q][4 * j + 3]};
         acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), B[j], acc[q], 0, 0, 0);
       }
-    }
   }
 
   // ---- combine waves, digits, scale/zero --------------------------------------------------
@@ -248,8 +254,8 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
       const float c0 = red[(w * 3 + 0) * 64 + tid];
       const float c1 = red[(w * 3 + 1) * 64 + tid];
       const float c2 = red[(w * 3 + 2) * 64 + tid];
-      // 2^20 (operand scale) * 2^5 (digit-0 quantum) / 2^E
-      qx += fmaf(fmaf(c2, inv11, c1), inv11, c0) * 33554432.f * desc[w];
+      // 2^24 (operand scale) * 2^9 (digit-0 quantum) * 2^-4 (slot scale) / 2^E
+      qx += fmaf(fmaf(c2, inv11, c1), inv11, c0) * 536870912.f * desc[w];
       xsum += wsum[w];
     }
     val = sc_n * qx - zr_n * xsum;
@@ -340,7 +346,7 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   int steps = hq_env_int("HQ_Q3_STEPS", 2);
   int nsplit = 0;
   if (waves != 4 && waves != 8 && waves != 16) waves = 16;
-  if (steps != 1 && steps != 2 && steps != 4) steps = 2;
+  if (steps != 1 && steps != 2 && steps != 4 && steps != 8) steps = 2;
   const int gpr = waves * 4 * steps;  // k-groups one workgroup covers
   (void)nsplit;
   nsplit = (G + gpr - 1) / gpr;
@@ -361,7 +367,7 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   if (waves == W && steps == S) return launch_matvec<W, S>(a, ntiles, stream);
   HQ_Q3_CASE(16, 1) HQ_Q3_CASE(16, 2) HQ_Q3_CASE(16, 4)
   HQ_Q3_CASE(8, 1) HQ_Q3_CASE(8, 2) HQ_Q3_CASE(8, 4)
-  HQ_Q3_CASE(4, 1) HQ_Q3_CASE(4, 2) HQ_Q3_CASE(4, 4)
+  HQ_Q3_CASE(4, 1) HQ_Q3_CASE(4, 2) HQ_Q3_CASE(4, 4) HQ_Q3_CASE(4, 8) HQ_Q3_CASE(8, 8)
 #undef HQ_Q3_CASE
   return HQ_ERR_BAD_ENUM;
 }

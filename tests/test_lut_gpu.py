@@ -20,16 +20,20 @@ def _run(hq, bW, alpha, qbias, x, group):
     return y.cpu().numpy()
 
 
+@pytest.mark.parametrize("path", [1, 0])  # 1: matrix-core kernel where the shape allows, 0: table kernel
 @pytest.mark.parametrize("K,N,nb,group,zero_bias,seed", [
     (4096, 16384, 3, 128, True, 1), (4096, 16384, 3, 128, False, 2), (1024, 4096, 8, 128, False, 3),
     (1024, 4096, 4, 128, False, 4), (512, 130, 3, 64, False, 5), (96, 64, 1, 32, False, 6),
-    (2048, 1001, 2, 2048, False, 7), (1536, 256, 3, 512, False, 8)])
-def test_vs_oracle(hq, oracle, K, N, nb, group, zero_bias, seed):
+    (2048, 1001, 2, 2048, False, 7), (1536, 256, 3, 512, False, 8), (640, 192, 5, 128, False, 9),
+    (8192, 64, 7, 256, False, 10), (384, 128, 6, 384, False, 11)])
+def test_vs_oracle(hq, oracle, monkeypatch, path, K, N, nb, group, zero_bias, seed):
+    monkeypatch.setenv("HQ_LUT_PATH", str(path))
     bW, alpha, qbias, x = oa.make_lut_problem(seed, K, N, nb, group, zero_bias)
     y = _run(hq, bW, alpha, qbias, x, group)
     ref = oracle.lut_gemv_f64(bW, alpha, qbias, x, group)
-    # fp32 sums rounded once to fp16: half an fp16 ulp of the result, far inside the fp16-accumulate bound
-    assert rel_err(y, ref) <= 2e-3
+    # fp32 sums rounded once to fp16 (the matrix-core path adds a truncation bias of
+    # ~4e-5 of the RMS, a fifth of the fp16 output rounding): far inside the contract
+    assert rel_err(y, ref, FLOOR_F16) <= 2e-3
     assert rel_err(y, ref) <= TOL_F16_ACC
 
 
@@ -37,7 +41,8 @@ def test_no_bias_pointer(hq, oracle):
     bW, alpha, _, x = oa.make_lut_problem(9, 1024, 512, 3, 128)
     y = _run(hq, bW, alpha, None, x, 128)
     ref = oracle.lut_gemv_f64(bW, alpha, None, x, 128)
-    assert rel_err(y, ref) <= 2e-3
+    assert rel_err(y, ref, FLOOR_F16) <= 2e-3
+    assert rel_err(y, ref) <= TOL_F16_ACC
 
 
 def test_closed_forms(hq, oracle):
