@@ -89,15 +89,13 @@ __device__ __forceinline__ void unpack16(uint32_t w0, uint32_t w1, uint32_t w2, 
   for (int r = 0; r < 16; ++r) a[r] = win[kRecipe[r].window] & mask_of(r);
 }
 
-template <int WAVES, int STEPS, bool XF16>
+template <int WAVES, int STEPS, bool XF16, bool MULTI>
 __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
-  // One round per workgroup: the host sizes gpw <= WAVES*4*STEPS.
-  // LDS: xs[WAVES][STEPS*4 groups][4 mfma][4 piece slots] uint4 | red[WAVES][3][64] | desc[WAVES] | xsum[WAVES]
+  // LDS: xs[WAVES][STEPS*4 groups][4 mfma][4 piece slots] uint4 | red[WAVES][3][64] | xsum[WAVES]
   extern __shared__ uint4 smem[];
   uint4* xs = smem;
   float* red = reinterpret_cast<float*>(smem + WAVES * STEPS * 64);
-  float* desc = red + WAVES * 3 * 64;
-  float* wsum = desc + WAVES;
+  float* wsum = red + WAVES * 3 * 64;
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int c = lane & 15, kb = lane >> 4;
@@ -108,9 +106,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   const size_t row_stride = (size_t)a.N;
   const int n = tile * 64 + tid;
 
-  // ---- issue every global load of this wave up front -------------------------------
-  // No load sits under a branch (addresses are clamped instead), so the compiler can
-  // count them and the wait for the activations does not wait for the weights.
+  // ---- loads that do not depend on the round ------------------------------------------------
   float sc_n = 0.f, zr_n = 0.f, y_old = 0.f;
   if (tid < 64) {
     const int nc = min(n, a.N - 1);
@@ -126,110 +122,145 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   const int k_lo = te & 31, k_hi = (te >> 5) & 31, p_lo = (te >> 10) & 7, p_hi = (te >> 13) & 7;
   // Scalar base pointers of this workgroup's slice plus 32-bit per-lane byte offsets.
   const char* xbase = reinterpret_cast<const char*>(a.x) + (size_t)g_begin * 32 * (XF16 ? 2 : 4);
-  float xr[STEPS][2];
-  uint32_t glc[STEPS];
-#pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-    glc[s] = (uint32_t)min(s * (WAVES * 4) + wv * 4 + kb, g_count - 1);
-    if (XF16) {
-      xr[s][0] = (float)*reinterpret_cast<const _Float16*>(xbase + (glc[s] * 32u + (uint32_t)k_lo) * 2u);
-      xr[s][1] = (float)*reinterpret_cast<const _Float16*>(xbase + (glc[s] * 32u + (uint32_t)k_hi) * 2u);
-    } else {
-      xr[s][0] = *reinterpret_cast<const float*>(xbase + (glc[s] * 32u + (uint32_t)k_lo) * 4u);
-      xr[s][1] = *reinterpret_cast<const float*>(xbase + (glc[s] * 32u + (uint32_t)k_hi) * 4u);
-    }
-  }
   // weights: out-of-range columns read the last valid quad (their results are never
-  // stored), out-of-range k-groups read a valid group and get zero activations below
+  // stored), out-of-range k-groups read a valid group and get zero activations
   const int tile_cols = min(64, a.N - tile * 64);           // multiple of 4
   const uint32_t col_off = (uint32_t)min(4 * c, tile_cols - 4) * 4u;
   const uint32_t row_bytes = (uint32_t)a.N * 4u;
   const char* wbase = reinterpret_cast<const char*>(a.w) + ((size_t)(3 * g_begin) * row_stride + (size_t)tile * 64) * 4;
-  uint32_t wreg[STEPS][3][4];
-#pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-#pragma unroll
-    for (int j = 0; j < 3; ++j) {
-      const uint32_t off = (glc[s] * 3u + (uint32_t)j) * row_bytes + col_off;
-      u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wbase + off));
-      wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
-    }
-  }
-#pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-    if (s * (WAVES * 4) + wv * 4 + kb >= g_count) { xr[s][0] = 0.f; xr[s][1] = 0.f; }
-  }
+  constexpr int GPR = WAVES * 4 * STEPS;  // k-groups per round
+  const int rounds = MULTI ? (g_count + GPR - 1) / GPR : 1;  // !MULTI: the host sized gpw <= GPR
 
-  // ---- stage this wave's activation digits in operand-slot order (wave-local) ----------
-  float amax = 0.f, asum = 0.f;
+  // Every global load of a round is issued up front and none sits under a branch
+  // (addresses are clamped instead), so the compiler can count them and the wait for the
+  // activations does not wait for the weights.
+  auto load_round = [&](int r, float (&xr)[STEPS][2], uint32_t (&wreg)[STEPS][3][4]) {
+    uint32_t glc[STEPS];
 #pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-    amax = fmaxf(amax, fmaxf(fabsf(xr[s][0]), fabsf(xr[s][1])));
-    asum += xr[s][0] + xr[s][1];
-  }
-  const float xmax = wave_max(amax);
-  asum = wave_sum(asum);
-  // 2^E * max|x| lies in [2^14, 2^15): digit 0 never overflows fp16.
-  int E = 14 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
-  E = xmax > 0.f ? max(-120, min(120, E)) : 0;
-  const float scaleE = pow2f(E);
+    for (int s = 0; s < STEPS; ++s) {
+      glc[s] = (uint32_t)min((r * STEPS + s) * (WAVES * 4) + wv * 4 + kb, g_count - 1);
+      if (XF16) {
+        xr[s][0] = (float)*reinterpret_cast<const _Float16*>(xbase + (glc[s] * 32u + (uint32_t)k_lo) * 2u);
+        xr[s][1] = (float)*reinterpret_cast<const _Float16*>(xbase + (glc[s] * 32u + (uint32_t)k_hi) * 2u);
+      } else {
+        xr[s][0] = *reinterpret_cast<const float*>(xbase + (glc[s] * 32u + (uint32_t)k_lo) * 4u);
+        xr[s][1] = *reinterpret_cast<const float*>(xbase + (glc[s] * 32u + (uint32_t)k_hi) * 4u);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const uint32_t off = (glc[s] * 3u + (uint32_t)j) * row_bytes + col_off;
+        u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wbase + off));
+        wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
+      }
+    }
+  };
+
   uint4* xs_w = xs + wv * (STEPS * 64);
-  // Fixed-point split of v = x * 2^(E + 4 - pos) (|v| < 2^(19-pos)) into three signed
-  // 11-bit digits with quanta 2^9, 2^-2, 2^-13, stored as plain fp16 integers.  With the
-  // operand value code*2^(pos-24) every digit-0 product is an integer below 2^13 in units
-  // of 2^-24, so a wave's digit-0 chain (at most 512 slots) is exact in the matrix core
-  // whatever its internal rounding is; digits 1 and 2 carry 2^-11 and 2^-22 of the weight.
-  const float sE_lo = scaleE * pow2f(4 - p_lo), sE_hi = scaleE * pow2f(4 - p_hi);
-#pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-    float d[2][3];
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      const float v = xr[s][e] * (e ? sE_hi : sE_lo);
-      d[e][0] = rintf(v * 0.001953125f);
-      const float r1 = v - d[e][0] * 512.f;   // exact
-      d[e][1] = rintf(r1 * 4.f);
-      const float r2 = r1 - d[e][1] * 0.25f;  // exact
-      d[e][2] = rintf(r2 * 8192.f);
-    }
-    // register c of MFMA j = c/4 of this k-group: dword c%4 of the 16-byte operand chunk
-    uint32_t* dst = reinterpret_cast<uint32_t*>(xs_w + ((s * 4 + kb) * 4 + (c >> 2)) * 4) + (c & 3);
-#pragma unroll
-    for (int p = 0; p < 3; ++p) {
-      const h2v pair = {(_Float16)d[0][p], (_Float16)d[1][p]};
-      dst[4 * p] = __builtin_bit_cast(uint32_t, pair);
-    }
-  }
-  // The digits are read back by other lanes of this wave only: order the LDS writes
-  // before the reads without a workgroup barrier.
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-
-  // ---- unpack + MFMA -----------------------------------------------------------------------
-  f4 acc[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
   const int piece = c < 3 ? c : 2;  // columns 3..15 of the MFMA are never read
+  float run[4][4];                  // per-digit sums of all rounds, already divided by 2^E
 #pragma unroll
-  for (int s = 0; s < STEPS; ++s) {
-    if (s * (WAVES * 4) + wv * 4 >= g_count) continue;  // wave-uniform
-    const uint4* xb = xs_w + (size_t)(s * 4 + kb) * 16 + piece;
-    h8 B[4];
+  for (int q = 0; q < 4; ++q)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) B[j] = __builtin_bit_cast(h8, xb[j * 4]);
-    // the four columns' chains are independent: issue them round-robin so that no MFMA
-    // waits for the one before it
-    uint32_t f[4][16];
+    for (int i = 0; i < 4; ++i) run[q][i] = 0.f;
+  float asum_total = 0.f;
+
+  float xr[STEPS][2];
+  uint32_t wreg[STEPS][3][4];
+  load_round(0, xr, wreg);
+  for (int r = 0; r < rounds; ++r) {
+    float xr_next[STEPS][2];
+    uint32_t wreg_next[STEPS][3][4];
+    if (MULTI && r + 1 < rounds) load_round(r + 1, xr_next, wreg_next);  // in flight during this round
+
+    // ---- stage this wave's activation digits in operand-slot order (wave-local) ----------
+    float amax = 0.f, asum = 0.f;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) unpack16(wreg[s][0][q], wreg[s][1][q], wreg[s][2][q], f[q]);
+    for (int s = 0; s < STEPS; ++s) {
+      if ((r * STEPS + s) * (WAVES * 4) + wv * 4 + kb >= g_count) { xr[s][0] = 0.f; xr[s][1] = 0.f; }
+      amax = fmaxf(amax, fmaxf(fabsf(xr[s][0]), fabsf(xr[s][1])));
+      asum += xr[s][0] + xr[s][1];
+    }
+    const float xmax = wave_max(amax);
+    asum_total += wave_sum(asum);
+    // 2^E * max|x| lies in [2^14, 2^15): digit 0 never overflows fp16.
+    int E = 14 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
+    E = xmax > 0.f ? max(-120, min(120, E)) : 0;
+    const float scaleE = pow2f(E);
+    // Fixed-point split of v = x * 2^(E + 4 - pos) (|v| < 2^(19-pos)) into three signed
+    // 11-bit digits with quanta 2^9, 2^-2, 2^-13, stored as plain fp16 integers.  With the
+    // operand value code*2^(pos-24) every digit-0 product is an integer below 2^13 in units
+    // of 2^-24, so a round's digit-0 chain (at most 512 slots) is exact in the matrix core
+    // whatever its internal rounding is; digits 1 and 2 carry 2^-11 and 2^-22 of the weight.
+    const float sE_lo = scaleE * pow2f(4 - p_lo), sE_hi = scaleE * pow2f(4 - p_hi);
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int s = 0; s < STEPS; ++s) {
+      float d[2][3];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const float v = xr[s][e] * (e ? sE_hi : sE_lo);
+        d[e][0] = rintf(v * 0.001953125f);
+        const float r1 = v - d[e][0] * 512.f;   // exact
+        d[e][1] = rintf(r1 * 4.f);
+        const float r2 = r1 - d[e][1] * 0.25f;  // exact
+        d[e][2] = rintf(r2 * 8192.f);
+      }
+      // register c of MFMA j = c/4 of this k-group: dword c%4 of the 16-byte operand chunk
+      uint32_t* dst = reinterpret_cast<uint32_t*>(xs_w + ((s * 4 + kb) * 4 + (c >> 2)) * 4) + (c & 3);
+#pragma unroll
+      for (int p = 0; p < 3; ++p) {
+        const h2v pair = {(_Float16)d[0][p], (_Float16)d[1][p]};
+        dst[4 * p] = __builtin_bit_cast(uint32_t, pair);
+      }
+    }
+    // The digits are read back by other lanes of this wave only: order the LDS writes
+    // before the reads without a workgroup barrier.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+
+    // ---- unpack + MFMA ---------------------------------------------------------------------
+    f4 acc[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      if ((r * STEPS + s) * (WAVES * 4) + wv * 4 >= g_count) continue;  // wave-uniform
+      const uint4* xb = xs_w + (size_t)(s * 4 + kb) * 16 + piece;
+      h8 B[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) B[j] = __builtin_bit_cast(h8, xb[j * 4]);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        u4v av = {f[q][4 * j], f[q][4 * j + 1], f[q][4 * j + 2], f[q][4 * j + 3]};
-        acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), B[j], acc[q], 0, 0, 0);
+        uint32_t f[16];
+        unpack16(wreg[s][0][q], wreg[s][1][q], wreg[s][2][q], f);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          u4v av = {f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]};
+          acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), B[j], acc[q], 0, 0, 0);
+        }
       }
+    }
+    const float descale = pow2f(-E);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) run[q][i] = fmaf(acc[q][i], descale, run[q][i]);
+    // the LDS digits of this round must be consumed before the next round overwrites them
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    if (MULTI && r + 1 < rounds) {
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        xr[s][0] = xr_next[s][0]; xr[s][1] = xr_next[s][1];
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) wreg[s][j][q] = wreg_next[s][j][q];
+      }
+    }
   }
 
   // ---- combine waves, digits, scale/zero --------------------------------------------------
@@ -238,12 +269,9 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) red[(wv * 3 + c) * 64 + 4 * (4 * kb + i) + q] = acc[q][i];
+      for (int i = 0; i < 4; ++i) red[(wv * 3 + c) * 64 + 4 * (4 * kb + i) + q] = run[q][i];
   }
-  if (lane == 0) {
-    desc[wv] = pow2f(-E);
-    wsum[wv] = asum;
-  }
+  if (lane == 0) wsum[wv] = asum_total;
   __syncthreads();
   float val = 0.f;
   if (tid < 64 && n < a.N) {
@@ -254,11 +282,11 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
       const float c0 = red[(w * 3 + 0) * 64 + tid];
       const float c1 = red[(w * 3 + 1) * 64 + tid];
       const float c2 = red[(w * 3 + 2) * 64 + tid];
-      // 2^24 (operand scale) * 2^9 (digit-0 quantum) * 2^-4 (slot scale) / 2^E
-      qx += fmaf(fmaf(c2, inv11, c1), inv11, c0) * 536870912.f * desc[w];
+      qx += fmaf(fmaf(c2, inv11, c1), inv11, c0);
       xsum += wsum[w];
     }
-    val = sc_n * qx - zr_n * xsum;
+    // 2^24 (operand scale) * 2^9 (digit-0 quantum) * 2^-4 (slot scale)
+    val = sc_n * (qx * 536870912.f) - zr_n * xsum;
     if (a.nsplit == 1) {
       a.y[n] = y_old + val;
     } else {
@@ -297,21 +325,25 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   }
 }
 
-template <int WAVES, int STEPS, bool XF16>
+template <int WAVES, int STEPS, bool XF16, bool MULTI>
 int launch_matvec_t(const Q3Args& a, int ntiles, hipStream_t stream) {
   const size_t smem = (size_t)WAVES * STEPS * 1024 + (size_t)WAVES * 3 * 64 * 4 + (size_t)WAVES * 2 * 4;
   static const hipError_t attr =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_matvec_kernel<WAVES, STEPS, XF16>),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_matvec_kernel<WAVES, STEPS, XF16, MULTI>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
   if (attr != hipSuccess) return (int)attr;
-  hipLaunchKernelGGL((q3_matvec_kernel<WAVES, STEPS, XF16>), dim3(ntiles, a.nsplit), dim3(WAVES * 64), smem,
+  hipLaunchKernelGGL((q3_matvec_kernel<WAVES, STEPS, XF16, MULTI>), dim3(ntiles, a.nsplit), dim3(WAVES * 64), smem,
                      stream, a);
   return hq_launch_status();
 }
 template <int WAVES, int STEPS>
 int launch_matvec(const Q3Args& a, int ntiles, hipStream_t stream) {
-  return a.x_f16 ? launch_matvec_t<WAVES, STEPS, true>(a, ntiles, stream)
-                 : launch_matvec_t<WAVES, STEPS, false>(a, ntiles, stream);
+  const bool multi = a.gpw > WAVES * 4 * STEPS;
+  if (a.x_f16)
+    return multi ? launch_matvec_t<WAVES, STEPS, true, true>(a, ntiles, stream)
+                 : launch_matvec_t<WAVES, STEPS, true, false>(a, ntiles, stream);
+  return multi ? launch_matvec_t<WAVES, STEPS, false, true>(a, ntiles, stream)
+               : launch_matvec_t<WAVES, STEPS, false, false>(a, ntiles, stream);
 }
 
 }  // namespace
@@ -340,17 +372,27 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
 
   const int G = K / 32;
   const int ntiles = (N + 63) / 64;
-  // Launch shape: WAVES waves per workgroup, each streaming STEPS k-groups per
-  // 16-lane quarter; K is split over ceil(G / (WAVES*4*STEPS)) workgroups per tile.
-  int waves = hq_env_int("HQ_Q3_WAVES", 16);
-  int steps = hq_env_int("HQ_Q3_STEPS", 2);
-  int nsplit = 0;
-  if (waves != 4 && waves != 8 && waves != 16) waves = 16;
-  if (steps != 1 && steps != 2 && steps != 4 && steps != 8) steps = 2;
-  const int gpr = waves * 4 * steps;  // k-groups one workgroup covers
-  (void)nsplit;
-  nsplit = (G + gpr - 1) / gpr;
-  const int gpw = gpr;
+  // Launch shape: a workgroup of WAVES waves covers WAVES*4*STEPS k-groups per round and
+  // walks its K range in rounds (the next round's loads are in flight during the current
+  // one).  K is split across workgroups only as far as needed to give every CU a
+  // workgroup: the split costs a device-scope round trip per workgroup.
+  int waves = hq_env_int("HQ_Q3_WAVES", 8);
+  int steps = hq_env_int("HQ_Q3_STEPS", 0);
+  if (waves != 4 && waves != 8 && waves != 16) waves = 8;
+  if (waves == 16) steps = 1;  // register budget of 16-wave workgroups
+  if (steps != 1 && steps != 2 && steps != 4 && (steps != 8 || waves != 4)) {
+    steps = 4;
+    while (steps > 1 && waves * 4 * (steps / 2) >= G) steps /= 2;  // short K: fewer steps
+  }
+  const int gpr = waves * 4 * steps;  // k-groups one workgroup covers per round
+  const int max_split = (G + gpr - 1) / gpr;
+  int nsplit = hq_env_int("HQ_Q3_KSPLIT", 0);
+  if (nsplit <= 0) nsplit = dev->cus / ntiles;  // only when there are fewer tiles than half the CUs
+  if (nsplit > max_split) nsplit = max_split;
+  if (nsplit < 1) nsplit = 1;
+  int gpw = (G + nsplit - 1) / nsplit;
+  gpw = (gpw + gpr - 1) / gpr * gpr;  // whole rounds
+  nsplit = (G + gpw - 1) / gpw;
 
   Q3Args a;
   a.x = x; a.w = reinterpret_cast<const uint32_t*>(qweight); a.scales = scales; a.zeros = zeros;
@@ -365,9 +407,9 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   }
 #define HQ_Q3_CASE(W, S) \
   if (waves == W && steps == S) return launch_matvec<W, S>(a, ntiles, stream);
-  HQ_Q3_CASE(16, 1) HQ_Q3_CASE(16, 2) HQ_Q3_CASE(16, 4)
+  HQ_Q3_CASE(16, 1)
   HQ_Q3_CASE(8, 1) HQ_Q3_CASE(8, 2) HQ_Q3_CASE(8, 4)
-  HQ_Q3_CASE(4, 1) HQ_Q3_CASE(4, 2) HQ_Q3_CASE(4, 4) HQ_Q3_CASE(4, 8) HQ_Q3_CASE(8, 8)
+  HQ_Q3_CASE(4, 1) HQ_Q3_CASE(4, 2) HQ_Q3_CASE(4, 4) HQ_Q3_CASE(4, 8)
 #undef HQ_Q3_CASE
   return HQ_ERR_BAD_ENUM;
 }

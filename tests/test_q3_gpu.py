@@ -111,18 +111,20 @@ def test_wide_dynamic_range_and_zero_vector(hq, oracle):
 
 
 def test_launch_shapes_match(hq, oracle, monkeypatch):
-    """Every launch shape (waves per workgroup x steps; K split over 1..8 workgroups
-    per tile) gives the same answer."""
+    """Every launch shape (waves per workgroup x steps x K split; one or several
+    rounds per workgroup) gives the same answer."""
     K, N = 4096, 1024
     codes, scales, zeros, x = oa.make_q3_problem(41, K, N)
     mat = oracle.q3_pack(codes)
     ref = oracle.q3_matvec_f64(x, mat, scales, zeros)
-    for waves, steps in [(16, 2), (8, 2), (4, 2), (4, 1), (16, 1), (8, 4), (4, 4), (16, 4), (8, 1)]:
+    for waves, steps, ks in [(8, 4, 0), (8, 2, 0), (4, 2, 1), (4, 1, 0), (16, 1, 1), (8, 4, 1), (4, 4, 2), (4, 8, 0),
+                             (8, 1, 3), (8, 1, 1), (4, 1, 1)]:
         monkeypatch.setenv("HQ_Q3_WAVES", str(waves))
         monkeypatch.setenv("HQ_Q3_STEPS", str(steps))
+        monkeypatch.setenv("HQ_Q3_KSPLIT", str(ks))
         for _ in range(2):  # twice: the arrival counters must reset themselves
             y = _run(hq, x, mat, scales, zeros)
-            assert rel_err(y, ref) <= 1e-4, (waves, steps)
+            assert rel_err(y, ref) <= 1e-4, (waves, steps, ks)
 
 
 def test_rejects_bad_arguments(hq):
