@@ -2,13 +2,16 @@
  * hq_oracle.c — CPU restatement of the reference arithmetic.  TEST
  * INFRASTRUCTURE ONLY (see hq_oracle.h): never linked into the product library.
  *
- * Build: gcc -O2 -ffp-contract=off -fPIC -shared hq_oracle.c -o libhq_oracle.so -lm
+ * Build: gcc -O2 -ffp-contract=off -fopenmp -fPIC -shared hq_oracle.c -o libhq_oracle.so -lm
  * (-ffp-contract=off matters: the fp32 restatements round after every multiply
  * and add, which is what the functions below document).
  */
 #include "hq_oracle.h"
 
 #include <math.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 #include <stdlib.h>
 #include <string.h>
 
@@ -121,17 +124,20 @@ void hqo_q3_unpack(const int32_t* mat, int K, int N, uint8_t* codes) {
     }
 }
 
-void hqo_q3_matvec_f32(const float* x, const int32_t* mat, float* mul,
-                       const float* scales, const float* zeros, int K, int N) {
+/* Columns [n0, n1) of the fp32 kernel; every column sees exactly the arithmetic of the
+ * reference thread that owns it, so any column partition gives identical results. */
+static void q3_matvec_f32_cols(const float* x, const int32_t* mat, float* mul, const float* scales,
+                               const float* zeros, int K, int N, int n0, int n1) {
   /* One 256-row block (8 groups) at a time, as the reference grid does
    * (BLOCKWIDTH=256, BLOCKHEIGHT=24, kernels.h:5-6,22-23). */
-  float* res = (float*)malloc(sizeof(float) * (size_t)N);
+  int W = n1 - n0;
+  float* res = (float*)malloc(sizeof(float) * (size_t)(W > 0 ? W : 1));
   int G = K / 32;
   for (int g0 = 0; g0 < G; g0 += 8) {
-    for (int n = 0; n < N; ++n) res[n] = 0.f;
+    for (int n = 0; n < W; ++n) res[n] = 0.f;
     int g1 = g0 + 8 < G ? g0 + 8 : G;
     for (int g = g0; g < g1; ++g) {
-      const uint32_t* r0 = (const uint32_t*)mat + (size_t)(3 * g) * N;
+      const uint32_t* r0 = (const uint32_t*)mat + (size_t)(3 * g) * N + n0;
       const uint32_t* r1 = r0 + N;
       const uint32_t* r2 = r1 + N;
       for (int i = 0; i < 32; ++i) {
@@ -140,21 +146,42 @@ void hqo_q3_matvec_f32(const float* x, const int32_t* mat, float* mul,
         const uint32_t* ra = wd == 0 ? r0 : (wd == 1 ? r1 : r2);
         const uint32_t* rb = wd == 0 ? r1 : r2;
         if (sh <= 29) {
-          for (int n = 0; n < N; ++n) {
+          for (int n = 0; n < W; ++n) {
             float q = (float)((ra[n] >> sh) & 7u);
-            res[n] += (scales[n] * q - zeros[n]) * xv; /* kernels.h:43-84 */
+            res[n] += (scales[n0 + n] * q - zeros[n0 + n]) * xv; /* kernels.h:43-84 */
           }
         } else {
-          for (int n = 0; n < N; ++n) {
+          for (int n = 0; n < W; ++n) {
             float q = (float)(((ra[n] >> sh) | (rb[n] << (32 - sh))) & 7u);
-            res[n] += (scales[n] * q - zeros[n]) * xv;
+            res[n] += (scales[n0 + n] * q - zeros[n0 + n]) * xv;
           }
         }
       }
     }
-    for (int n = 0; n < N; ++n) mul[n] += res[n]; /* atomicAdd, kernels.h:89 */
+    for (int n = 0; n < W; ++n) mul[n0 + n] += res[n]; /* atomicAdd, kernels.h:89 */
   }
   free(res);
+}
+
+void hqo_q3_matvec_f32(const float* x, const int32_t* mat, float* mul,
+                       const float* scales, const float* zeros, int K, int N) {
+  q3_matvec_f32_cols(x, mat, mul, scales, zeros, K, N, 0, N);
+}
+
+int hqo_q3_matvec_f32_omp(const float* x, const int32_t* mat, float* mul,
+                          const float* scales, const float* zeros, int K, int N) {
+  int threads = 1;
+#ifdef _OPENMP
+  threads = omp_get_max_threads();
+#endif
+  int chunk = 256; /* one reference block of columns per task */
+  int nchunks = (N + chunk - 1) / chunk;
+#pragma omp parallel for schedule(dynamic)
+  for (int c = 0; c < nchunks; ++c) {
+    int n0 = c * chunk, n1 = n0 + chunk < N ? n0 + chunk : N;
+    q3_matvec_f32_cols(x, mat, mul, scales, zeros, K, N, n0, n1);
+  }
+  return threads;
 }
 
 void hqo_q3_matvec_f64(const double* x, const int32_t* mat, double* y,

@@ -57,6 +57,11 @@ void hqo_q3_unpack(const int32_t* mat, int K, int N, uint8_t* codes);
 void hqo_q3_matvec_f32(const float* x, const int32_t* mat, float* mul,
                        const float* scales, const float* zeros, int K, int N);
 
+/* The same kernel with the columns spread over OpenMP threads (identical results: each
+ * column keeps its arithmetic order).  Returns the number of threads used. */
+int hqo_q3_matvec_f32_omp(const float* x, const int32_t* mat, float* mul,
+                          const float* scales, const float* zeros, int K, int N);
+
 /* Same sum in double precision, written to y (overwrites). */
 void hqo_q3_matvec_f64(const double* x, const int32_t* mat, double* y,
                        const float* scales, const float* zeros, int K, int N);

@@ -56,6 +56,14 @@ class Oracle:
                                    _p(zeros), K, N)
         return mul
 
+    def q3_matvec_f32_omp(self, x, mat, scales, zeros, mul=None):
+        """Returns (result, threads used)."""
+        K, N = x.size, mat.shape[1]
+        mul = np.zeros(N, np.float32) if mul is None else mul
+        threads = self.lib.hqo_q3_matvec_f32_omp(_p(np.ascontiguousarray(x, np.float32)), _p(mat), _p(mul),
+                                                 _p(scales), _p(zeros), K, N)
+        return mul, threads
+
     def q3_matvec_f64(self, x, mat, scales, zeros):
         K, N = x.size, mat.shape[1]
         y = np.zeros(N, np.float64)

@@ -2,6 +2,7 @@
 (compiled from the reference tree into oracle/_ref where that tree is mounted),
 closed forms, invariants and brute force.  Runs without a GPU."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -102,6 +103,9 @@ def test_q3_matvec_closed_forms_and_dense(o):
     xi = rng.integers(-8, 9, K).astype(np.float32)
     y = o.q3_matvec_f32(xi, mat, np.ones(N, np.float32), np.zeros(N, np.float32))
     assert np.array_equal(y.astype(np.int64), xi.astype(np.int64) @ codes.astype(np.int64))
+    # the OpenMP partition over columns changes nothing
+    yo, threads = o.q3_matvec_f32_omp(x, mat, s, z)
+    assert threads >= 1 and np.array_equal(yo, o.q3_matvec_f32(x, mat, s, z))
     # accumulate semantics of the reference (mul +=)
     y2 = o.q3_matvec_f32(xi, mat, np.ones(N, np.float32), np.zeros(N, np.float32), mul=np.full(N, 5, np.float32))
     assert np.array_equal(y2, y + 5)
@@ -283,3 +287,31 @@ def test_aqlm_closed_forms(o):
         book = cb3[m // 4].astype(np.float64)
         want = sum(book[int(np.uint16(codes[m, g]))] @ x[8 * g:8 * g + 8].astype(np.float64) for g in range(K // 8))
         assert np.isclose(y[m], want * float(sc[m]), rtol=1e-12, atol=1e-12)
+
+
+# ------------------------------------------------------------------ committed golden fixtures
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_golden_lut_fixture(o):
+    """Bit planes, alphas, biases and dense weights written by the reference's own host
+    loops (tests/golden/make_golden.py); needs neither the reference tree nor oracle/_ref."""
+    f = np.load(os.path.join(GOLDEN, "lut_fixture_256x256x3.npz"))
+    assert np.array_equal(o.bcq_pack(f["signs"]), f["bW"])
+    a16, b16 = f["alpha"].astype(np.float16), f["q_bias"].astype(np.float16)
+    W = o.bcq_dequant(f["bW"], a16, b16, 128)
+    assert np.allclose(W, f["weight"].T, atol=2e-3)  # reference keeps fp32 alphas, the kernels fp16
+    x16 = f["input"].astype(np.float16)
+    y = o.lut_gemv_f64(f["bW"], a16, b16, x16, 128)
+    assert np.allclose(y, x16.astype(np.float64) @ f["weight"].T.astype(np.float64), atol=5e-2)
+
+
+def test_golden_dquantize_outputs(o):
+    """Outputs of the reference host quantiser on a fixed vector.  The reference table is
+    not committed; the generated dynamic map differs from it by at most 2 ulps in a few
+    entries, which can move an input sitting within an ulp of a midpoint: allow 0.1%."""
+    f = np.load(os.path.join(GOLDEN, "dquantize_outputs.npz"))
+    got = o.quantize_dynamic8(o.dynamic_map(), f["A"])
+    assert np.mean(got != f["out"]) <= 1e-3
+    assert np.max(np.abs(got.astype(np.int32) - f["out"].astype(np.int32))) <= 1
