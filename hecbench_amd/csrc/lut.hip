@@ -5,9 +5,11 @@
 //
 //   y[n] = sum_k x[k] * ( q_bias[k/G][n] + sum_b alpha[k/G][b][n] * s(k,b,n) )
 //
-// For every 8-element sub-vector of x the 256 signed sums sum_j (+-x[j]) are
-// tabulated once per workgroup in LDS (fp32 entries), and each byte of a packed
-// bit-plane word becomes one table lookup.  A workgroup owns a tile of columns
+// Two kernels.  Shapes with group size % 128 == 0 and N % 64 == 0 run on the matrix cores
+// (bcq_mfma_kernel below: the packed bits themselves are the fp8 operands, no tables).
+// Every other shape runs the table kernel: for every 8-element sub-vector of x the 256
+// signed sums sum_j (+-x[j]) are tabulated once per workgroup in LDS (fp32 entries), and
+// each byte of a packed bit-plane word becomes one table lookup.  A workgroup owns a tile of columns
 // and a K slice of up to 512*iterations elements: per iteration it tabulates 64
 // sub-vectors (64 KB), wave w consumes the 128-element quarter w for all the
 // tile's columns, and the four waves' partial sums meet in LDS at the end.
@@ -186,31 +188,38 @@ __global__ __launch_bounds__(256) void lut_gemv_kernel(LutArgs a) {
 // ======================================================================================
 // Matrix-core path (group size a multiple of 128, N a multiple of 64).
 //
-// sum_k s*x = 2*sum_k bit*x - sum_k x.  A single bit left in place at bit p (p <= 9) of
-// an otherwise zero 16-bit half is the subnormal fp16 number 2^(p-24), so sixteen ANDs
-// (and one shift) turn a packed 32-bit word into the sixteen operand registers of four
-// 16x16x32 fp16 MFMAs; the factor 2^p is folded into the activation of that slot.  No
-// table, no LDS lookup, no bank conflicts.  Lane quarter kb streams k-word 4*quad + kb,
-// so one MFMA chain sums a whole 128-element quad of one bit plane for 64 columns (four
-// adjacent columns per lane, one 128-bit load per plane and quad); alpha is applied to the
-// chain's result in fp32.  Every B column holds the same activations, so the result is
-// replicated across the 16 lanes of a row group and each lane applies alpha to its own
-// four columns.
-typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+// sum_k s*x = 2*(sum_k bit*x - (sum_k x)/2).  An fp8 (e4m3) byte whose exponent field is
+// zero is the subnormal mantissa*2^-9, so a single weight bit left in place at bit p
+// (p <= 2) of an otherwise zero byte IS the fp8 number 2^(p-9): eight ANDs and two shifts
+// turn a packed 32-bit word into the eight operand registers (32 fp8 values) of one
+// 16x16x128 fp8 MFMA; the factor 2^p is folded into the activation of that slot.  No table,
+// no LDS lookup, no bank conflicts.  The activations of a round (256 of them per wave) are
+// scaled to 16-bit fixed point and split into four signed 4-bit digits carried by MFMA
+// columns 0..3, so every product is an integer and the matrix-core sums are exact.  Lane
+// quarter kb streams k-word 4*quad + kb, so one MFMA sums a whole 128-element quad of one
+// bit plane for 16 columns (four adjacent columns per lane and 128-bit load); alpha is
+// applied to that sum in fp32, per digit, and the digits are combined once at the end.
 typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
 
-// register r of a word: (bit in the low half, bit in the high half); both sit at
-// position p = r (r < 10) of their half, or r - 10 after a shift by 10 (r >= 10)
-__device__ __forceinline__ void unpack_bits(uint32_t w, uint32_t (&a)[16]) {
-  const uint32_t w10 = w >> 10;
+// operand register r of a word holds bit r of each of its four bytes, at mantissa bit p(r)
+__device__ __forceinline__ constexpr int bit_pos(int r) { return r < 6 ? r % 3 : r - 6; }
+__device__ __forceinline__ constexpr uint32_t bit_mask(int r) { return 0x01010101u << bit_pos(r); }
+
+__device__ __forceinline__ v8i unpack_bits_fp8(uint32_t w) {
+  const uint32_t w3 = w >> 3, w6 = w >> 6;
+  v8i a;
 #pragma unroll
-  for (int r = 0; r < 10; ++r) a[r] = w & (0x00010001u << r);
-#pragma unroll
-  for (int r = 10; r < 16; ++r) a[r] = w10 & (0x00010001u << (r - 10));
+  for (int r = 0; r < 8; ++r) a[r] = (int)((r < 3 ? w : (r < 6 ? w3 : w6)) & bit_mask(r));
+  return a;
 }
 
+__device__ __forceinline__ f4 mfma_fp8(v8i a, v8i b, f4 c) {
+  // fp8 x fp8, both block scales 2^0 (E8M0 code 127)
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+}
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v) {
@@ -219,13 +228,13 @@ __device__ __forceinline__ float dpp_f(float v) {
 __device__ __forceinline__ float lane_f(float v, int l) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
 }
-// Sum over the 64 lanes: four DPP butterfly steps per 16-lane row, then the row sums.
-__device__ __forceinline__ float wave_sum(float v) {
-  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
-  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
-  v += dpp_f<0x141>(v);  // row_half_mirror
-  v += dpp_f<0x140>(v);  // row_mirror
-  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
+// Maximum over the 64 lanes: four DPP butterfly steps per 16-lane row, then the row results.
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = fmaxf(v, dpp_f<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = fmaxf(v, dpp_f<0x141>(v));  // row_half_mirror
+  v = fmaxf(v, dpp_f<0x140>(v));  // row_mirror
+  return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
 }
 
 struct Half16 {  // sixteen fp16 values as two 128-bit loads
@@ -243,13 +252,12 @@ __device__ __forceinline__ Half16 load_half16(const _Float16* p) {
   return h;
 }
 
-// NB bit planes, QUADS 128-element quads per wave per round.
+// NB bit planes, QUADS 128-element quads per wave per round, WAVES waves per workgroup.
 template <int NB, int QUADS, int WAVES, bool BIAS>
 __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
-  constexpr int kMfmaWaves = WAVES;
   extern __shared__ float lds[];
-  u4v* xs = reinterpret_cast<u4v*>(lds);                 // [waves][QUADS][4 kb][4 j]
-  float* red = lds + kMfmaWaves * QUADS * 16 * 4;        // [waves][64]
+  uint32_t* xs = reinterpret_cast<uint32_t*>(lds);  // [waves][QUADS][4 kb][4 digits][8 regs] dwords
+  float* red = lds + WAVES * QUADS * 128;           // [waves][4 digits][64]
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int c = lane & 15, kb = lane >> 4;
   const int tile = blockIdx.x;
@@ -257,28 +265,33 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
   const size_t n0 = (size_t)tile * 64;
   const uint32_t col_off = 4u * c;   // first of the lane's 4 columns (N % 64 == 0: no partial tiles)
   const uint32_t acol = 16u * kb;    // first of the 16 columns this lane applies alpha to
-  // register c of a word holds bit c (low half) and bit c + 16 (high half), both at
-  // position p of their half
-  const int p = c < 10 ? c : c - 10;
-  const float slot_scale = __uint_as_float((uint32_t)(127 - p) << 23);  // 2^-p
-  u4v* xs_w = xs + wv * (QUADS * 16);
+  // staging role of lane (c, kb): elements k_lo = (c&7) + 16*(c>>3) and k_lo + 8 of k-word kb,
+  // i.e. operand register r = c&7, bytes 2*(c>>3) and 2*(c>>3)+1
+  const int r_slot = c & 7, k_lo = r_slot + 16 * (c >> 3);
+  const float slot_scale = __uint_as_float((uint32_t)(127 + 2 - bit_pos(r_slot)) << 23);  // 2^(2-p)
+  uint32_t* xs_w = xs + wv * (QUADS * 128);
+  const int digit = c & 3;  // MFMA column -> digit (columns 4..15 repeat them and are never read)
 
-  float run[4][4];
+  v8i ones;  // every slot's bit set: one MFMA with it sums the digits of a quad
+#pragma unroll
+  for (int r = 0; r < 8; ++r) ones[r] = (int)bit_mask(r);
+
+  float tot[4][4];
 #pragma unroll
   for (int q = 0; q < 4; ++q)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) run[q][i] = 0.f;
+    for (int i = 0; i < 4; ++i) tot[q][i] = 0.f;
 
-  for (int q0 = wv * QUADS; q0 < nquads; q0 += kMfmaWaves * QUADS) {
+  for (int q0 = wv * QUADS; q0 < nquads; q0 += WAVES * QUADS) {
     // ---- loads of this round (unconditional, clamped): activations, then packed words -------
     float xlo[QUADS], xhi[QUADS];
     u4v wq[QUADS][NB];
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
       const int quad = min(q0 + t, nquads - 1);
-      const _Float16* xp = a.x + (size_t)quad * 128 + 32 * kb;
-      xlo[t] = (float)xp[c];
-      xhi[t] = (float)xp[c + 16];
+      const _Float16* xp = a.x + (size_t)quad * 128 + 32 * kb + k_lo;
+      xlo[t] = (float)xp[0];
+      xhi[t] = (float)xp[8];
     }
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
@@ -288,19 +301,48 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
       for (int b = 0; b < NB; ++b)
         wq[t][b] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wp + (size_t)b * a.N));
     }
-    // ---- stage the activations in operand-slot order (wave-local) ---------------------------
-    float xsum[QUADS];
+    // ---- scale to 16-bit fixed point, split into four signed 4-bit digits, stage (wave-local)
+    float amax = 0.f;
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
       if (q0 + t >= nquads) { xlo[t] = 0.f; xhi[t] = 0.f; }
-      const h2v pair = {(_Float16)(xlo[t] * slot_scale), (_Float16)(xhi[t] * slot_scale)};
-      reinterpret_cast<uint32_t*>(xs_w + (t * 4 + kb) * 4 + (c >> 2))[c & 3] = __builtin_bit_cast(uint32_t, pair);
-      xsum[t] = wave_sum(xlo[t] + xhi[t]);  // sum of the quad's 128 activations
+      amax = fmaxf(amax, fmaxf(fabsf(xlo[t]), fabsf(xhi[t])));
+    }
+    const float xmax = wave_max(amax);
+    // 2^E * max|x| lies in [2^14, 2^15)
+    int E = 14 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
+    E = xmax > 0.f ? max(-120, min(120, E)) : 0;
+    const float scaleE = __uint_as_float((uint32_t)(E + 127) << 23);
+#pragma unroll
+    for (int t = 0; t < QUADS; ++t) {
+      float d[2][4];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const float X = rintf((e ? xhi[t] : xlo[t]) * scaleE);
+        d[e][0] = rintf(X * (1.f / 4096.f));
+        const float r1 = X - d[e][0] * 4096.f;
+        d[e][1] = rintf(r1 * (1.f / 256.f));
+        const float r2 = r1 - d[e][1] * 256.f;
+        d[e][2] = rintf(r2 * (1.f / 16.f));
+        d[e][3] = r2 - d[e][2] * 16.f;
+      }
+      uint16_t* dst = reinterpret_cast<uint16_t*>(xs_w + ((t * 4 + kb) * 4) * 8 + r_slot) + (c >> 3);
+#pragma unroll
+      for (int dg = 0; dg < 4; ++dg) {
+        // digit * 2^(2-p) is exact in fp8 (|digit| <= 8)
+        const int pk = __builtin_amdgcn_cvt_pk_fp8_f32(d[0][dg] * slot_scale, d[1][dg] * slot_scale, 0, false);
+        dst[dg * 16] = (uint16_t)pk;  // next digit: 8 registers = 16 halves further
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    // ---- MFMA chains --------------------------------------------------------------------------
+    // ---- MFMAs ------------------------------------------------------------------------------------
+    float run[4][4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) run[q][i] = 0.f;
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
       if (q0 + t >= nquads) break;  // wave-uniform
@@ -309,72 +351,73 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
       Half16 al[NB];
 #pragma unroll
       for (int b = 0; b < NB; ++b) al[b] = load_half16(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
-      h8 B[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) B[j] = __builtin_bit_cast(h8, xs_w[(t * 4 + kb) * 4 + j]);
-      const float half_x = xsum[t] * -2.98023223876953125e-8f;  // -(sum x)/2 in operand units (2^-24)
+      const u4v* bp = reinterpret_cast<const u4v*>(xs_w + ((t * 4 + kb) * 4 + digit) * 8);
+      const u4v b0 = bp[0], b1 = bp[1];
+      const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+      // digit sum of the quad (in operand units 2^-7), identical in all four result rows
+      const f4 dsum = mfma_fp8(ones, B, f4{0.f, 0.f, 0.f, 0.f});
+      const f4 init = {-0.5f * dsum[0], -0.5f * dsum[1], -0.5f * dsum[2], -0.5f * dsum[3]};
       if (BIAS) {
         const Half16 bi = load_half16(a.qbias + (size_t)g * a.N + n0 + acol);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) run[q][i] = fmaf(bi.get(4 * i + q), -half_x, run[q][i]);
+          for (int q = 0; q < 4; ++q) run[q][i] = fmaf(bi.get(4 * i + q), 0.5f * dsum[i], run[q][i]);
       }
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
         const uint32_t words[4] = {wq[t][b].x, wq[t][b].y, wq[t][b].z, wq[t][b].w};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          uint32_t f[16];
-          unpack_bits(words[q], f);
-          f4 acc = {half_x, half_x, half_x, half_x};  // chain result = sum bit*x - (sum x)/2
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const u4v av = {f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]};
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), B[j], acc, 0, 0, 0);
-          }
+          // one MFMA = this digit's sum over the quad of bit*x, minus half the digit sum
+          const f4 acc = mfma_fp8(unpack_bits_fp8(words[q]), B, init);
           // rows 4*kb + i of the tile's 16-column block q: column 16*kb + 4*i + q
 #pragma unroll
           for (int i = 0; i < 4; ++i) run[q][i] = fmaf(al[b].get(4 * i + q), acc[i], run[q][i]);
         }
       }
     }
-  }
-  // ---- combine the waves -------------------------------------------------------------------------
-  if (c == 0) {
+    const float descale = __uint_as_float((uint32_t)(127 - E) << 23);
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) red[wv * 64 + 16 * kb + 4 * i + q] = run[q][i];
+      for (int i = 0; i < 4; ++i) tot[q][i] = fmaf(run[q][i], descale, tot[q][i]);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+  }
+  // ---- combine digits and waves -------------------------------------------------------------------
+  if (c < 4) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[(wv * 4 + c) * 64 + 16 * kb + 4 * i + q] = tot[q][i];
   }
   __syncthreads();
   const int n = tile * 64 + tid;
   if (tid < 64 && n < a.N) {
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < kMfmaWaves; ++w) v += red[w * 64 + tid];
-    // operand scale 2^-24, and the chains hold half of sum s*x
-    a.y[n] = (_Float16)(v * 33554432.f);
+    for (int w = 0; w < WAVES; ++w) {
+      const float* rw = red + (w * 4) * 64 + tid;
+      v += ((rw[0] * 16.f + rw[64]) * 16.f + rw[128]) * 16.f + rw[192];
+    }
+    // operand units 2^-7, and the sums hold half of sum s*x
+    a.y[n] = (_Float16)(v * 256.f);
   }
 }
 
-template <int NB, int QUADS, int WAVES>
-int launch_bcq_mfma_w(const LutArgs& a, hipStream_t stream) {
-  const size_t smem = (size_t)WAVES * QUADS * 16 * 16 + (size_t)WAVES * 64 * 4;
+// Eight waves per workgroup (two per SIMD, up to 256 VGPRs each): sixteen-wave variants
+// spill and measured slower.
+template <int NB, int QUADS>
+int launch_bcq_mfma(const LutArgs& a, hipStream_t stream) {
+  constexpr int WAVES = 8;
+  const size_t smem = (size_t)WAVES * QUADS * 512 + (size_t)WAVES * 4 * 64 * 4;
   const int ntiles = a.N / 64;
   if (a.qbias)
     hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, true>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
   else
     hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, false>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
   return hq_launch_status();
-}
-// Waves per workgroup: 16 when K offers at least 16*QUADS quads (four waves per SIMD hide
-// the matrix-core latency of the dependent chains), otherwise 8.
-template <int NB, int QUADS>
-int launch_bcq_mfma(const LutArgs& a, hipStream_t stream) {
-  const int want = hq_env_int("HQ_LUT_WAVES", 0);
-  if (want == 8 || (want != 16 && (a.K >> 7) < 16 * QUADS)) return launch_bcq_mfma_w<NB, QUADS, 8>(a, stream);
-  return launch_bcq_mfma_w<NB, QUADS, 16>(a, stream);
 }
 
 }  // namespace
@@ -398,13 +441,13 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
     a.bW = bW; a.alpha = (const _Float16*)alpha; a.qbias = (const _Float16*)q_bias;
     a.x = (const _Float16*)x; a.y = (_Float16*)y; a.partial = nullptr; a.counters = nullptr;
     a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = K; a.nsplit = 1;
-    switch (nbits) {
+    switch (nbits) {  // quads per wave per round, bounded by the register budget
       case 1: return launch_bcq_mfma<1, 2>(a, stream);
       case 2: return launch_bcq_mfma<2, 2>(a, stream);
       case 3: return launch_bcq_mfma<3, 2>(a, stream);
       case 4: return launch_bcq_mfma<4, 2>(a, stream);
-      case 5: return launch_bcq_mfma<5, 1>(a, stream);
-      case 6: return launch_bcq_mfma<6, 1>(a, stream);
+      case 5: return launch_bcq_mfma<5, 2>(a, stream);
+      case 6: return launch_bcq_mfma<6, 2>(a, stream);
       case 7: return launch_bcq_mfma<7, 1>(a, stream);
       default: return launch_bcq_mfma<8, 1>(a, stream);
     }
