@@ -11,12 +11,12 @@ from .ops import (
     NF4, FP4,
     vecquant3matmul, vecquant3matmul_faster, q3_matvec, q3_gemm,
     dequant_4bit, quantize_dynamic8, lut_matmul, code1x16_matvec,
-    device_info, init,
+    device_info, init, q3_pack, bcq_pack, quantize_4bit,
 )
 
 __all__ = [
     "HqError", "EXPORTED_SYMBOLS", "LIB_PATH", "NF4", "FP4",
     "vecquant3matmul", "vecquant3matmul_faster", "q3_matvec", "q3_gemm",
     "dequant_4bit", "quantize_dynamic8", "lut_matmul", "code1x16_matvec",
-    "device_info", "init",
+    "device_info", "init", "q3_pack", "bcq_pack", "quantize_4bit",
 ]

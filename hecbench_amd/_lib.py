@@ -27,6 +27,10 @@ _SIGNATURES = {
                                _c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_void_p]),
     "hq_aqlm_matvec": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
                                   _c.c_int, _c.c_int, _c.POINTER(_c.c_int), _c.c_int, _c.c_void_p]),
+    "hq_q3_pack": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p]),
+    "hq_bcq_pack": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int, _c.c_int, _c.c_void_p]),
+    "hq_quantize_4bit": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int,
+                                    _c.c_int, _c.c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

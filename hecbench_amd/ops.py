@@ -128,3 +128,35 @@ def code1x16_matvec(codes, x, codebooks, codebook_a_sizes, codebook_stride_int4,
                                     codebook_stride_int4, _stream())
     _lib.check(rc, "hq_aqlm_matvec")
     return out
+
+
+def q3_pack(codes):
+    """codes uint8 [K][N] (0..7) -> qweight int32 [3K/32][N]."""
+    _dev(codes)
+    K, N = codes.shape
+    out = torch.empty((3 * K // 32, N), dtype=torch.int32, device=codes.device)
+    _lib.check(_lib.load().hq_q3_pack(_ptr(codes), _ptr(out), K, N, _stream()), "hq_q3_pack")
+    return out
+
+
+def bcq_pack(signs):
+    """signs int8 [K][nb][N] (> 0 means +1) -> bW int32 [K/32][nb][N]."""
+    _dev(signs)
+    K, nb, N = signs.shape
+    out = torch.empty((K // 32, nb, N), dtype=torch.int32, device=signs.device)
+    _lib.check(_lib.load().hq_bcq_pack(_ptr(signs), _ptr(out), K, N, nb, _stream()), "hq_bcq_pack")
+    return out
+
+
+def quantize_4bit(x, blocksize, table=NF4):
+    """x fp32/fp16 [n] -> (packed uint8 [ceil(n/2)], absmax fp32 [ceil(n/blocksize)])."""
+    _dev(x)
+    n = x.numel()
+    if x.dtype not in (torch.float16, torch.float32):
+        raise ValueError("x must be fp32 or fp16")
+    packed = torch.empty((n + 1) // 2, dtype=torch.uint8, device=x.device)
+    absmax = torch.empty((n + blocksize - 1) // blocksize, dtype=torch.float32, device=x.device)
+    rc = _lib.load().hq_quantize_4bit(_ptr(x), _F16 if x.dtype == torch.float16 else _F32, _ptr(packed), _ptr(absmax),
+                                      n, blocksize, table, _stream())
+    _lib.check(rc, "hq_quantize_4bit")
+    return packed, absmax

@@ -15,10 +15,10 @@
  *   - return value: 0 on success, a negative HQ_ERR_* code for a rejected
  *     argument (nothing is launched), or a positive hipError_t value;
  *   - nothing is printed; hq_strerror() turns a code into text;
- *   - the library keeps one small per-device workspace (split-K partial sums
- *     and arrival counters, allocated by hq_init() or by the first call on a
- *     device); calls that share a device must not overlap in time on different
- *     streams unless stated otherwise below.
+ *   - the library keeps one small workspace per (device, stream) pair (split-K
+ *     partial sums, arrival counters, re-ordered GEMM activations), allocated by
+ *     hq_init() or by the first call that needs it; calls on different streams
+ *     use different workspaces and may overlap.
  */
 #ifndef HQ_H
 #define HQ_H
@@ -135,6 +135,24 @@ int hq_lut_gemv(const uint32_t* bW, const void* alpha_fp16, const void* q_bias_f
 int hq_aqlm_matvec(const int16_t* codes, const void* codebooks_fp16, const void* scales_fp16,
                    const void* x_fp16, void* y_fp16, int M, int K,
                    const int codebook_a_sizes[4], int codebook_stride_int4, void* stream);
+
+/*
+ * Device-side packers and the 4-bit blockwise quantiser (inverses of the unpack /
+ * dequantise steps above, so the family round-trips on the GPU).
+ *
+ * hq_q3_pack: codes uint8[K][N] (values 0..7) -> qweight int32[3K/32][N] in the layout of
+ *   hq_q3_matvec; the host loop it replaces is the weight initialisation of
+ *   src/quant3MatMul-hip/main.cu:35-43 (generalised from the all-ones pattern).
+ * hq_bcq_pack: signs int8[K][nbits][N] (> 0 means +1) -> bW uint32[K/32][nbits][N];
+ *   replaces the packing loop of makeRandomWeight, src/lut-gemm-hip/main.cu:118-134.
+ * hq_quantize_4bit: x fp32/fp16 [n] -> packed nibbles (high nibble first) and one fp32
+ *   absmax per block; code = nearest table entry of x/absmax (NF4: a value exactly on the
+ *   midpoint of two entries takes the lower code).  No counterpart in the HeCBench tree.
+ */
+int hq_q3_pack(const uint8_t* codes, int32_t* qweight, int K, int N, void* stream);
+int hq_bcq_pack(const int8_t* signs, uint32_t* bW, int K, int N, int nbits, void* stream);
+int hq_quantize_4bit(const void* x, int x_dtype, uint8_t* packed, float* absmax, int64_t n_elems,
+                     int blocksize, int table, void* stream);
 
 #ifdef __cplusplus
 }

@@ -282,6 +282,44 @@ void hqo_dequant_4bit(const uint8_t* packed, const float* absmax, uint16_t* out,
   }
 }
 
+/* Blockwise 4-bit quantisation, PARITY UNPINNED (no counterpart in the reference):
+ * absmax = max|x| over the block, v = x * (1/absmax) in fp32, NF4 code = number of fp32
+ * midpoints (t[c]+t[c+1])*0.5 strictly below v; FP4 code = nearest magnitude (ties to the
+ * smaller), sign in bit 3.  x_is_f16: x holds binary16 bit patterns. */
+void hqo_quantize_4bit(const void* x, int x_is_f16, uint8_t* packed, float* absmax, int64_t n,
+                       int blocksize, int table) {
+  static const float mags[8] = {0.0f, 0.005208333333f, 0.16666667f, 0.25f, 0.33333333f, 0.5f, 0.66666667f, 1.0f};
+  static const unsigned code_of[8] = {0, 1, 6, 7, 4, 5, 2, 3};
+  int64_t nblocks = (n + blocksize - 1) / blocksize;
+  for (int64_t e = 0; e < (n + 1) / 2; ++e) packed[e] = 0;
+  for (int64_t b = 0; b < nblocks; ++b) {
+    int64_t e0 = b * blocksize, e1 = e0 + blocksize < n ? e0 + blocksize : n;
+    float amax = 0.f;
+    for (int64_t e = e0; e < e1; ++e) {
+      float v = x_is_f16 ? hqo_f16_to_f32(((const uint16_t*)x)[e]) : ((const float*)x)[e];
+      v = fabsf(v);
+      if (v > amax) amax = v;
+    }
+    absmax[b] = amax;
+    float inv = amax > 0.f ? 1.0f / amax : 0.f;
+    for (int64_t e = e0; e < e1; ++e) {
+      float v = (x_is_f16 ? hqo_f16_to_f32(((const uint16_t*)x)[e]) : ((const float*)x)[e]) * inv;
+      unsigned c = 0;
+      if (table == 0) {
+        for (int i = 0; i < 15; ++i)
+          if (v > (hqo_nf4_table[i] + hqo_nf4_table[i + 1]) * 0.5f) c = (unsigned)i + 1;
+      } else {
+        float a = fabsf(v);
+        unsigned idx = 0;
+        for (int i = 0; i < 7; ++i)
+          if (a > (mags[i] + mags[i + 1]) * 0.5f) idx = (unsigned)i + 1;
+        c = code_of[idx] | (v < 0.f ? 8u : 0u);
+      }
+      packed[e >> 1] |= (uint8_t)((e & 1) ? c : c << 4);
+    }
+  }
+}
+
 /* ------------------------------------------------ dynamic 8-bit quantize */
 
 uint8_t hqo_dquantize(const float* code, float x) {

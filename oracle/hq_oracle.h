@@ -87,6 +87,10 @@ void hqo_dequant_4bit(const uint8_t* packed, const float* absmax,
                       uint16_t* out_f16, int64_t n_elems, int blocksize,
                       int table /*0=NF4, 1=FP4*/);
 
+/* Inverse of hqo_dequant_4bit (PARITY UNPINNED): blockwise absmax, nearest table code. */
+void hqo_quantize_4bit(const void* x, int x_is_f16, uint8_t* packed, float* absmax, int64_t n,
+                       int blocksize, int table);
+
 /* ---- bitsandbytes dynamic 8-bit quantize (quantBnB) -------------------- */
 /* src/quantBnB-hip/main.cu:13-66 with STOCHASTIC=0. */
 uint8_t hqo_dquantize(const float* code256, float x);

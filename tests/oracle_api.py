@@ -92,6 +92,15 @@ class Oracle:
         self.lib.hqo_dequant_4bit(_p(packed), _p(absmax), _p(out), ctypes.c_int64(n), blocksize, table)
         return out.view(np.float16)
 
+    def quantize_4bit(self, x, blocksize, table=0):
+        n = x.size
+        is16 = x.dtype == np.float16
+        xb = np.ascontiguousarray(x).view(np.uint16) if is16 else np.ascontiguousarray(x, np.float32)
+        packed = np.zeros((n + 1) // 2, np.uint8)
+        absmax = np.zeros((n + blocksize - 1) // blocksize, np.float32)
+        self.lib.hqo_quantize_4bit(_p(xb), int(is16), _p(packed), _p(absmax), ctypes.c_int64(n), blocksize, table)
+        return packed, absmax
+
     # ---- dynamic 8-bit
     def dynamic_map(self):
         code = np.zeros(256, np.float32)

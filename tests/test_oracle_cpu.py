@@ -162,6 +162,29 @@ def test_dequant_4bit_properties(o):
     assert np.array_equal(o.fp4_table[8:], -o.fp4_table[:8])
 
 
+def test_quantize_4bit_is_nearest_code_and_round_trips(o):
+    rng = np.random.default_rng(12)
+    n, bs = 4096, 64
+    x = rng.standard_normal(n).astype(np.float32)
+    for table, tab in ((0, o.nf4_table), (1, o.fp4_table)):
+        packed, absmax = o.quantize_4bit(x, bs, table)
+        assert np.array_equal(absmax, np.abs(x).reshape(-1, bs).max(1))
+        codes = np.stack([packed >> 4, packed & 15], 1).reshape(-1)
+        v = x / np.repeat(absmax, bs)
+        d = np.abs(v[:, None].astype(np.float64) - tab[None, :].astype(np.float64))
+        assert np.all(d[np.arange(n), codes] <= d.min(1) + 1e-6)   # brute-force nearest entry
+        # dequantising the codes gives the nearest representable value, the block maximum exactly
+        deq = o.dequant_4bit(packed, absmax, n, bs, table).astype(np.float32)
+        assert np.max(np.abs(deq - x) / np.repeat(absmax, bs)) <= (0.17 if table == 0 else 0.17)
+        big = np.abs(x) == np.repeat(absmax, bs)
+        assert np.allclose(np.abs(deq[big]), absmax.astype(np.float16).astype(np.float32), rtol=0, atol=0)
+    # idempotence: quantising the dequantised values reproduces the codes
+    packed, absmax = o.quantize_4bit(x, bs, 0)
+    deq32 = (o.nf4_table[np.stack([packed >> 4, packed & 15], 1).reshape(-1)] * np.repeat(absmax, bs)).astype(np.float32)
+    p2, a2 = o.quantize_4bit(deq32, bs, 0)
+    assert np.array_equal(p2, packed) and np.array_equal(a2, absmax)
+
+
 # ------------------------------------------------------------------ dynamic 8-bit
 
 def test_dquantize_against_reference_host_function(o):
