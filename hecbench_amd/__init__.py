@@ -12,6 +12,7 @@ from .ops import (
     vecquant3matmul, vecquant3matmul_faster, q3_matvec, q3_gemm,
     dequant_4bit, quantize_dynamic8, lut_matmul, code1x16_matvec,
     device_info, init, q3_pack, bcq_pack, quantize_4bit,
+    static_scaled_int8_quant, dynamic_scaled_int8_quant,
 )
 
 __all__ = [
@@ -19,4 +20,5 @@ __all__ = [
     "vecquant3matmul", "vecquant3matmul_faster", "q3_matvec", "q3_gemm",
     "dequant_4bit", "quantize_dynamic8", "lut_matmul", "code1x16_matvec",
     "device_info", "init", "q3_pack", "bcq_pack", "quantize_4bit",
+    "static_scaled_int8_quant", "dynamic_scaled_int8_quant",
 ]

@@ -31,6 +31,10 @@ _SIGNATURES = {
     "hq_bcq_pack": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int, _c.c_int, _c.c_void_p]),
     "hq_quantize_4bit": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int,
                                     _c.c_int, _c.c_void_p]),
+    "hq_int8_quant_static": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_float,
+                                        _c.c_int, _c.c_int32, _c.c_void_p]),
+    "hq_int8_quant_dynamic": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64,
+                                         _c.c_int, _c.c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

@@ -160,3 +160,39 @@ def quantize_4bit(x, blocksize, table=NF4):
                                       n, blocksize, table, _stream())
     _lib.check(rc, "hq_quantize_4bit")
     return packed, absmax
+
+
+def _act_dtype(x):
+    if x.dtype == torch.float32:
+        return 0
+    if x.dtype == torch.float16:
+        return 1
+    if x.dtype == torch.bfloat16:
+        return 2
+    raise ValueError("activations must be fp32, fp16 or bf16")
+
+
+def static_scaled_int8_quant(x, scale, azp=None, out=None):
+    """static_scaled_int8_quant of src/quantVLLM-hip/main.cu:133-148; x [tokens][hidden]."""
+    _dev(x, out)
+    tokens, hidden = x.shape
+    if out is None:
+        out = torch.empty((tokens, hidden), dtype=torch.int8, device=x.device)
+    rc = _lib.load().hq_int8_quant_static(_ptr(x), _act_dtype(x), _ptr(out), tokens, hidden, float(scale),
+                                          0 if azp is None else 1, 0 if azp is None else int(azp), _stream())
+    _lib.check(rc, "hq_int8_quant_static")
+    return out
+
+
+def dynamic_scaled_int8_quant(x, with_azp=False, out=None):
+    """dynamic_scaled_int8_quant of src/quantVLLM-hip/main.cu:150-168; returns (out, scales, azp or None)."""
+    _dev(x, out)
+    tokens, hidden = x.shape
+    if out is None:
+        out = torch.empty((tokens, hidden), dtype=torch.int8, device=x.device)
+    scales = torch.empty(tokens, dtype=torch.float32, device=x.device)
+    azp = torch.empty(tokens, dtype=torch.int32, device=x.device) if with_azp else None
+    rc = _lib.load().hq_int8_quant_dynamic(_ptr(x), _act_dtype(x), _ptr(out), _ptr(scales), _ptr(azp), tokens, hidden,
+                                           _stream())
+    _lib.check(rc, "hq_int8_quant_dynamic")
+    return out, scales, azp

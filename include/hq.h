@@ -41,6 +41,7 @@ extern "C" {
 /* element types of the activation vector / matrix */
 #define HQ_DTYPE_F32 0
 #define HQ_DTYPE_F16 1
+#define HQ_DTYPE_BF16 2 /* accepted by the activation quantisers only */
 
 /* flags */
 #define HQ_FLAG_ACCUMULATE 1u /* y += result (reference wrapper semantics) */
@@ -153,6 +154,23 @@ int hq_q3_pack(const uint8_t* codes, int32_t* qweight, int K, int N, void* strea
 int hq_bcq_pack(const int8_t* signs, uint32_t* bW, int K, int N, int nbits, void* stream);
 int hq_quantize_4bit(const void* x, int x_dtype, uint8_t* packed, float* absmax, int64_t n_elems,
                      int blocksize, int table, void* stream);
+
+/*
+ * Per-token int8 activation quantisation, the step in front of a W8A8 matmul.
+ * x is [num_tokens][hidden_size] row-major in fp32, fp16 or bf16; out int8 of the same shape.
+ *   static : out = sat8(rne(x / scale))                       (has_azp == 0)
+ *            out = sat8(sat32(rne(x / scale)) + azp)          (has_azp != 0)
+ *   dynamic: azp == NULL: scales[t] = max|x_t| / 127, out = sat8(rne(x * (127 / max|x_t|)))
+ *            azp != NULL: scales[t] = (max_t - min_t) / 255, azp[t] = rne(-128 - min_t / scales[t]),
+ *                         out = sat8(sat32(rne(x / scales[t])) + azp[t])
+ * All arithmetic is fp32 IEEE (true division, round to nearest even): bit-exact with the
+ * reference host loops (src/quantVLLM-cuda/reference.h:1-93).  Replaces
+ * static_scaled_int8_quant / dynamic_scaled_int8_quant, src/quantVLLM-hip/main.cu:133-168.
+ */
+int hq_int8_quant_static(const void* x, int x_dtype, int8_t* out, int64_t num_tokens, int hidden_size,
+                         float scale, int has_azp, int32_t azp, void* stream);
+int hq_int8_quant_dynamic(const void* x, int x_dtype, int8_t* out, float* scales, int32_t* azp,
+                          int64_t num_tokens, int hidden_size, void* stream);
 
 #ifdef __cplusplus
 }

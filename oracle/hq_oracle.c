@@ -381,6 +381,70 @@ void hqo_dynamic_map(float* code) {
   qsort(code, 256, sizeof(float), cmp_float);
 }
 
+/* ------------------------------------------------ int8 activation quantisation */
+
+static float act_to_f32(const void* x, int dtype, int64_t i) {
+  if (dtype == 0) return ((const float*)x)[i];
+  if (dtype == 1) return hqo_f16_to_f32(((const uint16_t*)x)[i]);
+  uint32_t b = (uint32_t)((const uint16_t*)x)[i] << 16; /* bf16: upper half of an fp32 */
+  float f;
+  memcpy(&f, &b, 4);
+  return f;
+}
+/* src/quantVLLM-cuda/utils.h:9-61 */
+static int8_t f_to_i8_rn(float x) {
+  float d = nearbyintf(x);
+  d = d < -128.f ? -128.f : (127.f < d ? 127.f : d);
+  return (int8_t)d;
+}
+static int32_t f_to_i32_rn(float x) {
+  float d = nearbyintf(x);
+  if (d >= 2147483648.f) return INT32_MAX;
+  if (d <= -2147483648.f) return INT32_MIN;
+  return (int32_t)d;
+}
+static int8_t i32_to_i8(int32_t x) { return (int8_t)(x < -128 ? -128 : (127 < x ? 127 : x)); }
+
+/* src/quantVLLM-cuda/reference.h:1-31 */
+void hqo_int8_quant_static(const void* x, int dtype, int8_t* out, int64_t tokens, int hidden,
+                           float scale, int has_azp, int32_t azp) {
+  for (int64_t i = 0; i < tokens * hidden; ++i) {
+    float v = act_to_f32(x, dtype, i);
+    out[i] = has_azp ? i32_to_i8(f_to_i32_rn(v / scale) + azp) : f_to_i8_rn(v / scale);
+  }
+}
+
+/* src/quantVLLM-cuda/reference.h:33-93 */
+void hqo_int8_quant_dynamic(const void* x, int dtype, int8_t* out, float* scales, int32_t* azp,
+                            int64_t tokens, int hidden) {
+  for (int64_t t = 0; t < tokens; ++t) {
+    if (!azp) {
+      float absmax = 0.f;
+      for (int i = 0; i < hidden; ++i) {
+        float v = act_to_f32(x, dtype, t * hidden + i);
+        v = v > 0.f ? v : -v;
+        absmax = v > absmax ? v : absmax;
+      }
+      scales[t] = absmax / 127.0f;
+      float tmp = 127.0f / absmax;
+      for (int i = 0; i < hidden; ++i) out[t * hidden + i] = f_to_i8_rn(act_to_f32(x, dtype, t * hidden + i) * tmp);
+    } else {
+      float mx = 1.17549435e-38f, mn = 3.40282347e+38f; /* numeric_limits min() / max() */
+      for (int i = 0; i < hidden; ++i) {
+        float v = act_to_f32(x, dtype, t * hidden + i);
+        mx = v > mx ? v : mx;
+        mn = v < mn ? v : mn;
+      }
+      float sc = (mx - mn) / 255.0f;
+      int32_t z = (int32_t)nearbyintf(-128.0f - mn / sc);
+      scales[t] = sc;
+      azp[t] = z;
+      for (int i = 0; i < hidden; ++i)
+        out[t * hidden + i] = i32_to_i8(f_to_i32_rn(act_to_f32(x, dtype, t * hidden + i) / sc) + z);
+    }
+  }
+}
+
 /* -------------------------------------------------------------- LUT-GEMM */
 
 void hqo_bcq_pack(const int8_t* signs, int K, int N, int nb, uint32_t* bW) {

@@ -24,6 +24,9 @@
  *                             reference host loops compiled into oracle/_ref
  *                             (src/lut-gemm-hip/main.cu:118-146)
  *   AQLM                    : PARITY UNPINNED (the reference checks nothing)
+ *   int8 activation quant   : pinned by the reference host loops compiled into
+ *                             oracle/_ref (src/quantVLLM-cuda/reference.h)
+ *   4-bit blockwise quantize: PARITY UNPINNED (no counterpart in the reference)
  */
 #ifndef HQ_ORACLE_H
 #define HQ_ORACLE_H
@@ -98,6 +101,14 @@ void    hqo_quantize_dynamic8(const float* code256, const float* A, uint8_t* out
                               int64_t n);
 /* The signed dynamic map bitsandbytes builds (256 sorted fp32 values). */
 void    hqo_dynamic_map(float* code256);
+
+/* ---- per-token int8 activation quantisation (quantVLLM) ------------------ */
+/* src/quantVLLM-cuda/reference.h:1-93; dtype 0 = fp32, 1 = fp16 bits, 2 = bf16 bits.
+ * Pinned by the reference host loops compiled into oracle/_ref. */
+void hqo_int8_quant_static(const void* x, int dtype, int8_t* out, int64_t tokens, int hidden,
+                           float scale, int has_azp, int32_t azp);
+void hqo_int8_quant_dynamic(const void* x, int dtype, int8_t* out, float* scales,
+                            int32_t* azp /*nullable*/, int64_t tokens, int hidden);
 
 /* ---- LUT-GEMM (BCQ) ----------------------------------------------------- */
 /* bit packing of src/lut-gemm-hip/main.cu:118-134:

@@ -113,6 +113,33 @@ class Oracle:
         self.lib.hqo_quantize_dynamic8(_p(code), _p(A), _p(out), ctypes.c_int64(A.size))
         return out
 
+    # ---- int8 activation quantisation
+    @staticmethod
+    def _act(x):
+        import torch  # bf16 arrays arrive as torch tensors (numpy has no bfloat16)
+        if isinstance(x, torch.Tensor):
+            assert x.dtype == torch.bfloat16
+            return np.ascontiguousarray(x.view(torch.int16).numpy()).view(np.uint16), 2
+        if x.dtype == np.float16:
+            return np.ascontiguousarray(x).view(np.uint16), 1
+        return np.ascontiguousarray(x, np.float32), 0
+
+    def int8_quant_static(self, x, scale, azp=None):
+        xb, dt = self._act(x)
+        out = np.zeros(x.shape, np.int8)
+        self.lib.hqo_int8_quant_static(_p(xb), dt, _p(out), ctypes.c_int64(x.shape[0]), int(x.shape[1]),
+                                       ctypes.c_float(scale), 0 if azp is None else 1, 0 if azp is None else int(azp))
+        return out
+
+    def int8_quant_dynamic(self, x, with_azp=False):
+        xb, dt = self._act(x)
+        out = np.zeros(x.shape, np.int8)
+        scales = np.zeros(x.shape[0], np.float32)
+        azp = np.zeros(x.shape[0], np.int32) if with_azp else None
+        self.lib.hqo_int8_quant_dynamic(_p(xb), dt, _p(out), _p(scales), _p(azp), ctypes.c_int64(x.shape[0]),
+                                        int(x.shape[1]))
+        return out, scales, azp
+
     # ---- LUT-GEMM
     def bcq_pack(self, signs):
         K, nb, N = signs.shape

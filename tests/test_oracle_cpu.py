@@ -338,3 +338,55 @@ def test_golden_dquantize_outputs(o):
     got = o.quantize_dynamic8(o.dynamic_map(), f["A"])
     assert np.mean(got != f["out"]) <= 1e-3
     assert np.max(np.abs(got.astype(np.int32) - f["out"].astype(np.int32))) <= 1
+
+
+# ------------------------------------------------------------------ int8 activation quantisation
+
+def _act_inputs(dtype, tokens, hidden, seed):
+    import torch
+    rng = np.random.default_rng(seed)
+    # the reference fixture (rand() % 1000 - 300) plus fractional values and a few extremes
+    x = np.concatenate([rng.integers(-300, 700, size=(tokens // 2, hidden)).astype(np.float32),
+                        (rng.standard_normal((tokens - tokens // 2, hidden)) * 37.3).astype(np.float32)])
+    if hidden >= 4:
+        x[0, :4] = [0.05, -0.05, 0.15, 12.75]  # ties of x / 0.1
+    if dtype == "bf16":
+        return torch.from_numpy(x).to(torch.bfloat16)
+    return x.astype(np.float16 if dtype == "f16" else np.float32)
+
+
+@pytest.mark.parametrize("dtype,code", [("f32", 0), ("f16", 1), ("bf16", 2)])
+def test_int8_quant_against_reference_host_loops(o, dtype, code):
+    """The four host loops of src/quantVLLM-cuda/reference.h, compiled into oracle/_ref."""
+    ref = oa.load_ref_hip()
+    if ref is None or not hasattr(ref, "ref_int8_quant_static"):
+        pytest.skip("oracle/_ref/libhecref_hip.so not built (reference tree not mounted)")
+    tokens, hidden = 24, 200
+    x = _act_inputs(dtype, tokens, hidden, 3 + code)
+    xb, _ = o._act(x)
+    vp = lambda a: None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+    for azp in (None, 54, -200):
+        want = np.zeros((tokens, hidden), np.int8)
+        ref.ref_int8_quant_static(vp(xb), code, vp(want), ctypes.c_long(tokens), hidden, ctypes.c_float(0.1),
+                                  0 if azp is None else 1, 0 if azp is None else azp)
+        assert np.array_equal(o.int8_quant_static(x, 0.1, azp), want)
+    for with_azp in (False, True):
+        want = np.zeros((tokens, hidden), np.int8)
+        ws = np.zeros(tokens, np.float32)
+        wz = np.zeros(tokens, np.int32) if with_azp else None
+        ref.ref_int8_quant_dynamic(vp(xb), code, vp(want), vp(ws), vp(wz), ctypes.c_long(tokens), hidden)
+        got, gs, gz = o.int8_quant_dynamic(x, with_azp)
+        assert np.array_equal(got, want) and np.array_equal(gs, ws)
+        if with_azp:
+            assert np.array_equal(gz, wz)
+
+
+def test_int8_quant_closed_forms(o):
+    x = np.array([[0.04, 0.05, 0.15, 0.25, -0.05, -0.15, 100.0, -100.0, 12.7, 12.75]], np.float32)
+    q = o.int8_quant_static(x, 0.1)
+    # 0.05/0.1 etc. are not exact in fp32; the saturating ends and clear cases are
+    assert q[0, 0] == 0 and q[0, 6] == 127 and q[0, 7] == -128 and q[0, 8] == 127
+    q, s, _ = o.int8_quant_dynamic(np.array([[1.0, -2.0, 0.5, 2.0]], np.float32))
+    assert s[0] == np.float32(2.0) / np.float32(127.0) and list(q[0]) == [64, -127, 32, 127]
+    q, s, z = o.int8_quant_dynamic(np.array([[0.0, 255.0, 127.5, 51.0]], np.float32), with_azp=True)
+    assert s[0] == 1.0 and z[0] == -128 and list(q[0]) == [-128, 127, 0, -77]
