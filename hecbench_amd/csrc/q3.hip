@@ -7,23 +7,29 @@
 //
 // The kernel is HBM-bound only if a weight costs well under two VALU
 // instructions (17 MB / 8 TB/s leaves ~1.85 lane-ops per weight on 256 CUs), so
-// the integer codes are never converted one by one: each 32-bit window of the
-// packed string is ANDed into two subnormal-fp16 fields (see q3_recipe.h) and the
-// multiply-accumulate runs on the matrix cores as a 16x16x32 fp16 MFMA whose
-// "batch" dimension carries three fixed-point digits (11 bits each, 33 bits below
-// the largest |x|) of the fp32 activation vector.  Products and partial sums are
-// integers in units of one quantum, so the accumulation is exact; the only
-// roundings are the handful of fp32 operations of the epilogue.
+// the integer codes are never converted one by one.  The 96-bit string of a
+// k-group's 32 codes is, read six bits at a time, a string of 16 fp6 (e2m3)
+// numbers whose exponent bits happen to hold the next code: one AND per word
+// keeps the even codes as fp6 subnormals code/8, one funnel shift and AND per
+// word does the same for the odd codes, and the six registers are the A operand
+// of one 16x16x128 f8f6f4 MFMA (nine VALU instructions per 32 weights).  The B
+// operand carries the activations as fixed point: x * 2^E rounded to a 31-bit
+// integer, biased by 0x88888888 and cut into eight nibbles; a nibble 0..15 in an
+// otherwise zero byte is the fp8 (e4m3) number nibble * 2^-9, so no conversion
+// is needed, only a byte transpose.  MFMA column d holds nibble d, column 8 a
+// constant one (it yields sum_k q[k], which takes the bias out again).  Every
+// product and partial sum is a small integer, so the matrix-core accumulation
+// is exact; the roundings are those of the fp32 epilogue.
 //
 // Work split: a workgroup owns a 64-column tile and WAVES*4*STEPS consecutive
-// k-groups; a wave's 16-lane quarter `kb` streams one k-group per step as three
-// uint4 loads (4 adjacent columns x 3 packed rows), i.e. 256 contiguous bytes
-// per packed row per quarter.  A wave issues all its global loads first, stages
-// its own activations in LDS without a workgroup barrier, and meets the other
-// waves only in the final reduction.  When one workgroup covers all of K no
-// cross-workgroup reduction is needed; otherwise (split-K) the partial sums go to
-// a workspace and the last workgroup to arrive at a tile adds them in a fixed
-// order, so results do not depend on arrival order.
+// k-groups per round; a wave's 16-lane quarter `kb` streams one k-group per step
+// as three uint4 loads (4 adjacent columns x 3 packed rows), i.e. 256 contiguous
+// bytes per packed row per quarter.  A wave issues all its global loads first,
+// stages its own activation digits in LDS without a workgroup barrier, and meets
+// the other waves only in the final reduction.  When one workgroup covers all of
+// K no cross-workgroup reduction is needed; otherwise (split-K) the partial sums
+// go to a workspace and the last workgroup to arrive at a tile adds them in a
+// fixed order, so results do not depend on arrival order.
 #include "hq_internal.h"
 #include "q3_recipe.h"
 
@@ -75,27 +81,49 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
 }
 
-// Sixteen two-field registers of one column's k-group.
-__device__ __forceinline__ void unpack16(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t (&a)[16]) {
-  using namespace hq_q3;
-  const uint32_t win[7] = {w0,
-                           __builtin_amdgcn_alignbit(w1, w0, 4),
-                           __builtin_amdgcn_alignbit(w1, w0, 10),
-                           w1,
-                           __builtin_amdgcn_alignbit(w2, w1, 9),
-                           w2,
-                           w2 >> 7};
-#pragma unroll
-  for (int r = 0; r < 16; ++r) a[r] = win[kRecipe[r].window] & mask_of(r);
+// Bits of word `word` of the 96-bit string that belong to the low three bits of a 6-bit field.
+constexpr uint32_t low3_mask(int word) {
+  uint32_t m = 0;
+  for (int b = 0; b < 32; ++b)
+    if ((32 * word + b) % 6 < 3) m |= 1u << b;
+  return m;
+}
+
+// Row-wise broadcast of lane 8 of each 16-lane row (DPP row_newbcast:8).
+__device__ __forceinline__ float row_bcast8(float v) { return dpp_f<0x158>(v); }
+
+// 4x4 byte transpose: in[j] holds four digits of value j, out[i] digit i of the four values.
+__device__ __forceinline__ void transpose4(uint32_t a, uint32_t b, uint32_t c, uint32_t d, uint32_t (&o)[4]) {
+  const uint32_t p0 = __builtin_amdgcn_perm(b, a, 0x05010400u);  // a0 b0 a1 b1
+  const uint32_t p1 = __builtin_amdgcn_perm(b, a, 0x07030602u);  // a2 b2 a3 b3
+  const uint32_t p2 = __builtin_amdgcn_perm(d, c, 0x05010400u);
+  const uint32_t p3 = __builtin_amdgcn_perm(d, c, 0x07030602u);
+  o[0] = __builtin_amdgcn_perm(p2, p0, 0x05040100u);
+  o[1] = __builtin_amdgcn_perm(p2, p0, 0x07060302u);
+  o[2] = __builtin_amdgcn_perm(p3, p1, 0x05040100u);
+  o[3] = __builtin_amdgcn_perm(p3, p1, 0x07060302u);
+}
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef u4v u4v_a4 __attribute__((aligned(4)));
+typedef f4 f4_a4 __attribute__((aligned(4)));
+
+constexpr int kStepBytes = 1536;  // LDS bytes of one step's B operand rows (9 rows of 128 B, padded)
+constexpr int kRedStride = 68;    // floats per (wave, digit) row of the final reduction
+// Byte offset of step s inside a wave's digit area: the small skew spreads the four steps one
+// store instruction touches over different LDS banks.
+__device__ __forceinline__ constexpr int step_off(int s) {
+  return s * kStepBytes + (s & 1) * 32 + ((s >> 1) & 1) * 128;
 }
 
 template <int WAVES, int STEPS, bool XF16, bool MULTI>
 __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
-  // LDS: xs[WAVES][STEPS*4 groups][4 mfma][4 piece slots] uint4 | red[WAVES][3][64] | xsum[WAVES]
+  // LDS: dig[WAVES][STEPS * kStepBytes] | red[WAVES][8][kRedStride] | part[WAVES][64] | xsum[WAVES]
   extern __shared__ uint4 smem[];
-  uint4* xs = smem;
-  float* red = reinterpret_cast<float*>(smem + WAVES * STEPS * 64);
-  float* wsum = red + WAVES * 3 * 64;
+  char* dig = reinterpret_cast<char*>(smem);
+  float* red = reinterpret_cast<float*>(dig + WAVES * STEPS * kStepBytes);
+  float* part = red + WAVES * 8 * kRedStride;
+  float* wsum = part + WAVES * 64;
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int c = lane & 15, kb = lane >> 4;
@@ -114,12 +142,10 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     zr_n = a.zeros[nc];
     y_old = ((a.flags & HQ_FLAG_ACCUMULATE) && a.nsplit == 1) ? a.y[nc] : 0.f;
   }
-  // activations: lane (c, kb) owns the two codes that unpack16() leaves in register c
-  // of k-group kb (element k_lo in the low half, k_hi in the high half)
-  const uint64_t tw = c < 8 ? (c < 4 ? hq_q3::packed_entries(0) : hq_q3::packed_entries(1))
-                            : (c < 12 ? hq_q3::packed_entries(2) : hq_q3::packed_entries(3));
-  const uint32_t te = (uint32_t)(tw >> (16 * (c & 3))) & 0xffffu;
-  const int k_lo = te & 31, k_hi = (te >> 5) & 31, p_lo = (te >> 10) & 7, p_hi = (te >> 13) & 7;
+  // Activation staging: lane L converts the eight consecutive activations 8*xq .. 8*xq+7 of
+  // k-group xkb of step 4*pass + xs.
+  const int xs = lane >> 4, xkb = (lane >> 2) & 3, xq = lane & 3;
+  constexpr int XP = (STEPS + 3) / 4;  // staging passes per round
   // Scalar base pointers of this workgroup's slice plus 32-bit per-lane byte offsets.
   const char* xbase = reinterpret_cast<const char*>(a.x) + (size_t)g_begin * 32 * (XF16 ? 2 : 4);
   // weights: out-of-range columns read the last valid quad (their results are never
@@ -134,85 +160,106 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   // Every global load of a round is issued up front and none sits under a branch
   // (addresses are clamped instead), so the compiler can count them and the wait for the
   // activations does not wait for the weights.
-  auto load_round = [&](int r, float (&xr)[STEPS][2], uint32_t (&wreg)[STEPS][3][4]) {
-    uint32_t glc[STEPS];
+  auto load_round = [&](int r, float (&xr)[XP][8], uint32_t (&wreg)[STEPS][3][4]) {
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      glc[s] = (uint32_t)min((r * STEPS + s) * (WAVES * 4) + wv * 4 + kb, g_count - 1);
+    for (int p = 0; p < XP; ++p) {
+      const int s = min(4 * p + xs, STEPS - 1);
+      const uint32_t g = (uint32_t)min((r * STEPS + s) * (WAVES * 4) + wv * 4 + xkb, g_count - 1);
+      const uint32_t e = g * 32u + (uint32_t)xq * 8u;
       if (XF16) {
-        xr[s][0] = (float)*reinterpret_cast<const _Float16*>(xbase + (glc[s] * 32u + (uint32_t)k_lo) * 2u);
-        xr[s][1] = (float)*reinterpret_cast<const _Float16*>(xbase + (glc[s] * 32u + (uint32_t)k_hi) * 2u);
+        const u4v raw = *reinterpret_cast<const u4v_a4*>(xbase + e * 2u);
+        const h8 h = __builtin_bit_cast(h8, raw);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xr[p][j] = (float)h[j];
       } else {
-        xr[s][0] = *reinterpret_cast<const float*>(xbase + (glc[s] * 32u + (uint32_t)k_lo) * 4u);
-        xr[s][1] = *reinterpret_cast<const float*>(xbase + (glc[s] * 32u + (uint32_t)k_hi) * 4u);
+        const f4 lo = *reinterpret_cast<const f4_a4*>(xbase + e * 4u);
+        const f4 hi = *reinterpret_cast<const f4_a4*>(xbase + e * 4u + 16u);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { xr[p][j] = lo[j]; xr[p][4 + j] = hi[j]; }
       }
     }
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
+      const uint32_t g = (uint32_t)min((r * STEPS + s) * (WAVES * 4) + wv * 4 + kb, g_count - 1);
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
-        const uint32_t off = (glc[s] * 3u + (uint32_t)j) * row_bytes + col_off;
+        const uint32_t off = (g * 3u + (uint32_t)j) * row_bytes + col_off;
         u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wbase + off));
         wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
       }
     }
   };
 
-  uint4* xs_w = xs + wv * (STEPS * 64);
-  const int piece = c < 3 ? c : 2;  // columns 3..15 of the MFMA are never read
-  float run[4][4];                  // per-digit sums of all rounds, already divided by 2^E
+  char* dig_w = dig + wv * (STEPS * kStepBytes);
+  // Row 8 of every step is the constant one (fp8 0x01 = 2^-9, the unit of the digits).
+  if (lane < 32) {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+      *reinterpret_cast<uint32_t*>(dig_w + step_off(s) + 8 * 128 + lane * 4) = 0x01010101u;
+  }
+  float run[4][4];  // per-digit sums of all rounds (bias removed, divided by 2^E)
 #pragma unroll
   for (int q = 0; q < 4; ++q)
 #pragma unroll
     for (int i = 0; i < 4; ++i) run[q][i] = 0.f;
   float asum_total = 0.f;
+  constexpr uint32_t M0 = low3_mask(0), M1 = low3_mask(1), M2 = low3_mask(2);
 
-  float xr[STEPS][2];
+  float xr[XP][8];
   uint32_t wreg[STEPS][3][4];
   load_round(0, xr, wreg);
   for (int r = 0; r < rounds; ++r) {
-    float xr_next[STEPS][2];
+    float xr_next[XP][8];
     uint32_t wreg_next[STEPS][3][4];
     if (MULTI && r + 1 < rounds) load_round(r + 1, xr_next, wreg_next);  // in flight during this round
 
-    // ---- stage this wave's activation digits in operand-slot order (wave-local) ----------
+    // ---- stage this wave's activation digits (wave-local) ---------------------------------
     float amax = 0.f, asum = 0.f;
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      if ((r * STEPS + s) * (WAVES * 4) + wv * 4 + kb >= g_count) { xr[s][0] = 0.f; xr[s][1] = 0.f; }
-      amax = fmaxf(amax, fmaxf(fabsf(xr[s][0]), fabsf(xr[s][1])));
-      asum += xr[s][0] + xr[s][1];
+    for (int p = 0; p < XP; ++p) {
+      const int s = 4 * p + xs;
+      const bool live = s < STEPS && (r * STEPS + s) * (WAVES * 4) + wv * 4 + xkb < g_count;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (!live) xr[p][j] = 0.f;
+        amax = fmaxf(amax, fabsf(xr[p][j]));
+        asum += xr[p][j];
+      }
     }
     const float xmax = wave_max(amax);
     asum_total += wave_sum(asum);
-    // 2^E * max|x| lies in [2^14, 2^15): digit 0 never overflows fp16.
-    int E = 14 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
+    // 2^E * max|x| lies in [2^29, 2^30): v = rint(x * 2^E) + 0x88888888 never wraps, and its
+    // nibbles n_d satisfy v = sum_d 16^d (n_d - 8).
+    int E = 29 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
     E = xmax > 0.f ? max(-120, min(120, E)) : 0;
     const float scaleE = pow2f(E);
-    // Fixed-point split of v = x * 2^(E + 4 - pos) (|v| < 2^(19-pos)) into three signed
-    // 11-bit digits with quanta 2^9, 2^-2, 2^-13, stored as plain fp16 integers.  With the
-    // operand value code*2^(pos-24) every digit-0 product is an integer below 2^13 in units
-    // of 2^-24, so a round's digit-0 chain (at most 512 slots) is exact in the matrix core
-    // whatever its internal rounding is; digits 1 and 2 carry 2^-11 and 2^-22 of the weight.
-    const float sE_lo = scaleE * pow2f(4 - p_lo), sE_hi = scaleE * pow2f(4 - p_hi);
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      float d[2][3];
+    for (int p = 0; p < XP; ++p) {
+      uint32_t ev[8], od[8];
 #pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const float v = xr[s][e] * (e ? sE_hi : sE_lo);
-        d[e][0] = rintf(v * 0.001953125f);
-        const float r1 = v - d[e][0] * 512.f;   // exact
-        d[e][1] = rintf(r1 * 4.f);
-        const float r2 = r1 - d[e][1] * 0.25f;  // exact
-        d[e][2] = rintf(r2 * 8192.f);
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t t = (uint32_t)(int)rintf(xr[p][j] * scaleE) + 0x88888888u;
+        ev[j] = t & 0x0f0f0f0fu;         // nibbles 0 2 4 6
+        od[j] = (t >> 4) & 0x0f0f0f0fu;  // nibbles 1 3 5 7
       }
-      // register c of MFMA j = c/4 of this k-group: dword c%4 of the 16-byte operand chunk
-      uint32_t* dst = reinterpret_cast<uint32_t*>(xs_w + ((s * 4 + kb) * 4 + (c >> 2)) * 4) + (c & 3);
+      // A operand (fp6): lane quarter g holds K indices 32g .. 32g+31 of the MFMA, element k of the
+      // group at k/2 (even k) or 16 + k/2 (odd k).  B operand (fp8): lane quarter kb holds K indices
+      // 16kb .. 16kb+15 in its first four registers and 64+16kb .. 64+16kb+15 in the last four.
+      uint32_t de[2][4], dd[2][4];
+      transpose4(ev[0], ev[2], ev[4], ev[6], de[0]);
+      transpose4(ev[1], ev[3], ev[5], ev[7], de[1]);
+      transpose4(od[0], od[2], od[4], od[6], dd[0]);
+      transpose4(od[1], od[3], od[5], od[7], dd[1]);
+      const int s = 4 * p + xs;
+      if (s < STEPS) {
+        char* dst = dig_w + step_off(s) + (xkb & 1) * 64 + (xkb >> 1) * 16 + xq * 4;
 #pragma unroll
-      for (int p = 0; p < 3; ++p) {
-        const h2v pair = {(_Float16)d[0][p], (_Float16)d[1][p]};
-        dst[4 * p] = __builtin_bit_cast(uint32_t, pair);
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {  // h = 0: even elements, h = 1: odd elements (next lane quarter)
+            *reinterpret_cast<uint32_t*>(dst + (2 * i) * 128 + h * 32) = de[h][i];
+            *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * 128 + h * 32) = dd[h][i];
+          }
       }
     }
     // The digits are read back by other lanes of this wave only: order the LDS writes
@@ -221,72 +268,82 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 
-    // ---- unpack + MFMA ---------------------------------------------------------------------
+    // ---- mask + MFMA -----------------------------------------------------------------------
     f4 acc[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       if ((r * STEPS + s) * (WAVES * 4) + wv * 4 >= g_count) continue;  // wave-uniform
-      const uint4* xb = xs_w + (size_t)(s * 4 + kb) * 16 + piece;
-      h8 B[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) B[j] = __builtin_bit_cast(h8, xb[j * 4]);
+      // MFMA columns 9..15 are never read: they re-use row 8
+      const u4v* bp = reinterpret_cast<const u4v*>(dig_w + step_off(s) + min(c, 8) * 128 + kb * 32);
+      const u4v b0 = bp[0], b1 = bp[1];
+      const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        uint32_t f[16];
-        unpack16(wreg[s][0][q], wreg[s][1][q], wreg[s][2][q], f);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          u4v av = {f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]};
-          acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, av), B[j], acc[q], 0, 0, 0);
-        }
+        const uint32_t w0 = wreg[s][0][q], w1 = wreg[s][1][q], w2 = wreg[s][2][q];
+        const v8i A = {(int)(w0 & M0), (int)(w1 & M1), (int)(w2 & M2),
+                       (int)(__builtin_amdgcn_alignbit(w1, w0, 3) & M0),
+                       (int)(__builtin_amdgcn_alignbit(w2, w1, 3) & M1), (int)((w2 >> 3) & M2), 0, 0};
+        // A: fp6 e2m3 (cbsz 2), B: fp8 e4m3 (blgp 0), unit block scales
+        acc[q] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, acc[q], 2, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
       }
     }
+    // acc = 2^-12 * sum q*n_d (column d < 8), 2^-12 * sum q (column 8): take the bias out
+    // while everything is still an exact integer, then leave the round's fixed-point scale.
     const float descale = pow2f(-E);
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) run[q][i] = fmaf(acc[q][i], descale, run[q][i]);
+      for (int i = 0; i < 4; ++i) {
+        const float unbiased = fmaf(row_bcast8(acc[q][i]), -8.f, acc[q][i]);
+        run[q][i] = fmaf(unbiased, descale, run[q][i]);
+      }
     // the LDS digits of this round must be consumed before the next round overwrites them
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
     if (MULTI && r + 1 < rounds) {
 #pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        xr[s][0] = xr_next[s][0]; xr[s][1] = xr_next[s][1];
+      for (int p = 0; p < XP; ++p)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) xr[p][j] = xr_next[p][j];
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s)
 #pragma unroll
         for (int j = 0; j < 3; ++j)
 #pragma unroll
           for (int q = 0; q < 4; ++q) wreg[s][j][q] = wreg_next[s][j][q];
-      }
     }
   }
 
-  // ---- combine waves, digits, scale/zero --------------------------------------------------
-  // D[row = 4*kb + i][col = c]: row is the weight column (quarter-major), col the digit.
-  if (c < 3) {
+  // ---- combine digits, waves, scale/zero --------------------------------------------------
+  // D[row = 4*kb + i][col = c]: row is the weight column 4*row + q of the tile, col the digit.
+  if (c < 8) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) red[(wv * 3 + c) * 64 + 4 * (4 * kb + i) + q] = run[q][i];
+    for (int i = 0; i < 4; ++i) {
+      const f4 v = {run[0][i], run[1][i], run[2][i], run[3][i]};
+      *reinterpret_cast<f4*>(red + (wv * 8 + c) * kRedStride + 4 * (4 * kb + i)) = v;
+    }
   }
   if (lane == 0) wsum[wv] = asum_total;
   __syncthreads();
+  {
+    const float* rw = red + (wv * 8) * kRedStride + lane;
+    float h = rw[7 * kRedStride];
+#pragma unroll
+    for (int d = 6; d >= 0; --d) h = fmaf(h, 16.f, rw[d * kRedStride]);
+    part[wv * 64 + lane] = h;
+  }
+  __syncthreads();
   float val = 0.f;
   if (tid < 64 && n < a.N) {
-    const float inv11 = 1.f / 2048.f;
     float qx = 0.f, xsum = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      const float c0 = red[(w * 3 + 0) * 64 + tid];
-      const float c1 = red[(w * 3 + 1) * 64 + tid];
-      const float c2 = red[(w * 3 + 2) * 64 + tid];
-      qx += fmaf(fmaf(c2, inv11, c1), inv11, c0);
+      qx += part[w * 64 + tid];
       xsum += wsum[w];
     }
-    // 2^24 (operand scale) * 2^9 (digit-0 quantum) * 2^-4 (slot scale)
-    val = sc_n * (qx * 536870912.f) - zr_n * xsum;
+    val = sc_n * (qx * 4096.f) - zr_n * xsum;  // 2^12: fp6 unit 2^-3 times fp8 unit 2^-9
     if (a.nsplit == 1) {
       a.y[n] = y_old + val;
     } else {
@@ -327,7 +384,8 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
 
 template <int WAVES, int STEPS, bool XF16, bool MULTI>
 int launch_matvec_t(const Q3Args& a, int ntiles, hipStream_t stream) {
-  const size_t smem = (size_t)WAVES * STEPS * 1024 + (size_t)WAVES * 3 * 64 * 4 + (size_t)WAVES * 2 * 4;
+  const size_t smem = (size_t)WAVES * STEPS * kStepBytes + (size_t)WAVES * 8 * kRedStride * 4 + (size_t)WAVES * 64 * 4 +
+                      (size_t)WAVES * 4 + 16;
   static const hipError_t attr =
       hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_matvec_kernel<WAVES, STEPS, XF16, MULTI>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
