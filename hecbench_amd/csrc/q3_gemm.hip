@@ -13,11 +13,12 @@
 // activations by a small pre-pass that also reorders them into operand-slot order
 // ([k-group][mfma j][row][8 halves]) and computes the row sums for the zero term.
 // The main kernel streams the weights once: a workgroup (8 waves) owns 128 output
-// columns and all of K, walks K in chunks of 16 k-groups whose activation slices
-// are double-buffered in LDS, and each wave multiplies 2 k-groups x 128 columns x
-// 64 rows per chunk with 32x32x16 fp16 MFMAs (fp32 accumulate).  The eight waves'
-// accumulators are summed through LDS at the end and scale/zero are applied once
-// per output.
+// columns and all of K and walks K in steps of 16 k-groups; each wave owns two
+// k-groups of a step, loads their activation slices (from L2) and packed rows (from
+// HBM) straight into registers one step ahead, and multiplies 2 k-groups x 128
+// columns x 64 rows per step with 32x32x16 fp16 MFMAs (fp32 accumulate).  There is
+// no LDS traffic and no barrier in the loop.  The eight waves' accumulators are
+// summed through LDS at the end and scale/zero are applied once per output.
 #include "hq_internal.h"
 #include "q3_recipe.h"
 
@@ -29,22 +30,26 @@ typedef float f4v __attribute__((ext_vector_type(4)));
 typedef float f2v __attribute__((ext_vector_type(2)));
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 
-constexpr int kChunk = 16;   // k-groups per LDS chunk
-constexpr int kWaves = 8;
+constexpr int kChunk = 16;      // the pre-pass pads K to a multiple of this many k-groups
+constexpr int kWaves = 8;       // two per SIMD
+constexpr int kStepGroups = 16; // k-groups a workgroup consumes per step (two per wave)
 constexpr int kTileN = 128;  // output columns per workgroup
 
 
 // ---- pre-pass: activations -> operand-slot order, scaled by 2^-pos; row sums ----------------
-// grid (Mpad), block 256.  Ap[((g*4 + j)*Mpad + m)*8 + e] = A[m][32g + k] * 2^-pos(k) with
-// slot(k) = 8j + e; rows >= M and groups >= G hold zeros.
+// Ap[((g*4 + j)*Mpad + m)*8 + e] = A[m][32g + k] * 2^-pos(k) with slot(k) = 8j + e; rows >= M and
+// groups >= G hold zeros.  Blocks [0, Gpad/4): wave w of block b re-orders k-group 4b + w, lane =
+// row, so the 16-byte pieces of 64 rows form 1 KB contiguous stores.  Blocks [Gpad/4, Gpad/4 +
+// Mpad): one block per row sums the row in a fixed order (deterministic).
 __global__ __launch_bounds__(256) void q3_gemm_prep(const _Float16* __restrict__ A, _Float16* __restrict__ Ap,
                                                    float* __restrict__ rowsum, int M, int K, int Mpad,
                                                    int Gpad) {
-  const int m = blockIdx.x, tid = threadIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int G = K >> 5;
-  __shared__ float part[256];
-  float sum = 0.f;
-  for (int g = tid; g < Gpad; g += 256) {
+  const int nreorder = Gpad >> 2;
+  if ((int)blockIdx.x < nreorder) {
+    const int g = blockIdx.x * 4 + wv, m = lane;
+    if (m >= Mpad) return;
     _Float16 out[32];
 #pragma unroll
     for (int i = 0; i < 32; ++i) out[i] = (_Float16)0.f;
@@ -56,10 +61,9 @@ __global__ __launch_bounds__(256) void q3_gemm_prep(const _Float16* __restrict__
       const _Float16* in = reinterpret_cast<const _Float16*>(raw);
 #pragma unroll
       for (int k = 0; k < 32; ++k) {
-        const float v = (float)in[k];
-        sum += v;
         // exact power-of-two scaling (subnormal results lose bits below 2^-24 only)
-        out[hq_q3::slot_of(k)] = (_Float16)(v * __uint_as_float((uint32_t)(127 - hq_q3::pos_of(k)) << 23));
+        out[hq_q3::slot_of(k)] =
+            (_Float16)((float)in[k] * __uint_as_float((uint32_t)(127 - hq_q3::pos_of(k)) << 23));
       }
     }
 #pragma unroll
@@ -67,14 +71,38 @@ __global__ __launch_bounds__(256) void q3_gemm_prep(const _Float16* __restrict__
       u4v* dst = reinterpret_cast<u4v*>(Ap + ((size_t)(g * 4 + j) * Mpad + m) * 8);
       *dst = *reinterpret_cast<const u4v*>(out + 8 * j);
     }
+    return;
   }
-  part[tid] = sum;
+  // one block per row: every thread's loads are independent and issued together
+  const int m = (int)blockIdx.x - nreorder;
+  __shared__ float part[4];
+  float sum = 0.f;
+  if (m < M) {
+    const u4v* src = reinterpret_cast<const u4v*>(A + (size_t)m * K);
+    const int n16 = K >> 3;
+    for (int i0 = 0; i0 < n16; i0 += 4 * 256) {
+      u4v raw[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * 256 + (int)threadIdx.x;
+        raw[u] = src[min(i, n16 - 1)];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * 256 + (int)threadIdx.x;
+        const _Float16* in = reinterpret_cast<const _Float16*>(&raw[u]);
+        float s8 = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s8 += (float)in[e];
+        sum += i < n16 ? s8 : 0.f;
+      }
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  if (lane == 0) part[wv] = sum;
   __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) {
-    if (tid < s) part[tid] += part[tid + s];
-    __syncthreads();
-  }
-  if (tid == 0) rowsum[m] = part[0];
+  if (threadIdx.x == 0) rowsum[m] = (part[0] + part[1]) + (part[2] + part[3]);
 }
 
 // Sixteen two-field registers of one column's k-group (see q3_recipe.h).
@@ -105,18 +133,25 @@ struct GemmArgs {
 template <int MB>  // 32-row blocks of activations
 __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
   constexpr int Mpad = 32 * MB;
-  constexpr int CHUNK_U4 = kChunk * 4 * Mpad;  // 16-byte units of one activation chunk
-  constexpr int T = kWaves * 64;
-  constexpr int COPY = CHUNK_U4 / T;           // 16-byte units each thread copies per chunk
-  extern __shared__ u4v lds[];                 // 2 * CHUNK_U4 (double buffer); reused by the reduction
+  extern __shared__ u4v lds[];  // used by the final reduction only
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int nl = lane & 31, kb = lane >> 5;
   const int G = a.K >> 5;
-  const int nchunks = a.Gpad / kChunk;
+  const int nsteps = a.Gpad / kStepGroups;
   const int col0 = blockIdx.x * kTileN;
   const int col = min(col0 + 4 * nl, a.N - 4);  // out-of-range columns re-read valid data, never stored
   const size_t row_stride = (size_t)a.N;
+
+  // what the epilogue needs, fetched while the first operands are on their way
+  const int n_out = col0 + 4 * nl;
+  f4v sc = {0.f, 0.f, 0.f, 0.f}, zr = {0.f, 0.f, 0.f, 0.f};
+  if (n_out < a.N) {  // N % 4 == 0: the four columns are in range together
+    sc = *reinterpret_cast<const f4v*>(a.scales + n_out);
+    zr = *reinterpret_cast<const f4v*>(a.zeros + n_out);
+  }
+  constexpr int ROWS_PER_WAVE = Mpad / kWaves;
+  const float rs_lane = a.rowsum[wv * ROWS_PER_WAVE + (lane & (ROWS_PER_WAVE - 1))];
 
   f16v acc[MB][4];
 #pragma unroll
@@ -126,45 +161,35 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][q][i] = 0.f;
 
-  u4v stage[COPY];
-  uint32_t wreg[3][4];
-  auto load_chunk = [&](int ch) {
-    const u4v* src = a.Ap + (size_t)ch * CHUNK_U4;
-#pragma unroll
-    for (int i = 0; i < COPY; ++i) stage[i] = src[tid + i * T];
-    // this wave's two k-groups of the chunk: group index 2*wv + kb
-    const int g = min(ch * kChunk + 2 * wv + kb, G - 1);  // padded groups: any valid weights, zero activations
-    const uint32_t* p = a.w + (size_t)(3 * g) * row_stride + col;
+  // A wave owns k-groups 2*wv + kb of every step of kStepGroups k-groups and loads its
+  // operands straight into registers, one step ahead: the activations of one k-group (4 MFMA K-steps x MB row
+  // blocks, 16 bytes per lane each, 512 contiguous bytes per half wave) and three packed
+  // weight rows.  No LDS and no barrier in the loop: waves drift apart, so one wave's loads
+  // overlap the other waves' MFMAs.
+  const u4v* ap_lane = a.Ap + (size_t)((2 * wv + kb) * 4) * Mpad + nl;
+  auto load_step = [&](int t, u4v (&A)[4][MB], uint32_t (&wr)[3][4]) {
+    const int g = min(t * kStepGroups + 2 * wv + kb, G - 1);  // padded groups: any valid weights, zero activations
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
-      const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(p + j * row_stride));
-      wreg[j][0] = v.x; wreg[j][1] = v.y; wreg[j][2] = v.z; wreg[j][3] = v.w;
+      const u4v v = __builtin_nontemporal_load(
+          reinterpret_cast<const u4v*>(a.w + (size_t)(3 * g + j) * row_stride + col));
+      wr[j][0] = v.x; wr[j][1] = v.y; wr[j][2] = v.z; wr[j][3] = v.w;
     }
-  };
-  auto store_chunk = [&](int buf) {
-    u4v* dst = lds + buf * CHUNK_U4;
-#pragma unroll
-    for (int i = 0; i < COPY; ++i) dst[tid + i * T] = stage[i];
-  };
-
-  load_chunk(0);
-  store_chunk(0);
-  uint32_t wcur[3][4];
-#pragma unroll
-  for (int j = 0; j < 3; ++j)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) wcur[j][q] = wreg[j][q];
-  __syncthreads();
-
-  for (int ch = 0; ch < nchunks; ++ch) {
-    const bool more = ch + 1 < nchunks;
-    if (more) load_chunk(ch + 1);  // global loads in flight during the MFMAs
-    const u4v* abuf = lds + (ch & 1) * CHUNK_U4 + (size_t)((2 * wv + kb) * 4) * Mpad + nl;
-    h8 A[4][MB];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) A[j][mb] = __builtin_bit_cast(h8, abuf[j * Mpad + mb * 32]);
+      for (int mb = 0; mb < MB; ++mb) A[j][mb] = ap_lane[(size_t)t * (kStepGroups * 4 * Mpad) + j * Mpad + mb * 32];
+  };
+
+  u4v Acur[4][MB], Anext[4][MB];
+  uint32_t wcur[3][4], wnext[3][4];
+  load_step(0, Acur, wcur);
+
+  for (int t = 0; t < nsteps; ++t) {
+    // All of the next step's loads are issued before this step's MFMAs, so they have the
+    // whole step to arrive (the last trip re-reads its own step instead of branching).
+    load_step(min(t + 1, nsteps - 1), Anext, wnext);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       uint32_t f[16];
@@ -175,23 +200,25 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
         const h8 B = __builtin_bit_cast(h8, bv);
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          acc[mb][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[j][mb], B, acc[mb][q], 0, 0, 0);
+          acc[mb][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, Acur[j][mb]), B, acc[mb][q], 0, 0, 0);
       }
     }
-    if (more) {
-      store_chunk((ch + 1) & 1);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int j = 0; j < 3; ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) wcur[j][q] = wreg[j][q];
-    }
-    __syncthreads();
+      for (int mb = 0; mb < MB; ++mb) Acur[j][mb] = Anext[j][mb];
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) wcur[j][q] = wnext[j][q];
   }
+  __syncthreads();
 
-  // ---- sum the eight waves' accumulators through LDS ------------------------------------------
+  // ---- sum the waves' accumulators through LDS -------------------------------------------
   // D[row][col = nl]: register i of a lane holds row (i/4)*8 + kb*4 + i%4 of its 32-row block;
   // the four accumulators q of a lane are four adjacent output columns 4*nl + q.
-  float* red = reinterpret_cast<float*>(lds);  // regions of [Mpad][128] floats
+  float* red = reinterpret_cast<float*>(lds);  // kWaves/2 regions of [Mpad][128] floats
   constexpr int REGION = Mpad * kTileN;
   auto put = [&](int region) {
 #pragma unroll
@@ -203,9 +230,10 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
         *reinterpret_cast<f4v*>(red + (size_t)region * REGION + m * kTileN + 4 * nl) = v;
       }
   };
-  if (wv >= 4) put(wv - 4);
+  constexpr int H = kWaves / 2;
+  if (wv >= H) put(wv - H);
   __syncthreads();
-  if (wv < 4) {
+  if (wv < H) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -216,27 +244,23 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
       }
   }
   __syncthreads();
-  if (wv < 4) put(wv);
+  if (wv < H) put(wv);
   __syncthreads();
-  // every wave finishes Mpad/8 rows: lane -> two adjacent columns
-  const int n = col0 + 2 * lane;
-  if (n < a.N) {  // N % 4 == 0 and n even: n + 1 < N as well
-    const f2v sc = *reinterpret_cast<const f2v*>(a.scales + n);
-    const f2v zr = *reinterpret_cast<const f2v*>(a.zeros + n);
+  // every wave finishes Mpad/kWaves rows: half wave kb takes every other row, lane -> four columns
 #pragma unroll
-    for (int r = 0; r < Mpad / kWaves; ++r) {
-      const int m = wv * (Mpad / kWaves) + r;
-      if (m >= a.M) break;
-      f2v s = {0.f, 0.f};
+  for (int r = kb; r < ROWS_PER_WAVE; r += 2) {
+    const int m = wv * ROWS_PER_WAVE + r;
+    const float rs = __shfl(rs_lane, r);  // every lane takes part (the row sum lives in lane r)
+    if (m < a.M && n_out < a.N) {
+      f4v v = *reinterpret_cast<const f4v*>(red + m * kTileN + 4 * nl);
 #pragma unroll
-      for (int region = 0; region < 4; ++region) {
-        const f2v v = *reinterpret_cast<const f2v*>(red + (size_t)region * REGION + m * kTileN + 2 * lane);
-        s.x += v.x; s.y += v.y;
-      }
-      const float rs = a.rowsum[m];
-      f2v o = {sc.x * (s.x * 16777216.f) - zr.x * rs, sc.y * (s.y * 16777216.f) - zr.y * rs};
-      f2v* dst = reinterpret_cast<f2v*>(a.out + (size_t)m * a.N + n);
-      if (a.flags & HQ_FLAG_ACCUMULATE) { const f2v old = *dst; o.x += old.x; o.y += old.y; }
+      for (int region = 1; region < H; ++region)
+        v += *reinterpret_cast<const f4v*>(red + (size_t)region * REGION + m * kTileN + 4 * nl);
+      f4v o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = sc[e] * (v[e] * 16777216.f) - zr[e] * rs;
+      f4v* dst = reinterpret_cast<f4v*>(a.out + (size_t)m * a.N + n_out);
+      if (a.flags & HQ_FLAG_ACCUMULATE) { const f4v old = *dst; o += old; }
       *dst = o;
     }
   }
@@ -245,8 +269,7 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
 template <int MB>
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   constexpr int Mpad = 32 * MB;
-  const size_t smem = (size_t)2 * kChunk * 4 * Mpad * 16;
-  static_assert((size_t)4 * Mpad * kTileN * 4 <= (size_t)2 * kChunk * 4 * Mpad * 16, "reduction regions fit the chunk buffers");
+  const size_t smem = (size_t)(kWaves / 2) * Mpad * kTileN * 4;  // reduction regions
   static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_gemm_kernel<MB>),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (attr != hipSuccess) return (int)attr;
@@ -259,7 +282,7 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream) {
 int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
                       int K, int N, int M, unsigned flags, hipStream_t stream) {
   if (((uintptr_t)x & 15) || (K & 7)) return HQ_ERR_MISALIGNED;
-  if (((uintptr_t)scales & 7) || ((uintptr_t)zeros & 7) || ((uintptr_t)y & 7)) return HQ_ERR_MISALIGNED;
+  if (((uintptr_t)scales & 15) || ((uintptr_t)zeros & 15) || ((uintptr_t)y & 15)) return HQ_ERR_MISALIGNED;
   const int G = K / 32;
   const int Gpad = (G + kChunk - 1) / kChunk * kChunk;
   const size_t ap_halves = (size_t)Gpad * 4 * 64 * 8;
@@ -274,7 +297,8 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
     const int MB = Mb > 32 ? 2 : 1;
     const int Mpad = 32 * MB;
     const _Float16* A = reinterpret_cast<const _Float16*>(x) + (size_t)m0 * K;
-    hipLaunchKernelGGL(q3_gemm_prep, dim3(Mpad), dim3(256), 0, stream, A, Ap, rowsum, Mb, K, Mpad, Gpad);
+    hipLaunchKernelGGL(q3_gemm_prep, dim3(Gpad / 4 + Mpad), dim3(256), 0, stream, A, Ap, rowsum, Mb, K, Mpad,
+                       Gpad);
     rc = hq_launch_status();
     if (rc != HQ_OK) return rc;
     GemmArgs a;
