@@ -188,37 +188,33 @@ __global__ __launch_bounds__(256) void lut_gemv_kernel(LutArgs a) {
 // ======================================================================================
 // Matrix-core path (group size a multiple of 128, N a multiple of 64).
 //
-// sum_k s*x = 2*(sum_k bit*x - (sum_k x)/2).  An fp8 (e4m3) byte whose exponent field is
-// zero is the subnormal mantissa*2^-9, so a single weight bit left in place at bit p
-// (p <= 2) of an otherwise zero byte IS the fp8 number 2^(p-9): eight ANDs and two shifts
-// turn a packed 32-bit word into the eight operand registers (32 fp8 values) of one
-// 16x16x128 fp8 MFMA; the factor 2^p is folded into the activation of that slot.  No table,
-// no LDS lookup, no bank conflicts.  The activations of a round (256 of them per wave) are
-// scaled to 16-bit fixed point and split into four signed 4-bit digits carried by MFMA
-// columns 0..3, so every product is an integer and the matrix-core sums are exact.  Lane
-// quarter kb streams k-word 4*quad + kb, so one MFMA sums a whole 128-element quad of one
-// bit plane for 16 columns (four adjacent columns per lane and 128-bit load); alpha is
-// applied to that sum in fp32, per digit, and the digits are combined once at the end.
+// sum_k s*x = 2*(sum_k bit*x - (sum_k x)/2).  An fp4 (e2m1) nibble with only its lowest bit set
+// is the number 0.5, so `(word >> p) & 0x11111111` (p = 0..3) turns a packed 32-bit word into
+// the four operand registers (32 fp4 values) of one 16x16x128 f8f6f4 MFMA: seven VALU
+// instructions per 32 weights, no table, no LDS lookup.  The activations of a round are
+// scaled to 16-bit fixed point, biased by 0x8888 and cut into four nibbles; a nibble 0..15 in
+// an otherwise zero byte is the fp8 (e4m3) number nibble * 2^-9, so the digits need no
+// conversion, only a byte transpose.  MFMA column d carries nibble d, column 4 a constant one
+// (it counts the set bits, which takes the bias out at the very end), so every product is an
+// integer and the matrix-core sums are exact.  Lane quarter kb streams k-word 4*quad + kb, so
+// one MFMA sums a whole 128-element quad of one bit plane for 16 columns (four adjacent
+// columns per lane and 128-bit load); alpha is applied to that sum in fp32, per MFMA column,
+// and the columns are combined once at the end.
 typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 
-// operand register r of a word holds bit r of each of its four bytes, at mantissa bit p(r)
-__device__ __forceinline__ constexpr int bit_pos(int r) { return r < 6 ? r % 3 : r - 6; }
-__device__ __forceinline__ constexpr uint32_t bit_mask(int r) { return 0x01010101u << bit_pos(r); }
-
-__device__ __forceinline__ v8i unpack_bits_fp8(uint32_t w) {
-  const uint32_t w3 = w >> 3, w6 = w >> 6;
-  v8i a;
-#pragma unroll
-  for (int r = 0; r < 8; ++r) a[r] = (int)((r < 3 ? w : (r < 6 ? w3 : w6)) & bit_mask(r));
+// A operand: element 8p + i of a lane quarter is bit 4i + p of its word.
+__device__ __forceinline__ v8i unpack_bits_fp4(uint32_t w) {
+  const v8i a = {(int)(w & 0x11111111u), (int)((w >> 1) & 0x11111111u), (int)((w >> 2) & 0x11111111u),
+                 (int)((w >> 3) & 0x11111111u), 0, 0, 0, 0};
   return a;
 }
 
-__device__ __forceinline__ f4 mfma_fp8(v8i a, v8i b, f4 c) {
-  // fp8 x fp8, both block scales 2^0 (E8M0 code 127)
-  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+__device__ __forceinline__ f4 mfma_fp4_fp8(v8i a, v8i b, f4 c) {
+  // A fp4 e2m1 (cbsz 4), B fp8 e4m3 (blgp 0), both block scales 2^0 (E8M0 code 127)
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 4, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
 }
 
 template <int CTRL>
@@ -238,26 +234,24 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 struct Half16 {  // sixteen fp16 values as two 128-bit loads
-  u4v lo, hi;
-  __device__ __forceinline__ float get(int i) const {
-    const uint32_t w[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    const uint32_t d = w[i >> 1];
-    return (float)__builtin_bit_cast(_Float16, (uint16_t)((i & 1) ? (d >> 16) : (d & 0xffffu)));
-  }
+  h8 lo, hi;
+  __device__ __forceinline__ float get(int i) const { return (float)(i < 8 ? lo[i] : hi[i - 8]); }
 };
 __device__ __forceinline__ Half16 load_half16(const _Float16* p) {
   Half16 h;
-  h.lo = reinterpret_cast<const u4v*>(p)[0];
-  h.hi = reinterpret_cast<const u4v*>(p)[1];
+  h.lo = reinterpret_cast<const h8*>(p)[0];
+  h.hi = reinterpret_cast<const h8*>(p)[1];
   return h;
 }
+
+constexpr int kQuadBytes = 5 * 128;  // B operand rows of one quad: four digits and the ones row
 
 // NB bit planes, QUADS 128-element quads per wave per round, WAVES waves per workgroup.
 template <int NB, int QUADS, int WAVES, bool BIAS>
 __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
   extern __shared__ float lds[];
-  uint32_t* xs = reinterpret_cast<uint32_t*>(lds);  // [waves][QUADS][4 kb][4 digits][8 regs] dwords
-  float* red = lds + WAVES * QUADS * 128;           // [waves][4 digits][64]
+  char* xs = reinterpret_cast<char*>(lds);                             // [waves][QUADS][5 rows][4 kb][32 B]
+  float* red = reinterpret_cast<float*>(xs + WAVES * QUADS * kQuadBytes);  // [waves][5 columns][64]
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int c = lane & 15, kb = lane >> 4;
   const int tile = blockIdx.x;
@@ -265,16 +259,24 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
   const size_t n0 = (size_t)tile * 64;
   const uint32_t col_off = 4u * c;   // first of the lane's 4 columns (N % 64 == 0: no partial tiles)
   const uint32_t acol = 16u * kb;    // first of the 16 columns this lane applies alpha to
-  // staging role of lane (c, kb): elements k_lo = (c&7) + 16*(c>>3) and k_lo + 8 of k-word kb,
-  // i.e. operand register r = c&7, bytes 2*(c>>3) and 2*(c>>3)+1
-  const int r_slot = c & 7, k_lo = r_slot + 16 * (c >> 3);
-  const float slot_scale = __uint_as_float((uint32_t)(127 + 2 - bit_pos(r_slot)) << 23);  // 2^(2-p)
-  uint32_t* xs_w = xs + wv * (QUADS * 128);
-  const int digit = c & 3;  // MFMA column -> digit (columns 4..15 repeat them and are never read)
+  char* xs_w = xs + wv * (QUADS * kQuadBytes);
+  // Staging role of a lane: 32 lanes per quad; lane (sa, sp, sh) owns the four activations
+  // k = 32*sa + 4*(4*sh + j) + sp, j = 0..3, i.e. A elements 8*sp + 4*sh + j of word sa.  The
+  // fp8 operand of lane quarter b holds MFMA K indices 16b .. 16b+15 in bytes 0..15 and
+  // 64+16b .. 64+16b+15 in bytes 16..31, the fp4 operand of quarter sa holds 32sa .. 32sa+31.
+  const int st = lane >> 5, sa = (lane >> 3) & 3, sp = (lane >> 1) & 3, sh = lane & 1;
+  const int e0 = 8 * sp + 4 * sh;
+  const int s_quarter = 2 * (sa & 1) + (e0 >> 4), s_byte = 16 * (sa >> 1) + (e0 & 15);
+  constexpr int SP = (QUADS + 1) / 2;  // staging passes per round (two quads per pass)
 
   v8i ones;  // every slot's bit set: one MFMA with it sums the digits of a quad
 #pragma unroll
-  for (int r = 0; r < 8; ++r) ones[r] = (int)bit_mask(r);
+  for (int r = 0; r < 8; ++r) ones[r] = r < 4 ? 0x11111111 : 0;
+  // row 4 of every quad is the constant one (fp8 0x01 = 2^-9, the unit of the digits)
+  if (lane < 32) {
+#pragma unroll
+    for (int t = 0; t < QUADS; ++t) *reinterpret_cast<uint32_t*>(xs_w + t * kQuadBytes + 4 * 128 + lane * 4) = 0x01010101u;
+  }
 
   float tot[4][4];
 #pragma unroll
@@ -284,14 +286,14 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
 
   for (int q0 = wv * QUADS; q0 < nquads; q0 += WAVES * QUADS) {
     // ---- loads of this round (unconditional, clamped): activations, then packed words -------
-    float xlo[QUADS], xhi[QUADS];
+    float xv[SP][4];
     u4v wq[QUADS][NB];
 #pragma unroll
-    for (int t = 0; t < QUADS; ++t) {
-      const int quad = min(q0 + t, nquads - 1);
-      const _Float16* xp = a.x + (size_t)quad * 128 + 32 * kb + k_lo;
-      xlo[t] = (float)xp[0];
-      xhi[t] = (float)xp[8];
+    for (int sp_ = 0; sp_ < SP; ++sp_) {
+      const int quad = min(q0 + min(2 * sp_ + st, QUADS - 1), nquads - 1);
+      const _Float16* xp = a.x + (size_t)quad * 128 + 32 * sa + 16 * sh + sp;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xv[sp_][j] = (float)xp[4 * j];
     }
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
@@ -301,37 +303,54 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
       for (int b = 0; b < NB; ++b)
         wq[t][b] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wp + (size_t)b * a.N));
     }
-    // ---- scale to 16-bit fixed point, split into four signed 4-bit digits, stage (wave-local)
-    float amax = 0.f;
+    // alpha and bias of the round's quads: issued here so that they arrive with the words
+    Half16 al[QUADS][NB], bi[QUADS];
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
-      if (q0 + t >= nquads) { xlo[t] = 0.f; xhi[t] = 0.f; }
-      amax = fmaxf(amax, fmaxf(fabsf(xlo[t]), fabsf(xhi[t])));
+      const int g = (min(q0 + t, nquads - 1) * 128) / a.G;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) al[t][b] = load_half16(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
+      if (BIAS) bi[t] = load_half16(a.qbias + (size_t)g * a.N + n0 + acol);
+    }
+    // ---- scale to 16-bit fixed point, bias, cut into nibbles, stage (wave-local) ------------
+    float amax = 0.f;
+#pragma unroll
+    for (int sp_ = 0; sp_ < SP; ++sp_) {
+      const int t = 2 * sp_ + st;
+      const bool live = t < QUADS && q0 + t < nquads;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (!live) xv[sp_][j] = 0.f;
+        amax = fmaxf(amax, fabsf(xv[sp_][j]));
+      }
     }
     const float xmax = wave_max(amax);
-    // 2^E * max|x| lies in [2^14, 2^15)
-    int E = 14 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
+    // 2^E * max|x| lies in [2^13, 2^14): v = rint(x * 2^E) + 0x8888 stays inside 16 bits and its
+    // nibbles n_d satisfy v = sum_d 16^d (n_d - 8)
+    int E = 13 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
     E = xmax > 0.f ? max(-120, min(120, E)) : 0;
     const float scaleE = __uint_as_float((uint32_t)(E + 127) << 23);
 #pragma unroll
-    for (int t = 0; t < QUADS; ++t) {
-      float d[2][4];
+    for (int sp_ = 0; sp_ < SP; ++sp_) {
+      uint32_t ev[4], od[4];
 #pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const float X = rintf((e ? xhi[t] : xlo[t]) * scaleE);
-        d[e][0] = rintf(X * (1.f / 4096.f));
-        const float r1 = X - d[e][0] * 4096.f;
-        d[e][1] = rintf(r1 * (1.f / 256.f));
-        const float r2 = r1 - d[e][1] * 256.f;
-        d[e][2] = rintf(r2 * (1.f / 16.f));
-        d[e][3] = r2 - d[e][2] * 16.f;
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t u = (uint32_t)((int)rintf(xv[sp_][j] * scaleE) + 0x8888);
+        ev[j] = u & 0x0f0fu;         // nibbles 0 (byte 0) and 2 (byte 1)
+        od[j] = (u >> 4) & 0x0f0fu;  // nibbles 1 and 3
       }
-      uint16_t* dst = reinterpret_cast<uint16_t*>(xs_w + ((t * 4 + kb) * 4) * 8 + r_slot) + (c >> 3);
+      // byte transposes: digit d of the four activations in one dword
+      const uint32_t pe = __builtin_amdgcn_perm(ev[1], ev[0], 0x05010400u);  // a0 b0 a2 b2
+      const uint32_t qe = __builtin_amdgcn_perm(ev[3], ev[2], 0x05010400u);  // c0 d0 c2 d2
+      const uint32_t po = __builtin_amdgcn_perm(od[1], od[0], 0x05010400u);
+      const uint32_t qo = __builtin_amdgcn_perm(od[3], od[2], 0x05010400u);
+      const uint32_t dg[4] = {__builtin_amdgcn_perm(qe, pe, 0x05040100u), __builtin_amdgcn_perm(qo, po, 0x05040100u),
+                              __builtin_amdgcn_perm(qe, pe, 0x07060302u), __builtin_amdgcn_perm(qo, po, 0x07060302u)};
+      const int t = 2 * sp_ + st;
+      if (t < QUADS) {
+        char* dst = xs_w + t * kQuadBytes + s_quarter * 32 + s_byte;
 #pragma unroll
-      for (int dg = 0; dg < 4; ++dg) {
-        // digit * 2^(2-p) is exact in fp8 (|digit| <= 8)
-        const int pk = __builtin_amdgcn_cvt_pk_fp8_f32(d[0][dg] * slot_scale, d[1][dg] * slot_scale, 0, false);
-        dst[dg * 16] = (uint16_t)pk;  // next digit: 8 registers = 16 halves further
+        for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(dst + d * 128) = dg[d];
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -346,34 +365,30 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
       if (q0 + t >= nquads) break;  // wave-uniform
-      const int quad = q0 + t;
-      const int g = (quad * 128) / a.G;
-      Half16 al[NB];
-#pragma unroll
-      for (int b = 0; b < NB; ++b) al[b] = load_half16(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
-      const u4v* bp = reinterpret_cast<const u4v*>(xs_w + ((t * 4 + kb) * 4 + digit) * 8);
+      // MFMA columns 5..15 are never read: they re-use the ones row
+      const u4v* bp = reinterpret_cast<const u4v*>(xs_w + t * kQuadBytes + min(c, 4) * 128 + kb * 32);
       const u4v b0 = bp[0], b1 = bp[1];
       const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
-      // digit sum of the quad (in operand units 2^-7), identical in all four result rows
-      const f4 dsum = mfma_fp8(ones, B, f4{0.f, 0.f, 0.f, 0.f});
+      // column sum of the quad (digits 0..3: sum of the nibbles; column 4: 128), in units of
+      // 2^-10, identical in all four result rows
+      const f4 dsum = mfma_fp4_fp8(ones, B, f4{0.f, 0.f, 0.f, 0.f});
       const f4 init = {-0.5f * dsum[0], -0.5f * dsum[1], -0.5f * dsum[2], -0.5f * dsum[3]};
       if (BIAS) {
-        const Half16 bi = load_half16(a.qbias + (size_t)g * a.N + n0 + acol);
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) run[q][i] = fmaf(bi.get(4 * i + q), 0.5f * dsum[i], run[q][i]);
+          for (int q = 0; q < 4; ++q) run[q][i] = fmaf(bi[t].get(4 * i + q), 0.5f * dsum[i], run[q][i]);
       }
 #pragma unroll
       for (int b = 0; b < NB; ++b) {
         const uint32_t words[4] = {wq[t][b].x, wq[t][b].y, wq[t][b].z, wq[t][b].w};
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          // one MFMA = this digit's sum over the quad of bit*x, minus half the digit sum
-          const f4 acc = mfma_fp8(unpack_bits_fp8(words[q]), B, init);
+          // one MFMA = this column's sum over the quad of bit*nibble, minus half the column sum
+          const f4 acc = mfma_fp4_fp8(unpack_bits_fp4(words[q]), B, init);
           // rows 4*kb + i of the tile's 16-column block q: column 16*kb + 4*i + q
 #pragma unroll
-          for (int i = 0; i < 4; ++i) run[q][i] = fmaf(al[b].get(4 * i + q), acc[i], run[q][i]);
+          for (int i = 0; i < 4; ++i) run[q][i] = fmaf(al[t][b].get(4 * i + q), acc[i], run[q][i]);
         }
       }
     }
@@ -385,12 +400,12 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
   }
-  // ---- combine digits and waves -------------------------------------------------------------------
-  if (c < 4) {
+  // ---- combine columns and waves ------------------------------------------------------------------
+  if (c < 5) {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) red[(wv * 4 + c) * 64 + 16 * kb + 4 * i + q] = tot[q][i];
+      for (int i = 0; i < 4; ++i) red[(wv * 5 + c) * 64 + 16 * kb + 4 * i + q] = tot[q][i];
   }
   __syncthreads();
   const int n = tile * 64 + tid;
@@ -398,11 +413,12 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
     float v = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      const float* rw = red + (w * 4) * 64 + tid;
-      v += ((rw[0] * 16.f + rw[64]) * 16.f + rw[128]) * 16.f + rw[192];
+      const float* rw = red + (w * 5) * 64 + tid;
+      // digits 3..0, then the bias of 8 per nibble times the (centred) bit count of column 4
+      v += (((rw[192] * 16.f + rw[128]) * 16.f + rw[64]) * 16.f + rw[0]) - 34952.f * rw[256];
     }
-    // operand units 2^-7, and the sums hold half of sum s*x
-    a.y[n] = (_Float16)(v * 256.f);
+    // operand units 2^-10, and the sums hold half of sum s*x
+    a.y[n] = (_Float16)(v * 2048.f);
   }
 }
 
@@ -411,7 +427,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
 template <int NB, int QUADS>
 int launch_bcq_mfma(const LutArgs& a, hipStream_t stream) {
   constexpr int WAVES = 8;
-  const size_t smem = (size_t)WAVES * QUADS * 512 + (size_t)WAVES * 4 * 64 * 4;
+  const size_t smem = (size_t)WAVES * QUADS * kQuadBytes + (size_t)WAVES * 5 * 64 * 4;
   const int ntiles = a.N / 64;
   if (a.qbias)
     hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, true>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
