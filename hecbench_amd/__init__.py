@@ -13,6 +13,7 @@ from .ops import (
     dequant_4bit, quantize_dynamic8, lut_matmul, code1x16_matvec,
     device_info, init, q3_pack, bcq_pack, quantize_4bit,
     static_scaled_int8_quant, dynamic_scaled_int8_quant,
+    gemv_fp16, gemv_int8, gemv_int4, mxfp4_qdq,
 )
 
 __all__ = [
@@ -21,4 +22,5 @@ __all__ = [
     "dequant_4bit", "quantize_dynamic8", "lut_matmul", "code1x16_matvec",
     "device_info", "init", "q3_pack", "bcq_pack", "quantize_4bit",
     "static_scaled_int8_quant", "dynamic_scaled_int8_quant",
+    "gemv_fp16", "gemv_int8", "gemv_int4", "mxfp4_qdq",
 ]

@@ -35,6 +35,12 @@ _SIGNATURES = {
                                         _c.c_int, _c.c_int32, _c.c_void_p]),
     "hq_int8_quant_dynamic": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64,
                                          _c.c_int, _c.c_void_p]),
+    "hq_gemv_fp16": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int, _c.c_void_p]),
+    "hq_gemv_int8": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int, _c.c_float,
+                                _c.c_float, _c.c_void_p]),
+    "hq_gemv_int4": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int, _c.c_float,
+                                _c.c_float, _c.c_void_p]),
+    "hq_mxfp4_qdq": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

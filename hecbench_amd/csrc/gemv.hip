@@ -1,0 +1,196 @@
+// Dense and weight-quantised matrix-vector products for gfx950 (fp16 vector, fp16 result):
+//
+//   fp16 : res[r] = f16( sum_j mat[r][j] * vec[j] )
+//   int8 : res[r] = f16( scale * sum_j (mat[r][j] - zp) * vec[j] ),  mat int8
+//   int4 : res[r] = f16( scale * sum_j (nib[r][j] - zp) * vec[j] ),  two codes per byte, code j in the
+//          low nibble of byte j/2 for even j and in the high nibble for odd j
+//
+// Replaces gemv_fp16 / gemv_quantized_int8 / gemv_quantized_int4 and their launchers
+// (src/gemv-hip/kernels.h:66-311, src/gemv-hip/gemv.cu:10-133 in the HeCBench tree).  Like
+// the reference, scale and zero point are rounded to fp16 before use and sums are kept in
+// fp32; unlike it, the zero point is taken out once per row ( sum (q - zp) v = sum q v -
+// zp sum v ), which leaves a sign-extending conversion and one fused multiply-add per int8 weight and
+// 11 instructions per 8 int4 weights.
+//
+// A wave owns R consecutive rows and walks the columns in steps of 64 lanes x 16 bytes of
+// matrix per row (1 KB contiguous per wave and row); the matching piece of the vector is
+// loaded once and used for the R rows.  A 4-bit code left in place in the low bits of
+// a 16-bit half is the fp16 subnormal code * 2^-24, so `word >> 4i & 0x000f000f` is a pair
+// of operands for a two-term fp16 dot product with fp32 accumulation (exact products).
+// Lanes are combined with DPP butterflies; one rounding to fp16 at the end.
+#include "hq_internal.h"
+
+namespace {
+
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ h2v as_h2(uint32_t v) { return __builtin_bit_cast(h2v, v); }
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_f(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f<0x141>(v);  // row_half_mirror
+  v += dpp_f<0x140>(v);  // row_mirror
+  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
+}
+
+enum { kF16 = 0, kI8 = 1, kI4 = 2 };
+
+struct GemvArgs {
+  const char* mat;
+  const u4v* vec;  // fp16, 16-byte units
+  _Float16* res;
+  int rows, n;
+  float scale, zp;  // already rounded to fp16 precision
+};
+
+template <int MODE> struct Geom;
+template <> struct Geom<kF16> { static constexpr int kPerUnit = 8, kVecUnits = 1; };   // weights per 16-byte unit
+template <> struct Geom<kI8> { static constexpr int kPerUnit = 16, kVecUnits = 2; };
+template <> struct Geom<kI4> { static constexpr int kPerUnit = 32, kVecUnits = 4; };
+
+// Sum of the sixteen-byte vector piece (eight halves) in fp32.
+__device__ __forceinline__ float sum8(u4v v, float acc) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  const h2v one = {(_Float16)1.f, (_Float16)1.f};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_fdot2(as_h2(w[i]), one, acc, false);
+  return acc;
+}
+
+template <int MODE, int R>
+__global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
+  using G = Geom<MODE>;
+  const int lane = threadIdx.x & 63;
+  const int wave = (blockIdx.x * 256 + threadIdx.x) >> 6;
+  const int row0 = wave * R;
+  if (row0 >= a.rows) return;  // wave-uniform
+  const int units = a.n / G::kPerUnit;  // 16-byte units per matrix row
+  const size_t row_bytes = (size_t)units * 16;
+  const u4v* rowp[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    rowp[r] = reinterpret_cast<const u4v*>(a.mat + (size_t)min(row0 + r, a.rows - 1) * row_bytes);
+
+  float acc[R], vsum = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.f;
+
+  for (int u = lane; u < units; u += 64) {
+    u4v m[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) m[r] = __builtin_nontemporal_load(rowp[r] + u);
+    u4v v[G::kVecUnits];
+#pragma unroll
+    for (int i = 0; i < G::kVecUnits; ++i) v[i] = a.vec[(size_t)u * G::kVecUnits + i];
+    uint32_t vw[4 * G::kVecUnits];
+#pragma unroll
+    for (int i = 0; i < G::kVecUnits; ++i) { vw[4 * i] = v[i].x; vw[4 * i + 1] = v[i].y; vw[4 * i + 2] = v[i].z; vw[4 * i + 3] = v[i].w; }
+
+    if (MODE == kF16) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const uint32_t mw[4] = {m[r].x, m[r].y, m[r].z, m[r].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[r] = __builtin_amdgcn_fdot2(as_h2(mw[i]), as_h2(vw[i]), acc[r], false);
+      }
+    } else if (MODE == kI8) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) vsum = sum8(v[i], vsum);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const uint32_t mw[4] = {m[r].x, m[r].y, m[r].z, m[r].w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          // bytes 0..3 of word d are columns 4d..4d+3: vector halves vw[2d].lo, .hi, vw[2d+1].lo, .hi
+          const h2v x01 = as_h2(vw[2 * d]), x23 = as_h2(vw[2 * d + 1]);
+          acc[r] = fmaf((float)x01[0], (float)(int8_t)(mw[d] & 0xffu), acc[r]);
+          acc[r] = fmaf((float)x01[1], (float)(int8_t)((mw[d] >> 8) & 0xffu), acc[r]);
+          acc[r] = fmaf((float)x23[0], (float)(int8_t)((mw[d] >> 16) & 0xffu), acc[r]);
+          acc[r] = fmaf((float)x23[1], (float)(int8_t)(mw[d] >> 24), acc[r]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) vsum = sum8(v[i], vsum);
+      // word d holds columns 8d..8d+7 in nibbles 0..7; `(w >> 4i) & 0x000f000f` pairs columns
+      // i and i+4, so the vector halves are paired the same way once for all rows
+      uint32_t pv[4][4];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        pv[d][0] = __builtin_amdgcn_perm(vw[4 * d + 2], vw[4 * d], 0x05040100u);      // v0 v4
+        pv[d][1] = __builtin_amdgcn_perm(vw[4 * d + 2], vw[4 * d], 0x07060302u);      // v1 v5
+        pv[d][2] = __builtin_amdgcn_perm(vw[4 * d + 3], vw[4 * d + 1], 0x05040100u);  // v2 v6
+        pv[d][3] = __builtin_amdgcn_perm(vw[4 * d + 3], vw[4 * d + 1], 0x07060302u);  // v3 v7
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const uint32_t mw[4] = {m[r].x, m[r].y, m[r].z, m[r].w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[r] = __builtin_amdgcn_fdot2(as_h2((mw[d] >> (4 * i)) & 0x000f000fu), as_h2(pv[d][i]), acc[r], false);
+      }
+    }
+  }
+
+  const float vs = MODE == kF16 ? 0.f : wave_sum(vsum);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float s = wave_sum(acc[r]);
+    if (MODE == kI8) s = a.scale * (s - a.zp * vs);
+    if (MODE == kI4) s = a.scale * (s * 16777216.f - a.zp * vs);  // codes were fp16 subnormals code * 2^-24
+    if (lane == 0 && row0 + r < a.rows) a.res[row0 + r] = (_Float16)s;
+  }
+}
+
+template <int MODE>
+int launch_gemv(const void* mat, const void* vec, void* res, int rows, int n, float scale, float zp,
+                hipStream_t stream) {
+  if (!mat || !vec || !res) return HQ_ERR_NULL_POINTER;
+  if (rows <= 0 || n <= 0 || (n % Geom<MODE>::kPerUnit)) return HQ_ERR_BAD_SHAPE;
+  if (((uintptr_t)mat & 15) || ((uintptr_t)vec & 15) || ((uintptr_t)res & 1)) return HQ_ERR_MISALIGNED;
+  const HqDevice* dev = nullptr;
+  int rc = hq_current_device(&dev);
+  if (rc != HQ_OK) return rc;
+  GemvArgs a;
+  a.mat = reinterpret_cast<const char*>(mat);
+  a.vec = reinterpret_cast<const u4v*>(vec);
+  a.res = reinterpret_cast<_Float16*>(res);
+  a.rows = rows; a.n = n;
+  a.scale = (float)(_Float16)scale;  // the reference rounds both to fp16 (src/gemv-hip/gemv.cu:18-19)
+  a.zp = (float)(_Float16)zp;
+  // several rows per wave (the vector piece is loaded and prepared once for them) once there are
+  // enough rows to fill the chip with such waves
+  constexpr int RMAX = MODE == kI4 ? 4 : 2;
+  if (rows >= dev->cus * 16 * RMAX) {
+    const int waves = (rows + RMAX - 1) / RMAX;
+    hipLaunchKernelGGL((gemv_kernel<MODE, RMAX>), dim3((waves + 3) / 4), dim3(256), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((gemv_kernel<MODE, 1>), dim3((rows + 3) / 4), dim3(256), 0, stream, a);
+  }
+  return hq_launch_status();
+}
+
+}  // namespace
+
+extern "C" int hq_gemv_fp16(const void* mat, const void* vec, void* res, int rows, int n, void* stream) {
+  return launch_gemv<kF16>(mat, vec, res, rows, n, 1.f, 0.f, (hipStream_t)stream);
+}
+extern "C" int hq_gemv_int8(const int8_t* mat, const void* vec, void* res, int rows, int n, float scale,
+                            float zero_point, void* stream) {
+  return launch_gemv<kI8>(mat, vec, res, rows, n, scale, zero_point, (hipStream_t)stream);
+}
+extern "C" int hq_gemv_int4(const uint8_t* mat, const void* vec, void* res, int rows, int n, float scale,
+                            float zero_point, void* stream) {
+  return launch_gemv<kI4>(mat, vec, res, rows, n, scale, zero_point, (hipStream_t)stream);
+}

@@ -196,3 +196,52 @@ def dynamic_scaled_int8_quant(x, with_azp=False, out=None):
                                            _stream())
     _lib.check(rc, "hq_int8_quant_dynamic")
     return out, scales, azp
+
+
+def gemv_fp16(mat, vec, out=None):
+    """solve_gemv_with_params of src/gemv-hip/gemv.cu:94-133: res = mat @ vec (fp16 in, fp32 sums, fp16 out)."""
+    _dev(mat, vec, out)
+    rows, n = mat.shape
+    if out is None:
+        out = torch.empty(rows, dtype=torch.float16, device=mat.device)
+    rc = _lib.load().hq_gemv_fp16(_ptr(mat), _ptr(vec), _ptr(out), rows, n, _stream())
+    _lib.check(rc, "hq_gemv_fp16")
+    return out
+
+
+def gemv_int8(mat, vec, scale, zero_point, out=None):
+    """solve_gemv_int8_quantized_with_params of src/gemv-hip/gemv.cu:52-92 (mat int8 [rows][n])."""
+    _dev(mat, vec, out)
+    rows, n = mat.shape
+    if out is None:
+        out = torch.empty(rows, dtype=torch.float16, device=mat.device)
+    rc = _lib.load().hq_gemv_int8(_ptr(mat), _ptr(vec), _ptr(out), rows, n, float(scale), float(zero_point),
+                                  _stream())
+    _lib.check(rc, "hq_gemv_int8")
+    return out
+
+
+def gemv_int4(mat, vec, scale, zero_point, out=None):
+    """solve_gemv_int4_quantized_with_params of src/gemv-hip/gemv.cu:10-50 (mat uint8 [rows][n/2], low nibble
+    first)."""
+    _dev(mat, vec, out)
+    rows, half_n = mat.shape
+    if out is None:
+        out = torch.empty(rows, dtype=torch.float16, device=mat.device)
+    rc = _lib.load().hq_gemv_int4(_ptr(mat), _ptr(vec), _ptr(out), rows, 2 * half_n, float(scale),
+                                  float(zero_point), _stream())
+    _lib.check(rc, "hq_gemv_int4")
+    return out
+
+
+def mxfp4_qdq(x, out=None):
+    """mxfp4<T>() of src/mxfp4-hip/main.cu:144-171: microscaling fp4 quantise-dequantise of an fp16 / bf16 tensor
+    whose element count is a multiple of 32."""
+    _dev(x, out)
+    if x.dtype not in (torch.float16, torch.bfloat16):
+        raise TypeError("mxfp4_qdq takes fp16 or bf16 tensors")
+    if out is None:
+        out = torch.empty_like(x)
+    rc = _lib.load().hq_mxfp4_qdq(_ptr(x), _ptr(out), x.numel(), 1 if x.dtype == torch.float16 else 2, _stream())
+    _lib.check(rc, "hq_mxfp4_qdq")
+    return out

@@ -41,7 +41,7 @@ extern "C" {
 /* element types of the activation vector / matrix */
 #define HQ_DTYPE_F32 0
 #define HQ_DTYPE_F16 1
-#define HQ_DTYPE_BF16 2 /* accepted by the activation quantisers only */
+#define HQ_DTYPE_BF16 2 /* accepted by the activation quantisers and hq_mxfp4_qdq only */
 
 /* flags */
 #define HQ_FLAG_ACCUMULATE 1u /* y += result (reference wrapper semantics) */
@@ -171,6 +171,36 @@ int hq_int8_quant_static(const void* x, int x_dtype, int8_t* out, int64_t num_to
                          float scale, int has_azp, int32_t azp, void* stream);
 int hq_int8_quant_dynamic(const void* x, int x_dtype, int8_t* out, float* scales, int32_t* azp,
                           int64_t num_tokens, int hidden_size, void* stream);
+
+/*
+ * Dense / weight-quantised matrix-vector products with an fp16 vector and fp16 result
+ * (mat is [rows][n] row-major, sums in fp32, one rounding to fp16):
+ *   hq_gemv_fp16: res[r] = sum_j mat[r][j] * vec[j]                     mat fp16;  n % 8 == 0
+ *   hq_gemv_int8: res[r] = scale * sum_j (mat[r][j] - zero_point) * vec[j]   mat int8;  n % 16 == 0
+ *   hq_gemv_int4: the same with 4-bit unsigned codes, two per byte: column j is the low nibble
+ *                 of byte j/2 for even j, the high nibble for odd j;  n % 32 == 0
+ * scale and zero_point are rounded to fp16 first, as the reference launchers do.  mat and vec
+ * 16-byte aligned.  Replace solve_gemv_with_params / solve_gemv_int8_quantized_with_params /
+ * solve_gemv_int4_quantized_with_params, src/gemv-hip/gemv.cu:10-133 (kernels
+ * src/gemv-hip/kernels.h:66-311); the reference's block_dim_x/block_dim_y tuning arguments have no
+ * counterpart (the launch shape is chosen from the CU count).
+ */
+int hq_gemv_fp16(const void* mat_fp16, const void* vec_fp16, void* res_fp16, int rows, int n, void* stream);
+int hq_gemv_int8(const int8_t* mat, const void* vec_fp16, void* res_fp16, int rows, int n, float scale,
+                 float zero_point, void* stream);
+int hq_gemv_int4(const uint8_t* mat_packed, const void* vec_fp16, void* res_fp16, int rows, int n, float scale,
+                 float zero_point, void* stream);
+
+/*
+ * Microscaling fp4 quantise-dequantise: groups of 32 consecutive elements share the scale
+ * 2^(e-2), 2^e being the group's largest magnitude rounded to a power of two (carry at a
+ * mantissa of 0.75); out = scale * e2m1(in / scale) with round-to-nearest-even onto
+ * {0, .5, 1, 1.5, 2, 3, 4, 6} and saturation.  dtype HQ_DTYPE_F16 or HQ_DTYPE_BF16; n_elems a
+ * multiple of 32; 16-byte aligned pointers; in and out must not overlap.  Bit-exact with the reference
+ * kernel for finite data.  Replaces mxfp4<T>(y, a, numel, niters), src/mxfp4-hip/main.cu:144-171
+ * (kernel main.cu:109-142), without its timing loop and printing.
+ */
+int hq_mxfp4_qdq(const void* in, void* out, int64_t n_elems, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

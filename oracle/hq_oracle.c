@@ -591,3 +591,93 @@ void hqo_aqlm_matvec(const int16_t* codes, const uint16_t* codebooks,
     }
   }
 }
+
+/* ------------------------------------------------------------------ gemv */
+
+/* src/gemv-hip/kernels.h:66-311 (kernels) and src/gemv-hip/gemv.cu:134-190 (the reference's own
+ * statement of the result: sum of (q - zero_point) * scale * vec).  scale and zero_point are
+ * rounded to fp16 first (gemv.cu:18-19); the sum is taken in double. */
+void hqo_gemv(const void* mat, int mode, const uint16_t* vec, uint16_t* res_f16, double* res_f64,
+              int rows, int n, float scale, float zero_point) {
+  const double sc = mode ? (double)hqo_f16_to_f32(hqo_f32_to_f16(scale)) : 1.0;
+  const double zp = mode ? (double)hqo_f16_to_f32(hqo_f32_to_f16(zero_point)) : 0.0;
+  for (int r = 0; r < rows; ++r) {
+    double s = 0.0;
+    for (int j = 0; j < n; ++j) {
+      double q;
+      if (mode == 0) q = (double)hqo_f16_to_f32(((const uint16_t*)mat)[(size_t)r * n + j]);
+      else if (mode == 1) q = (double)((const int8_t*)mat)[(size_t)r * n + j];
+      else {
+        const uint8_t b = ((const uint8_t*)mat)[(size_t)r * (n / 2) + j / 2];
+        q = (double)((j & 1) ? (b >> 4) : (b & 15)); /* kernels.h:15-21: X = low nibble pairs with vec[2j] */
+      }
+      s += (q - zp) * (double)hqo_f16_to_f32(vec[j]);
+    }
+    s *= sc;
+    if (res_f64) res_f64[r] = s;
+    if (res_f16) res_f16[r] = hqo_f64_to_f16(s);
+  }
+}
+
+/* ----------------------------------------------------------------- mxfp4 */
+
+static uint16_t f32_to_bf16(float f) { /* round to nearest even */
+  uint32_t b;
+  memcpy(&b, &f, 4);
+  if ((b & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((b >> 16) | 0x40u);
+  b += 0x7fffu + ((b >> 16) & 1u);
+  return (uint16_t)(b >> 16);
+}
+static float bf16_to_f32(uint16_t h) {
+  uint32_t b = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &b, 4);
+  return f;
+}
+
+/* Nearest e2m1 value (0, .5, 1, 1.5, 2, 3, 4, 6), ties to the even mantissa, saturating at 6:
+ * what fp16_to_fp4_simulate (src/mxfp4-hip/main.cu:19-107) produces for finite inputs. */
+static float round_to_e2m1(float a) {
+  float m = fabsf(a), r;
+  if (m < 2.f) r = nearbyintf(m * 2.f) * 0.5f;
+  else if (m < 4.f) r = nearbyintf(m);
+  else r = fminf(nearbyintf(m * 0.5f) * 2.f, 6.f);
+  return copysignf(r, a);
+}
+
+/* Microscaling fp4 quantise-dequantise in place of qdq_mxfp4_kernel, src/mxfp4-hip/main.cu:109-142:
+ * per group of 32: the largest magnitude, rounded to a power of two with the carry at a mantissa
+ * of 0.75 (main.cu:124-126), gives the shared scale 2^(e-2) clamped to the E8M0 range
+ * (main.cu:128-132); every element is divided by it, rounded to e2m1 and multiplied back
+ * (main.cu:134-141).  Groups whose rounded maximum is zero give zeros (the reference divides by a
+ * zero scale there). */
+void hqo_mxfp4_qdq(const uint16_t* in, uint16_t* out, int64_t n, int is_bf16) {
+  const int mant = is_bf16 ? 7 : 10;
+  for (int64_t g = 0; g + 32 <= n; g += 32) {
+    uint16_t mx = 0;
+    for (int i = 0; i < 32; ++i) {
+      uint16_t a = in[g + i] & 0x7fffu;
+      if (a > mx) mx = a; /* magnitudes of one format order like their bit patterns */
+    }
+    const uint16_t rounded = (uint16_t)((mx + (1u << (mant - 2))) & (0xffffu << mant) & 0x7fffu);
+    const float bmax = is_bf16 ? bf16_to_f32(rounded) : hqo_f16_to_f32(rounded);
+    if (!(bmax > 0.f)) {
+      for (int i = 0; i < 32; ++i) out[g + i] = (uint16_t)(in[g + i] & 0x8000u);
+      continue;
+    }
+    int e;
+    frexpf(bmax, &e); /* bmax = 0.5 * 2^e exactly */
+    e -= 1;
+    int scale_exp = 127 + (e - 2 < 127 ? e - 2 : 127);
+    if (scale_exp < 0) scale_exp = 0;
+    float scale = ldexpf(1.f, scale_exp - 127);
+    scale = is_bf16 ? bf16_to_f32(f32_to_bf16(scale)) : hqo_f16_to_f32(hqo_f32_to_f16(scale));
+    for (int i = 0; i < 32; ++i) {
+      const float x = is_bf16 ? bf16_to_f32(in[g + i]) : hqo_f16_to_f32(in[g + i]);
+      const float q = x / scale; /* then rounded to the storage type, as __hdiv does */
+      const float qs = is_bf16 ? bf16_to_f32(f32_to_bf16(q)) : hqo_f16_to_f32(hqo_f32_to_f16(q));
+      const float r = round_to_e2m1(qs) * scale;
+      out[g + i] = is_bf16 ? f32_to_bf16(r) : hqo_f32_to_f16(r);
+    }
+  }
+}

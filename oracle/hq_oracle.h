@@ -27,6 +27,12 @@
  *   int8 activation quant   : pinned by the reference host loops compiled into
  *                             oracle/_ref (src/quantVLLM-cuda/reference.h)
  *   4-bit blockwise quantize: PARITY UNPINNED (no counterpart in the reference)
+ *   gemv fp16 / int8 / int4 : the reference's own statement of the result is its device-side
+ *                             checker (src/gemv-hip/gemv.cu:134-190); pinned by closed forms and,
+ *                             on a GPU, by the reference kernels compiled into oracle/_ref
+ *   mxfp4 quantise-dequantise: pinned by the reference's verification table
+ *                             (src/mxfp4-cuda/verify.h) and, on a GPU, by the reference kernel
+ *                             compiled into oracle/_ref
  */
 #ifndef HQ_ORACLE_H
 #define HQ_ORACLE_H
@@ -139,6 +145,17 @@ void hqo_aqlm_matvec(const int16_t* codes, const uint16_t* codebooks_f16,
                      const uint16_t* scales_f16, const uint16_t* x_f16,
                      uint16_t* y_f16, double* y_f64 /*nullable*/, int M, int K,
                      const int cb_a_sizes[4], int cb_stride_int4, int mode);
+
+/* ---- gemv (src/gemv-hip) --------------------------------------------------- */
+/* mode 0: mat fp16 [rows][n]; 1: int8 [rows][n]; 2: 4-bit codes, uint8 [rows][n/2], column j in the
+ * low nibble of byte j/2 for even j.  res = scale * sum_j (q - zero_point) * vec[j] in double with
+ * scale/zero_point rounded to fp16 first (ignored for mode 0); res_f16 / res_f64 may be NULL. */
+void hqo_gemv(const void* mat, int mode, const uint16_t* vec_f16, uint16_t* res_f16, double* res_f64,
+              int rows, int n, float scale, float zero_point);
+
+/* ---- mxfp4 quantise-dequantise (src/mxfp4-hip/main.cu:19-142) ---------------- */
+/* in/out: fp16 or bf16 bit patterns, n a multiple of 32 (groups of 32 share a power-of-two scale). */
+void hqo_mxfp4_qdq(const uint16_t* in, uint16_t* out, int64_t n, int is_bf16);
 
 #ifdef __cplusplus
 }

@@ -140,6 +140,27 @@ class Oracle:
                                         int(x.shape[1]))
         return out, scales, azp
 
+    # ---- gemv
+    def gemv(self, mat, mode, vec16, scale=1.0, zero_point=0.0):
+        """mode 0 fp16 / 1 int8 / 2 packed int4; returns (fp16 result, double result)."""
+        rows = mat.shape[0]
+        n = vec16.size
+        mat = np.ascontiguousarray(mat)
+        r16 = np.zeros(rows, np.uint16)
+        r64 = np.zeros(rows, np.float64)
+        mp = mat.view(np.uint16) if mode == 0 else mat
+        self.lib.hqo_gemv(_p(mp), mode, _p(vec16.view(np.uint16)), _p(r16), _p(r64), rows, n,
+                          ctypes.c_float(scale), ctypes.c_float(zero_point))
+        return r16.view(np.float16), r64
+
+    # ---- mxfp4
+    def mxfp4_qdq(self, bits, is_bf16):
+        """bits: uint16 patterns of fp16 / bf16 values; returns the quantise-dequantised patterns."""
+        bits = np.ascontiguousarray(bits, np.uint16)
+        out = np.zeros_like(bits)
+        self.lib.hqo_mxfp4_qdq(_p(bits), _p(out), ctypes.c_int64(bits.size), int(is_bf16))
+        return out
+
     # ---- LUT-GEMM
     def bcq_pack(self, signs):
         K, nb, N = signs.shape

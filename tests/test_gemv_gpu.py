@@ -1,0 +1,107 @@
+"""Parity of the dense / int8 / int4 matrix-vector products with the CPU oracle and, where it was
+built, with the reference kernels themselves (same device buffers), through the C ABI."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from tests import oracle_api as oa
+from tests.test_gemv_mxfp4_cpu import gemv_problem
+
+pytestmark = pytest.mark.gpu
+
+SCALE, ZP = 0.0625, 0.01     # the reference's default -u / -v (src/gemv-hip/main.cu:35-36)
+
+
+def _run(hq, mat, vec, mode):
+    import torch
+    dm = torch.from_numpy(mat).to("cuda:0")
+    dv = torch.from_numpy(vec).to("cuda:0")
+    if mode == 0:
+        out = hq.gemv_fp16(dm, dv)
+    elif mode == 1:
+        out = hq.gemv_int8(dm, dv, SCALE, ZP)
+    else:
+        out = hq.gemv_int4(dm, dv, SCALE, ZP)
+    torch.cuda.synchronize()
+    return out.cpu().numpy(), dm, dv
+
+
+def _check(got16, ref64):
+    # one rounding to fp16 (half an ulp, 2^-11 relative) on top of fp32 sums whose error is a few
+    # 1e-6 of the typical output size
+    got = got16.astype(np.float64)
+    rms = float(np.sqrt(np.mean(ref64 ** 2)))
+    bound = np.abs(ref64) * 2.0 ** -10 + 1e-5 * rms + 2.0 ** -24
+    assert np.all(np.abs(got - ref64) <= bound), float(np.max(np.abs(got - ref64) / bound))
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("rows,n", [(512, 512), (37, 1024), (1, 32), (9000, 2048), (3, 16384), (130, 96), (16390, 64)])
+def test_vs_oracle(hq, oracle, rows, n, mode):
+    mat, vec = gemv_problem(rows + n + mode, rows, n, mode)
+    got, _, _ = _run(hq, mat, vec, mode)
+    _, r64 = oracle.gemv(mat, mode, vec, SCALE, ZP)
+    _check(got, r64)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_signed_data_and_extremes(hq, oracle, mode):
+    """Signed vector entries (cancellation) and the extreme codes -128 / 127 / 0 / 15."""
+    rng = np.random.default_rng(3)
+    rows, n = 64, 4096
+    vec = rng.standard_normal(n).astype(np.float16)
+    if mode == 0:
+        mat = rng.standard_normal((rows, n)).astype(np.float16)
+    elif mode == 1:
+        mat = rng.choice(np.array([-128, 127, 0, 1], np.int8), (rows, n))
+    else:
+        mat = rng.choice(np.array([0x00, 0xFF, 0xF0, 0x0F], np.uint8), (rows, n // 2))
+    got, _, _ = _run(hq, mat, vec, mode)
+    _, r64 = oracle.gemv(mat, mode, vec, SCALE, ZP)
+    # zero-mean sums: error relative to the size of the terms, not of the (cancelled) result
+    dense = np.abs(mat.astype(np.float64)).max() if mode != 2 else 15.0
+    scale = np.sqrt(n) * dense * (SCALE if mode else 1.0)
+    assert np.max(np.abs(got.astype(np.float64) - r64)) <= 2e-3 * scale
+
+
+def test_rejects_bad_arguments(hq):
+    import torch
+    from hecbench_amd import HqError
+    v = torch.zeros(40, dtype=torch.float16, device="cuda:0")
+    with pytest.raises(HqError):
+        hq.gemv_fp16(torch.zeros(4, 36, dtype=torch.float16, device="cuda:0"), v)     # n % 8
+    with pytest.raises(HqError):
+        hq.gemv_int8(torch.zeros(4, 40, dtype=torch.int8, device="cuda:0"), v, 1.0, 0.0)   # n % 16
+    with pytest.raises(HqError):
+        hq.gemv_int4(torch.zeros(4, 20, dtype=torch.uint8, device="cuda:0"), v, 1.0, 0.0)  # n % 32
+
+
+@pytest.mark.parametrize("n,bx,by", [(512, 32, 4), (2048, 128, 8)])
+def test_vs_reference_kernels(hq, oracle, n, bx, by):
+    """The reference's three kernels on the same device buffers, with the launch shapes of its run
+    lines (src/gemv-hip/Makefile:55-57): both sides within the reference's own acceptance band
+    (0.125 * n / 512, gemv.cu:143) of each other and of the exact result."""
+    import torch
+    ref = oa.load_ref_hip()
+    if ref is None or not hasattr(ref, "ref_gemv_fp16"):
+        pytest.skip("oracle/_ref was not built with the gemv kernels")
+    vp = ctypes.c_void_p
+    for mode in (0, 1, 2):
+        mat, vec = gemv_problem(11 * mode + n, n, n, mode)
+        got, dm, dv = _run(hq, mat, vec, mode)
+        res = torch.zeros(n, dtype=torch.float16, device="cuda:0")
+        args = [vp(dm.data_ptr()), vp(dv.data_ptr()), vp(res.data_ptr()), ctypes.c_uint(n)]
+        if mode == 0:
+            ref.ref_gemv_fp16(*args, ctypes.c_uint(bx), ctypes.c_uint(by), None)
+        else:
+            fn = ref.ref_gemv_int8 if mode == 1 else ref.ref_gemv_int4
+            fn(*args, ctypes.c_float(SCALE), ctypes.c_float(ZP), ctypes.c_uint(bx), ctypes.c_uint(by), None)
+        torch.cuda.synchronize()
+        theirs = res.cpu().numpy().astype(np.float64)
+        _, r64 = oracle.gemv(mat, mode, vec, SCALE, ZP)
+        band = 0.125 * n / 512
+        assert np.max(np.abs(theirs - r64)) <= band
+        assert np.max(np.abs(got.astype(np.float64) - theirs)) <= band
+        # and this library is at least as close to the exact result as the reference kernel
+        assert np.max(np.abs(got.astype(np.float64) - r64)) <= np.max(np.abs(theirs - r64)) + 1e-6
