@@ -26,7 +26,7 @@ ROWS = 3 * K // 32
 ALGO_BYTES = ROWS * N * 4 + 2 * N * 4 + K * 4 + N * 4   # weights + scale/zero + x + y = 17,056,768
 # HBM bytes per launch of the matvec kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what
 # the same counter reads for a plain 256 MiB device copy (profiles/q3_matvec_4096x11008.txt).
-Q3_TRAFFIC_BYTES = 17267233
+Q3_TRAFFIC_BYTES = 17267238
 
 
 def _time_loop(fn, n_buffers, steps, warmup):
@@ -180,6 +180,34 @@ def bench_others(steps, warmup):
                                     "frac_hbm": b * st / secs / 1e9 / HBM_PEAK_GBS,
                                     "TFLOPs": fl * st / secs / 1e12,
                                     "frac_mfma_f16": fl * st / secs / 1e12 / MFMA_F16_PEAK_TFLOPS}
+    del mats, Ag, og
+    # next rows: dense / int8 / int4 gemv at the reference's run size 16384 x 16384 (the weight buffers are
+    # rotated so that at least 512 MB of distinct data passes between two uses of a buffer) and mxfp4
+    # quantise-dequantise of 4096 x 4096 fp16 elements (rotate 16 x 67 MB)
+    ng = 16384
+    vg = torch.rand(ng, device=dev, generator=g).half()
+    rg = torch.empty(ng, dtype=torch.float16, device=dev)
+    st = max(50, steps // 8)
+    for name, nbuf, make, call, bytes_per in (
+            ("gemv_fp16_16384", 2, lambda: torch.rand(ng, ng, device=dev, generator=g).half(),
+             lambda m: hq.gemv_fp16(m, vg, out=rg), 2.0),
+            ("gemv_int8_16384", 3, lambda: torch.randint(-128, 128, (ng, ng), dtype=torch.int8, device=dev, generator=g),
+             lambda m: hq.gemv_int8(m, vg, 0.0625, 0.01, out=rg), 1.0),
+            ("gemv_int4_16384", 5, lambda: torch.randint(0, 256, (ng, ng // 2), dtype=torch.uint8, device=dev, generator=g),
+             lambda m: hq.gemv_int4(m, vg, 0.0625, 0.01, out=rg), 0.5)):
+        bufs = [make() for _ in range(nbuf)]
+        secs = _time_loop(lambda i: call(bufs[i]), nbuf, st, 5)
+        b = bytes_per * ng * ng + 4.0 * ng
+        out[name] = {"us": secs / st * 1e6, "GBps": b * st / secs / 1e9, "frac_hbm": b * st / secs / 1e9 / HBM_PEAK_GBS}
+        del bufs
+    nm = 4096 * 4096
+    nb = 16
+    src = [torch.randn(nm, device=dev, generator=g).half() for _ in range(nb)]
+    dst = [torch.empty(nm, dtype=torch.float16, device=dev) for _ in range(nb)]
+    secs = _time_loop(lambda i: hq.mxfp4_qdq(src[i], out=dst[i]), nb, steps, warmup)
+    b = 4.0 * nm
+    out["mxfp4_qdq_4096x4096_f16"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
+                                      "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
     return out
 
 
