@@ -105,8 +105,6 @@ __device__ __forceinline__ void transpose4(uint32_t a, uint32_t b, uint32_t c, u
 }
 
 typedef int v8i __attribute__((ext_vector_type(8)));
-typedef u4v u4v_a4 __attribute__((aligned(4)));
-typedef f4 f4_a4 __attribute__((aligned(4)));
 
 constexpr int kStepBytes = 1536;  // LDS bytes of one step's B operand rows (9 rows of 128 B, padded)
 constexpr int kRedStride = 68;    // floats per (wave, digit) row of the final reduction
@@ -167,13 +165,13 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
       const uint32_t g = (uint32_t)min((r * STEPS + s) * (WAVES * 4) + wv * 4 + xkb, g_count - 1);
       const uint32_t e = g * 32u + (uint32_t)xq * 8u;
       if (XF16) {
-        const u4v raw = *reinterpret_cast<const u4v_a4*>(xbase + e * 2u);
+        const u4v raw = *reinterpret_cast<const u4v*>(xbase + e * 2u);
         const h8 h = __builtin_bit_cast(h8, raw);
 #pragma unroll
         for (int j = 0; j < 8; ++j) xr[p][j] = (float)h[j];
       } else {
-        const f4 lo = *reinterpret_cast<const f4_a4*>(xbase + e * 4u);
-        const f4 hi = *reinterpret_cast<const f4_a4*>(xbase + e * 4u + 16u);
+        const f4 lo = *reinterpret_cast<const f4*>(xbase + e * 4u);
+        const f4 hi = *reinterpret_cast<const f4*>(xbase + e * 4u + 16u);
 #pragma unroll
         for (int j = 0; j < 4; ++j) { xr[p][j] = lo[j]; xr[p][4 + j] = hi[j]; }
       }
@@ -417,7 +415,7 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   if (x_dtype != HQ_DTYPE_F32 && x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
   if (flags & ~HQ_FLAG_ACCUMULATE) return HQ_ERR_BAD_ENUM;
   if (K <= 0 || N <= 0 || batch_M <= 0 || (K & 31) || (N & 3)) return HQ_ERR_BAD_SHAPE;
-  if (((uintptr_t)qweight & 15) || ((uintptr_t)x & (x_dtype == HQ_DTYPE_F16 ? 3 : 7)) ||
+  if (((uintptr_t)qweight & 15) || ((uintptr_t)x & 15) ||  // activations are read with 128-bit loads
       ((uintptr_t)y & 3) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
     return HQ_ERR_MISALIGNED;
   const HqDevice* dev = nullptr;

@@ -97,7 +97,7 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  * the pre-multiplied scale*zero_point.
  *   x        : [batch_M][K] row-major, fp32 (HQ_DTYPE_F32) or fp16 (HQ_DTYPE_F16)
  *   y        : fp32 [batch_M][N]
- *   K % 32 == 0, N % 4 == 0, batch_M >= 1; qweight 16-byte aligned.
+ *   K % 32 == 0, N % 4 == 0, batch_M >= 1; qweight and x 16-byte aligned.
  * Products are accumulated in fp32 for both dtypes (the reference's fp16
  * variant accumulates 16 terms in fp16; this library is never less accurate).
  * batch_M == 1 replaces vecquant3matmul / vecquant3matmul_faster

@@ -47,6 +47,7 @@ def test_argument_validation_needs_no_gpu():
     assert lib.hq_q3_matvec(16, 0, 16, 16, 16, 16, 4096, 11006, 1, 0, None) == -2
     assert lib.hq_q3_matvec(16, 7, 16, 16, 16, 16, 4096, 11008, 1, 0, None) == -3
     assert lib.hq_q3_matvec(16, 0, 20, 16, 16, 16, 4096, 11008, 1, 0, None) == -4
+    assert lib.hq_q3_matvec(24, 0, 16, 16, 16, 16, 4096, 11008, 1, 0, None) == -4   # x: 128-bit loads
     assert lib.hq_dequant_nf4(None, None, None, 64, 64, 0, None) == -1
     assert lib.hq_dequant_nf4(None, None, None, 0, 64, 0, None) == 0
     assert lib.hq_dequant_nf4(16, 16, 16, 64, 63, 0, None) == -2
