@@ -211,6 +211,43 @@ def bench_others(steps, warmup):
     return out
 
 
+def cpu_others():
+    """Serial CPU times of the oracle for the other configurations (one host core; bounded samples, scaled to
+    the full problem where a sample is used).  Reported next to the GPU numbers, never a target."""
+    import numpy as np
+    from tests import oracle_api as oa
+    o = oa.load_oracle()
+    out = {}
+
+    def timed(fn, reps=1):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return (time.perf_counter() - t0) / reps
+
+    packed, absmax = oa.make_nf4_problem(0, 4096 * 4096, 64)
+    out["nf4_dequant_4096x4096"] = {"cpu_us": timed(lambda: o.dequant_4bit(packed, absmax, 4096 * 4096, 64), 3) * 1e6,
+                                    "sample": "3 full calls"}
+    bW, alpha, qb, x = oa.make_lut_problem(0, 4096, 2048, 3, 128)
+    out["lut_gemv_4096x16384_q3"] = {"cpu_us": timed(lambda: o.lut_gemv_f64(bW, alpha, qb, x, 128)) * 8 * 1e6,
+                                     "sample": "2048 of 16384 columns, scaled x8"}
+    codes, cb, sc, xa = oa.make_aqlm_problem(0, 4096, 4096)
+    out["aqlm_4096x4096"] = {"cpu_us": timed(lambda: o.aqlm_matvec(codes, cb, sc, xa, (4096, 0, 0, 0), 65536), 3) * 1e6,
+                             "sample": "3 full calls"}
+    codes, scales, zeros, A = oa.make_q3_problem(0, 8192, 1024, np.float16, batch=4)
+    mat = o.q3_pack(codes)
+    out["q3_gemm_64x8192x28672"] = {"cpu_us": timed(lambda: o.q3_gemm(A, mat, scales, zeros)) * 16 * 28 * 1e6,
+                                    "sample": "4 of 64 rows x 1024 of 28672 columns, scaled x448"}
+    rng = np.random.default_rng(0)
+    m8 = rng.integers(-128, 128, (1024, 16384)).astype(np.int8)
+    v = rng.uniform(0, 1, 16384).astype(np.float16)
+    out["gemv_int8_16384"] = {"cpu_us": timed(lambda: o.gemv(m8, 1, v, 0.0625, 0.01)) * 16 * 1e6,
+                              "sample": "1024 of 16384 rows, scaled x16"}
+    bits = rng.standard_normal(4096 * 4096).astype(np.float16).view(np.uint16)
+    out["mxfp4_qdq_4096x4096_f16"] = {"cpu_us": timed(lambda: o.mxfp4_qdq(bits, False)) * 1e6, "sample": "1 full call"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -265,6 +302,10 @@ def main():
         result["cpu_baseline"] = cpu_baseline_q3(state)
     if args.all:
         result["other_configs"] = bench_others(max(200, args.steps // 8), 50)
+        if not args.no_cpu:
+            for name, cpu in cpu_others().items():
+                result["other_configs"][name]["cpu_serial"] = {"us": round(cpu["cpu_us"], 1), "cores": 1,
+                                                               "kind": "port", "sample": cpu["sample"]}
     print(json.dumps(result))
 
 
