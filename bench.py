@@ -119,17 +119,31 @@ def bench_others(steps, warmup):
     import numpy as np
     import torch
     import hecbench_amd as hq
+    from hecbench_amd import _lib
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev)
     g.manual_seed(99)
     out = {}
+    # raw C-ABI calls with prepared arguments: the Python wrappers cost as much as the short kernels take
+    lib = _lib.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def vp(t):
+        return ctypes.c_void_p(t.data_ptr())
+
+    def check(rc):
+        if rc:
+            raise RuntimeError(lib.hq_strerror(rc).decode())
+
     # config 0: NF4 dequant 4096x4096, blocksize 64 (rotate 14 x 43 MB)
     n = 4096 * 4096
     nb = 14
     packed = [torch.randint(0, 256, (n // 2,), dtype=torch.uint8, device=dev, generator=g) for _ in range(nb)]
     absmax = [torch.empty(n // 64, device=dev).uniform_(0.5, 2.0, generator=g) for _ in range(nb)]
     outs = [torch.empty(n, dtype=torch.float16, device=dev) for _ in range(nb)]
-    secs = _time_loop(lambda i: hq.dequant_4bit(packed[i], absmax[i], n, 64, 0, out=outs[i]), nb, steps, warmup)
+    args = [(vp(packed[i]), vp(absmax[i]), vp(outs[i])) for i in range(nb)]
+    secs = _time_loop(lambda i: check(lib.hq_dequant_nf4(args[i][0], args[i][1], args[i][2], n, 64, 0, stream)),
+                      nb, steps, warmup)
     b = n // 2 + n // 64 * 4 + 64 + n * 2
     out["nf4_dequant_4096x4096"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
                                     "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
@@ -143,7 +157,10 @@ def bench_others(steps, warmup):
     qb = torch.zeros(Kl // 128, Nl, dtype=torch.float16, device=dev)
     xl = torch.randn(Kl, device=dev, generator=g).half()
     yl = torch.empty(Nl, dtype=torch.float16, device=dev)
-    secs = _time_loop(lambda i: hq.lut_matmul(xl, bW[i], alpha[i], qb, 128, out=yl), nb, steps, warmup)
+    args = [(vp(bW[i]), vp(alpha[i])) for i in range(nb)]
+    pq, px, py = vp(qb), vp(xl), vp(yl)
+    secs = _time_loop(lambda i: check(lib.hq_lut_gemv(args[i][0], args[i][1], pq, px, py, Kl, Nl, 3, 128, stream)),
+                      nb, steps, warmup)
     b = Kl // 32 * 3 * Nl * 4 + Kl // 128 * 3 * Nl * 2 + Kl // 128 * Nl * 2 + Kl * 2 + Nl * 2
     out["lut_gemv_4096x16384_q3"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
                                      "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
@@ -157,7 +174,10 @@ def bench_others(steps, warmup):
     sc = torch.empty(Ma, device=dev).uniform_(0.5, 1.5, generator=g).half()
     xa = torch.randn(Ka, device=dev, generator=g).half()
     ya = torch.empty(Ma, dtype=torch.float16, device=dev)
-    secs = _time_loop(lambda i: hq.code1x16_matvec(codes[i], xa, cb, (Ma, 0, 0, 0), 65536, scales=sc, out=ya),
+    args = [vp(c) for c in codes]
+    pcb, psc, pxa, pya = vp(cb), vp(sc), vp(xa), vp(ya)
+    sizes = (ctypes.c_int * 4)(Ma, 0, 0, 0)
+    secs = _time_loop(lambda i: check(lib.hq_aqlm_matvec(args[i], pcb, psc, pxa, pya, Ma, Ka, sizes, 65536, stream)),
                       nb, steps, warmup)
     b = Ma * Ka // 8 * 2 + 65536 * 16 + 3 * Ka * 2
     out["aqlm_4096x4096"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,

@@ -56,8 +56,13 @@ def main():
             ref.ref_vecquant3matmul_faster(vp(x16), vp(mats[it[0] % nbuf]), vp(y), vp(s), vp(z), rows, N)
             it[0] += 1
 
+        lib = hq._lib.load()  # raw C-ABI calls with prepared arguments: a Python wrapper would cost more
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)  # than these kernels take
+        pm = [vp(m) for m in mats]
+        px, ps, pz, py = vp(x), vp(s), vp(z), vp(y)
+
         def ours():
-            hq.q3_matvec(x, mats[it[0] % nbuf], s, z, out=y)
+            lib.hq_q3_matvec(px, 0, pm[it[0] % nbuf], ps, pz, py, K, N, 1, 0, stream)
             it[0] += 1
 
         n = 300 if K > 8192 else 2000
@@ -72,7 +77,7 @@ def main():
     y16 = torch.zeros(N, dtype=torch.float16, device=dev)
     print(f"LUT-GEMM K={K} N={N} q=3 (hot cache): reference matmul() "
           f"{timeit(lambda: ref.ref_lut_matmul(vp(y16), vp(x16), vp(bW), vp(al), vp(qb), K, N, nb, K // G), 300):.2f} us, "
-          f"libhq {timeit(lambda: hq.lut_matmul(x16, bW, al, qb, G, out=y16), 300):.2f} us")
+          f"libhq {timeit(lambda: lib.hq_lut_gemv(vp(bW), vp(al), vp(qb), vp(x16), vp(y16), K, N, nb, G, stream), 300):.2f} us")
     # AQLM, reference problem
     M, K = 12288, 4096
     codes = torch.randint(-32768, 32768, (M, K // 8), dtype=torch.int16, device=dev, generator=g)
@@ -92,6 +97,33 @@ def main():
     print(f"kQuantize n={n}: reference kernel "
           f"{timeit(lambda: ref.ref_kquantize(vp(code), vp(A), vp(out), ctypes.c_long(n), None), 50):.2f} us, "
           f"libhq {timeit(lambda: hq.quantize_dynamic8(code, A, out=out), 50):.2f} us")
+    # gemv at the reference's run size and launch shape (src/gemv-hip/Makefile:55)
+    n = 16384
+    vec = torch.rand(n, device=dev, generator=g).half()
+    res = torch.zeros(n, dtype=torch.float16, device=dev)
+    cu, cf = ctypes.c_uint, ctypes.c_float
+    m16 = torch.rand(n, n, device=dev, generator=g).half()
+    print(f"gemv fp16 {n}: reference kernel (512,2) "
+          f"{timeit(lambda: ref.ref_gemv_fp16(vp(m16), vp(vec), vp(res), cu(n), cu(512), cu(2), None), 50):.1f} us, "
+          f"libhq {timeit(lambda: hq.gemv_fp16(m16, vec, out=res), 50):.1f} us")
+    del m16
+    m8 = torch.randint(-128, 128, (n, n), dtype=torch.int8, device=dev, generator=g)
+    print(f"gemv int8 {n}: reference kernel (512,2) "
+          f"{timeit(lambda: ref.ref_gemv_int8(vp(m8), vp(vec), vp(res), cu(n), cf(0.0625), cf(0.01), cu(512), cu(2), None), 50):.1f} us, "
+          f"libhq {timeit(lambda: hq.gemv_int8(m8, vec, 0.0625, 0.01, out=res), 50):.1f} us")
+    del m8
+    m4 = torch.randint(0, 256, (n, n // 2), dtype=torch.uint8, device=dev, generator=g)
+    print(f"gemv int4 {n}: reference kernel (512,2) "
+          f"{timeit(lambda: ref.ref_gemv_int4(vp(m4), vp(vec), vp(res), cu(n), cf(0.0625), cf(0.01), cu(512), cu(2), None), 50):.1f} us, "
+          f"libhq {timeit(lambda: hq.gemv_int4(m4, vec, 0.0625, 0.01, out=res), 50):.1f} us")
+    del m4
+    # mxfp4 quantise-dequantise, 2^28 fp16 elements (beyond the Infinity Cache)
+    nel = 1 << 28
+    src = torch.randn(nel, device=dev, generator=g).half()
+    dst = torch.empty_like(src)
+    print(f"mxfp4 fp16 n={nel}: reference kernel "
+          f"{timeit(lambda: ref.ref_mxfp4_qdq(vp(src), vp(dst), ctypes.c_int(nel), ctypes.c_int(0), None), 20):.1f} us, "
+          f"libhq {timeit(lambda: hq.mxfp4_qdq(src, out=dst), 20):.1f} us")
 
 
 if __name__ == "__main__":
