@@ -34,56 +34,76 @@ __device__ __forceinline__ float round_to_e2m1(float m) {
   return m < 2.f ? lo : (m < 4.f ? mid : hi);
 }
 
+// Quantise-dequantise of one lane's 8 elements (4 words); `mx` is the lane's largest magnitude on
+// entry and is completed over the group's four lanes here.
+template <bool BF16>
+__device__ __forceinline__ u4v qdq_unit(const u4v raw) {
+  constexpr int MANT = BF16 ? 7 : 10;
+  constexpr int BIAS = BF16 ? 127 : 15;
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  uint32_t mx = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) mx = max(mx, max(w[i] & 0x7fffu, (w[i] >> 16) & 0x7fffu));
+  mx = max(mx, dpp_u<0xB1>(mx));  // quad_perm [1,0,3,2]
+  mx = max(mx, dpp_u<0x4E>(mx));  // quad_perm [2,3,0,1]
+  const uint32_t rounded = (mx + (1u << (MANT - 2))) & (0xffffu << MANT) & 0x7fffu;
+  const int e = (int)(rounded >> MANT) - BIAS;
+  const int scale_exp = max(0, 127 + min(e - 2, 127));  // E8M0 code of the scale
+  // 2^(scale_exp - 127) and its reciprocal; code 0 is 2^-127, an fp32 subnormal
+  const float scale = scale_exp > 0 ? __uint_as_float((uint32_t)scale_exp << 23) : __uint_as_float(0x00400000u);
+  const float inv = scale_exp == 0 ? 1.7014118346046923e38f
+                                   : (scale_exp < 254 ? __uint_as_float((uint32_t)(254 - scale_exp) << 23)
+                                                      : __uint_as_float(0x00400000u));
+  uint32_t o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    // magnitudes only: the sign bits are copied over at the end (a multiply fused with the
+    // conversion would turn -0 into +0)
+    float x0, x1;
+    if (BF16) {
+      x0 = __uint_as_float((w[i] << 16) & 0x7fff0000u);
+      x1 = __uint_as_float(w[i] & 0x7fff0000u);
+    } else {
+      x0 = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] & 0x7fffu));
+      x1 = (float)__builtin_bit_cast(_Float16, (uint16_t)((w[i] >> 16) & 0x7fffu));
+    }
+    const float r0 = round_to_e2m1(x0 * inv) * scale, r1 = round_to_e2m1(x1 * inv) * scale;
+    uint32_t mag;
+    if (rounded == 0) {
+      mag = 0;
+    } else if (BF16) {
+      mag = (__float_as_uint(r0) >> 16) | (__float_as_uint(r1) & 0xffff0000u);  // exact: two mantissa bits
+    } else {
+      mag = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)r0) |
+            ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)r1) << 16);
+    }
+    o[i] = mag | (w[i] & 0x80008000u);
+  }
+  const u4v res = {o[0], o[1], o[2], o[3]};
+  return res;
+}
+
+constexpr int kUnroll = 4;  // 16-byte units per thread and trip, all loaded before the first is used
+
+// units is a multiple of 4, and a thread's units are 256 apart, so the four lanes of a group are
+// in range or out of range together and the quad permutes never read an idle lane's data.
 template <bool BF16>
 __global__ __launch_bounds__(256) void mxfp4_qdq_kernel(const u4v* __restrict__ in, u4v* __restrict__ out,
                                                        int64_t units) {
-  constexpr int MANT = BF16 ? 7 : 10;
-  constexpr int BIAS = BF16 ? 127 : 15;
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < units; u += stride) {
-    const u4v raw = in[u];
-    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-    uint32_t mx = 0;
+  const int64_t stride = (int64_t)gridDim.x * 256 * kUnroll;
+  for (int64_t base = (int64_t)blockIdx.x * 256 * kUnroll + threadIdx.x; base < units; base += stride) {
+    u4v raw[kUnroll];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) mx = max(mx, max(w[i] & 0x7fffu, (w[i] >> 16) & 0x7fffu));
-    // the four lanes of a group (units is a multiple of 4, so a quad is in range as a whole)
-    mx = max(mx, dpp_u<0xB1>(mx));  // quad_perm [1,0,3,2]
-    mx = max(mx, dpp_u<0x4E>(mx));  // quad_perm [2,3,0,1]
-    const uint32_t rounded = (mx + (1u << (MANT - 2))) & (0xffffu << MANT) & 0x7fffu;
-    const int e = (int)(rounded >> MANT) - BIAS;
-    const int scale_exp = max(0, 127 + min(e - 2, 127));  // E8M0 code of the scale
-    // 2^(scale_exp - 127) and its reciprocal; code 0 is 2^-127, an fp32 subnormal
-    const float scale = scale_exp > 0 ? __uint_as_float((uint32_t)scale_exp << 23) : __uint_as_float(0x00400000u);
-    const float inv = scale_exp == 0 ? 1.7014118346046923e38f
-                                     : (scale_exp < 254 ? __uint_as_float((uint32_t)(254 - scale_exp) << 23)
-                                                        : __uint_as_float(0x00400000u));
-    uint32_t o[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      // magnitudes only: the sign bits are copied over at the end (a multiply fused with the
-      // conversion would turn -0 into +0)
-      float x0, x1;
-      if (BF16) {
-        x0 = __uint_as_float((w[i] << 16) & 0x7fff0000u);
-        x1 = __uint_as_float(w[i] & 0x7fff0000u);
-      } else {
-        x0 = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] & 0x7fffu));
-        x1 = (float)__builtin_bit_cast(_Float16, (uint16_t)((w[i] >> 16) & 0x7fffu));
-      }
-      const float r0 = round_to_e2m1(x0 * inv) * scale, r1 = round_to_e2m1(x1 * inv) * scale;
-      uint32_t mag;
-      if (rounded == 0) {
-        mag = 0;
-      } else if (BF16) {
-        mag = (__float_as_uint(r0) >> 16) | (__float_as_uint(r1) & 0xffff0000u);  // exact: two mantissa bits
-      } else {
-        mag = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)r0) |
-              ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)r1) << 16);
-      }
-      o[i] = mag | (w[i] & 0x80008000u);
+    for (int k = 0; k < kUnroll; ++k) {
+      const int64_t u = base + k * 256;
+      raw[k] = in[u < units ? u : base];
     }
-    const u4v res = {o[0], o[1], o[2], o[3]};
-    __builtin_nontemporal_store(res, out + u);
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const int64_t u = base + k * 256;
+      const u4v res = qdq_unit<BF16>(raw[k]);
+      if (u < units) __builtin_nontemporal_store(res, out + u);
+    }
   }
 }
 
@@ -100,7 +120,7 @@ extern "C" int hq_mxfp4_qdq(const void* in, void* out, int64_t n_elems, int dtyp
   int rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
   const int64_t units = n_elems / 8;
-  int64_t blocks = (units + 255) / 256;
+  int64_t blocks = (units + 256 * kUnroll - 1) / (256 * kUnroll);
   const int64_t cap = (int64_t)dev->cus * 32;  // grid-stride beyond that
   if (blocks > cap) blocks = cap;
   if (dtype == HQ_DTYPE_BF16)
