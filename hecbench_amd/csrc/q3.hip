@@ -106,7 +106,8 @@ __device__ __forceinline__ void transpose4(uint32_t a, uint32_t b, uint32_t c, u
 
 typedef int v8i __attribute__((ext_vector_type(8)));
 
-constexpr int kStepBytes = 1536;  // LDS bytes of one step's B operand rows (9 rows of 128 B, padded)
+constexpr int kRowBytes = 144;    // one B operand row (4 lane quarters x 32 B) plus 16 B: rows start 4 banks apart
+constexpr int kStepBytes = 1536;  // LDS bytes of one step's nine B operand rows, padded
 constexpr int kRedStride = 68;    // floats per (wave, digit) row of the final reduction
 // Byte offset of step s inside a wave's digit area: the small skew spreads the four steps one
 // store instruction touches over different LDS banks.
@@ -193,7 +194,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   if (lane < 32) {
 #pragma unroll
     for (int s = 0; s < STEPS; ++s)
-      *reinterpret_cast<uint32_t*>(dig_w + step_off(s) + 8 * 128 + lane * 4) = 0x01010101u;
+      *reinterpret_cast<uint32_t*>(dig_w + step_off(s) + 8 * kRowBytes + lane * 4) = 0x01010101u;
   }
   float run[4][4];  // per-digit sums of all rounds (bias removed, divided by 2^E)
 #pragma unroll
@@ -255,8 +256,8 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int h = 0; h < 2; ++h) {  // h = 0: even elements, h = 1: odd elements (next lane quarter)
-            *reinterpret_cast<uint32_t*>(dst + (2 * i) * 128 + h * 32) = de[h][i];
-            *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * 128 + h * 32) = dd[h][i];
+            *reinterpret_cast<uint32_t*>(dst + (2 * i) * kRowBytes + h * 32) = de[h][i];
+            *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * kRowBytes + h * 32) = dd[h][i];
           }
       }
     }
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     for (int s = 0; s < STEPS; ++s) {
       if ((r * STEPS + s) * (WAVES * 4) + wv * 4 >= g_count) continue;  // wave-uniform
       // MFMA columns 9..15 are never read: they re-use row 8
-      const u4v* bp = reinterpret_cast<const u4v*>(dig_w + step_off(s) + min(c, 8) * 128 + kb * 32);
+      const u4v* bp = reinterpret_cast<const u4v*>(dig_w + step_off(s) + min(c, 8) * kRowBytes + kb * 32);
       const u4v b0 = bp[0], b1 = bp[1];
       const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
 #pragma unroll
