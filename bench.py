@@ -228,6 +228,17 @@ def bench_others(steps, warmup):
     b = 4.0 * nm
     out["mxfp4_qdq_4096x4096_f16"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
                                       "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
+    del src, dst
+    # the quantBnB benchmark's own kernel at its default size: 16,777,216 floats -> 8-bit codes (rotate 8 x 84 MB)
+    nq = 16777216
+    nb = 8
+    code = torch.linspace(-1.0, 1.0, 256, device=dev)  # any sorted 256-entry table costs the same to search
+    As = [torch.randn(nq, device=dev, generator=g) for _ in range(nb)]
+    qs = [torch.empty(nq, dtype=torch.uint8, device=dev) for _ in range(nb)]
+    secs = _time_loop(lambda i: hq.quantize_dynamic8(code, As[i], out=qs[i]), nb, st, 5)
+    b = 5.0 * nq + 1024
+    out["quantize_dynamic8_16777216"] = {"us": secs / st * 1e6, "GBps": b * st / secs / 1e9,
+                                         "frac_hbm": b * st / secs / 1e9 / HBM_PEAK_GBS}
     return out
 
 
@@ -265,6 +276,20 @@ def cpu_others():
                               "sample": "1024 of 16384 rows, scaled x16"}
     bits = rng.standard_normal(4096 * 4096).astype(np.float16).view(np.uint16)
     out["mxfp4_qdq_4096x4096_f16"] = {"cpu_us": timed(lambda: o.mxfp4_qdq(bits, False)) * 1e6, "sample": "1 full call"}
+    # 8-bit quantiser: the reference's own host function where oracle/_ref holds it, else the oracle's restatement
+    A = rng.standard_normal(1 << 21).astype(np.float32)
+    q = np.zeros(A.size, np.uint8)
+    ref = oa.load_ref_cpu()
+    if ref is not None:
+        fn = lambda: ref.ref_dquantize_n(A.ctypes.data_as(ctypes.c_void_p), q.ctypes.data_as(ctypes.c_void_p),
+                                         ctypes.c_long(A.size))
+        kind = "reference"
+    else:
+        code = o.dynamic_map()
+        fn = lambda: o.quantize_dynamic8(code, A)
+        kind = "port"
+    out["quantize_dynamic8_16777216"] = {"cpu_us": timed(fn) * 8 * 1e6, "kind": kind,
+                                         "sample": "2,097,152 of 16,777,216 elements, scaled x8"}
     return out
 
 
@@ -325,7 +350,8 @@ def main():
         if not args.no_cpu:
             for name, cpu in cpu_others().items():
                 result["other_configs"][name]["cpu_serial"] = {"us": round(cpu["cpu_us"], 1), "cores": 1,
-                                                               "kind": "port", "sample": cpu["sample"]}
+                                                               "kind": cpu.get("kind", "port"),
+                                                               "sample": cpu["sample"]}
     print(json.dumps(result))
 
 
