@@ -59,7 +59,7 @@ def test_matvec_f32_vs_oracle(hq, oracle, K, N, seed):
     assert rel_err(y, ref64) <= 1e-4
 
 
-@pytest.mark.parametrize("K,N,seed", [(4096, 11008, 21), (512, 256, 22)])
+@pytest.mark.parametrize("K,N,seed", [(4096, 11008, 21), (512, 256, 22), (32, 4, 23), (160, 132, 24), (8192, 512, 25)])
 def test_matvec_f16_vs_oracle(hq, oracle, K, N, seed):
     codes, scales, zeros, x = oa.make_q3_problem(seed, K, N, x_dtype=np.float16)
     mat = oracle.q3_pack(codes)
