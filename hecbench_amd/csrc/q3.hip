@@ -343,6 +343,8 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
       xsum += wsum[w];
     }
     val = sc_n * (qx * 4096.f) - zr_n * xsum;  // 2^12: fp6 unit 2^-3 times fp8 unit 2^-9
+    val = fmaf(xsum, 0.f, val);  // a NaN or infinity among the activations makes the result NaN (the
+                                 // fixed-point digits cannot carry it)
     if (a.nsplit == 1) {
       a.y[n] = y_old + val;
     } else {

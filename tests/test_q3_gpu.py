@@ -110,6 +110,18 @@ def test_wide_dynamic_range_and_zero_vector(hq, oracle):
     assert (y == 0).all()
 
 
+def test_non_finite_activations_propagate(hq, oracle):
+    K, N = 512, 128
+    codes, scales, zeros, x = oa.make_q3_problem(33, K, N)
+    mat = oracle.q3_pack(codes)
+    for bad in (np.nan, np.inf, -np.inf):
+        xs = x.copy()
+        xs[77] = bad
+        for z in (zeros, np.zeros_like(zeros)):
+            y = _run(hq, xs, mat, scales, z)
+            assert not np.isfinite(y).any(), bad
+
+
 def test_launch_shapes_match(hq, oracle, monkeypatch):
     """Every launch shape (waves per workgroup x steps x K split; one or several
     rounds per workgroup) gives the same answer."""
