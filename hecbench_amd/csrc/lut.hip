@@ -233,6 +233,14 @@ __device__ __forceinline__ float wave_max(float v) {
   return fmaxf(fmaxf(lane_f(v, 0), lane_f(v, 16)), fmaxf(lane_f(v, 32), lane_f(v, 48)));
 }
 
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp_f<0xB1>(v);
+  v += dpp_f<0x4E>(v);
+  v += dpp_f<0x141>(v);
+  v += dpp_f<0x140>(v);
+  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
+}
+
 struct Half16 {  // sixteen fp16 values as two 128-bit loads
   h8 lo, hi;
   __device__ __forceinline__ float get(int i) const { return (float)(i < 8 ? lo[i] : hi[i - 8]); }
@@ -252,6 +260,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
   extern __shared__ float lds[];
   char* xs = reinterpret_cast<char*>(lds);                             // [waves][QUADS][5 rows][4 kb][32 B]
   float* red = reinterpret_cast<float*>(xs + WAVES * QUADS * kQuadBytes);  // [waves][5 columns][64]
+  float* poison_w = red + WAVES * 5 * 64;                                  // [waves]
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int c = lane & 15, kb = lane >> 4;
   const int tile = blockIdx.x;
@@ -283,6 +292,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
   for (int q = 0; q < 4; ++q)
 #pragma unroll
     for (int i = 0; i < 4; ++i) tot[q][i] = 0.f;
+  float poison = 0.f;  // becomes NaN when an activation is NaN or infinite (the digits cannot carry that)
 
   for (int q0 = wv * QUADS; q0 < nquads; q0 += WAVES * QUADS) {
     // ---- loads of this round (unconditional, clamped): activations, then packed words -------
@@ -321,6 +331,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         if (!live) xv[sp_][j] = 0.f;
+        poison = fmaf(xv[sp_][j], 0.f, poison);
         amax = fmaxf(amax, fabsf(xv[sp_][j]));
       }
     }
@@ -401,6 +412,10 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
     __builtin_amdgcn_wave_barrier();
   }
   // ---- combine columns and waves ------------------------------------------------------------------
+  {
+    const float wp = wave_sum(poison);
+    if (lane == 0) poison_w[wv] = wp;
+  }
   if (c < 5) {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
@@ -416,6 +431,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
       const float* rw = red + (w * 5) * 64 + tid;
       // digits 3..0, then the bias of 8 per nibble times the (centred) bit count of column 4
       v += (((rw[192] * 16.f + rw[128]) * 16.f + rw[64]) * 16.f + rw[0]) - 34952.f * rw[256];
+      v += poison_w[w];
     }
     // operand units 2^-10, and the sums hold half of sum s*x
     a.y[n] = (_Float16)(v * 2048.f);
@@ -427,7 +443,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
 template <int NB, int QUADS>
 int launch_bcq_mfma(const LutArgs& a, hipStream_t stream) {
   constexpr int WAVES = 8;
-  const size_t smem = (size_t)WAVES * QUADS * kQuadBytes + (size_t)WAVES * 5 * 64 * 4;
+  const size_t smem = (size_t)WAVES * QUADS * kQuadBytes + (size_t)WAVES * 5 * 64 * 4 + (size_t)WAVES * 4;
   const int ntiles = a.N / 64;
   if (a.qbias)
     hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, true>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);

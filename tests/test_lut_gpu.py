@@ -82,3 +82,16 @@ def test_vs_reference_kernel(hq, oracle):
     # the reference accumulates everything in fp16 (and across 128 K tiles with fp16 atomics)
     assert rel_err(y.cpu().numpy(), r, FLOOR_F16) <= TOL_F16_ACC
     assert rel_err(y.cpu().numpy(), exact) <= rel_err(r, exact)
+
+
+def test_non_finite_activations_propagate(hq, oracle):
+    import torch
+    bW, alpha, qb, x = oa.make_lut_problem(55, 1024, 256, 3, 128)
+    dev = "cuda:0"
+    for bad in (np.nan, np.inf):
+        xs = x.copy()
+        xs[300] = bad
+        y = hq.lut_matmul(torch.from_numpy(xs).to(dev), torch.from_numpy(bW.view(np.int32)).to(dev),
+                          torch.from_numpy(alpha).to(dev), torch.from_numpy(qb).to(dev), 128)
+        torch.cuda.synchronize()
+        assert not np.isfinite(y.cpu().numpy().astype(np.float32)).any(), bad
