@@ -15,6 +15,8 @@
  *   - return value: 0 on success, a negative HQ_ERR_* code for a rejected
  *     argument (nothing is launched), or a positive hipError_t value;
  *   - nothing is printed; hq_strerror() turns a code into text;
+ *   - a NaN or an infinity among the activations makes the affected outputs non-finite (the
+ *     fixed-point matrix-core paths give NaN where the reference arithmetic would give +-Inf);
  *   - the library keeps one small workspace per (device, stream) pair (split-K
  *     partial sums, arrival counters, re-ordered GEMM activations), allocated by
  *     hq_init() or by the first call that needs it; calls on different streams
