@@ -23,7 +23,9 @@
  *   LUT-GEMM                : bit packing + dequant formula pinned by the
  *                             reference host loops compiled into oracle/_ref
  *                             (src/lut-gemm-hip/main.cu:118-146)
- *   AQLM                    : PARITY UNPINNED (the reference checks nothing)
+ *   AQLM                    : the reference checks nothing; pinned by a golden output of the
+ *                             reference kernel itself (tests/golden/aqlm_reference_kernel.npz,
+ *                             bit-identical in mode 1) and by closed forms
  *   int8 activation quant   : pinned by the reference host loops compiled into
  *                             oracle/_ref (src/quantVLLM-cuda/reference.h)
  *   4-bit blockwise quantize: PARITY UNPINNED (no counterpart in the reference)
@@ -136,7 +138,7 @@ void hqo_lut_gemv_f16(const uint32_t* bW, const uint16_t* alpha_f16,
                       const uint16_t* qbias_f16, const uint16_t* x_f16,
                       uint16_t* y_f16, int K, int N, int nb, int group);
 
-/* ---- AQLM 1x16 (PARITY UNPINNED) ---------------------------------------- */
+/* ---- AQLM 1x16 ------------------------------------------------------------ */
 /* src/quantAQLM-hip/main.cu:29-101.  mode 0: double accumulation;
  * mode 1: the reference's arithmetic (4 chained hfma2 per code, halves widened
  * and summed in fp32 in lane order, fp32 shuffle-down tree over 64 lanes).
