@@ -290,7 +290,34 @@ def cpu_others():
         kind = "port"
     out["quantize_dynamic8_16777216"] = {"cpu_us": timed(fn) * 8 * 1e6, "kind": kind,
                                          "sample": "2,097,152 of 16,777,216 elements, scaled x8"}
+    omp = reference_quantbnb_omp()
+    if omp is not None:
+        out["quantize_dynamic8_16777216"]["reference_omp"] = omp
     return out
+
+
+def reference_quantbnb_omp():
+    """The reference's own quantBnB-omp program (compiled into oracle/_ref where the HeCBench tree was mounted),
+    run host-only with OMP_TARGET_OFFLOAD=DISABLED in a child process; returns what it prints, or None."""
+    import re
+    import subprocess
+    from tests import oracle_api as oa
+    if not os.path.exists(oa.REF_CPU_SO):
+        return None
+    code = ("import ctypes,sys; lib=ctypes.CDLL(sys.argv[1]); "
+            "argv=(ctypes.c_char_p*3)(b'main', b'16777216', b'3'); sys.exit(lib.ref_quantbnb_omp_main(3, argv))")
+    env = dict(os.environ, OMP_TARGET_OFFLOAD="DISABLED")
+    try:
+        r = subprocess.run([sys.executable, "-c", code, oa.REF_CPU_SO], capture_output=True, text=True, env=env,
+                           timeout=120)
+    except subprocess.TimeoutExpired:
+        return None
+    m = re.search(r"Average execution time of kQuantize kernel with block size \d+: ([0-9.]+) \(us\)", r.stdout)
+    if not m:
+        return None
+    return {"us": float(m.group(1)), "cores": os.cpu_count(), "kind": "reference",
+            "sample": "quantBnB-omp main, 16,777,216 elements x 3, OMP_TARGET_OFFLOAD=DISABLED",
+            "verdict": "PASS" if "PASS" in r.stdout else "FAIL"}
 
 
 def main():
@@ -352,6 +379,8 @@ def main():
                 result["other_configs"][name]["cpu_serial"] = {"us": round(cpu["cpu_us"], 1), "cores": 1,
                                                                "kind": cpu.get("kind", "port"),
                                                                "sample": cpu["sample"]}
+                if "reference_omp" in cpu:
+                    result["other_configs"][name]["cpu_reference_omp"] = cpu["reference_omp"]
     print(json.dumps(result))
 
 
