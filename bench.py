@@ -315,7 +315,8 @@ def reference_quantbnb_omp():
     m = re.search(r"Average execution time of kQuantize kernel with block size \d+: ([0-9.]+) \(us\)", r.stdout)
     if not m:
         return None
-    return {"us": float(m.group(1)), "cores": os.cpu_count(), "kind": "reference",
+    return {"us": float(m.group(1)), "cores": int(os.environ.get("OMP_NUM_THREADS") or os.cpu_count()),
+            "kind": "reference",
             "sample": "quantBnB-omp main, 16,777,216 elements x 3, OMP_TARGET_OFFLOAD=DISABLED",
             "verdict": "PASS" if "PASS" in r.stdout else "FAIL"}
 
