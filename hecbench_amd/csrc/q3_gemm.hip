@@ -150,8 +150,13 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
     sc = *reinterpret_cast<const f4v*>(a.scales + n_out);
     zr = *reinterpret_cast<const f4v*>(a.zeros + n_out);
   }
-  constexpr int ROWS_PER_WAVE = Mpad / kWaves;
-  const float rs_lane = a.rowsum[wv * ROWS_PER_WAVE + (lane & (ROWS_PER_WAVE - 1))];
+  // In the final reduction a wave finishes rows 4*wv .. 4*wv+3 of every 32-row block: half wave kb takes
+  // rows 4*wv + 2*kb and 4*wv + 2*kb + 1, lane nl four adjacent columns.
+  float rs[MB][2];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) rs[mb][j] = a.rowsum[mb * 32 + 4 * wv + 2 * kb + j];
 
   f16v acc[MB][4];
 #pragma unroll
@@ -215,53 +220,39 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
   }
   __syncthreads();
 
-  // ---- sum the waves' accumulators through LDS -------------------------------------------
+  // ---- sum the waves' accumulators through LDS, one 32-row block at a time -------------------
   // D[row][col = nl]: register i of a lane holds row (i/4)*8 + kb*4 + i%4 of its 32-row block;
-  // the four accumulators q of a lane are four adjacent output columns 4*nl + q.
-  float* red = reinterpret_cast<float*>(lds);  // kWaves/2 regions of [Mpad][128] floats
-  constexpr int REGION = Mpad * kTileN;
-  auto put = [&](int region) {
+  // the four accumulators q of a lane are four adjacent output columns 4*nl + q.  Every wave writes
+  // its block to its own region ([32][128] floats), then every wave sums four rows over the eight
+  // regions, applies scale / zero and stores them: all waves are busy in both phases.
+  float* red = reinterpret_cast<float*>(lds);
+  constexpr int REGION = 32 * kTileN;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+  for (int mb = 0; mb < MB; ++mb) {
+    if (mb) __syncthreads();  // the previous block has been read
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int m = mb * 32 + (i >> 2) * 8 + kb * 4 + (i & 3);
-        f4v v = {acc[mb][0][i], acc[mb][1][i], acc[mb][2][i], acc[mb][3][i]};
-        *reinterpret_cast<f4v*>(red + (size_t)region * REGION + m * kTileN + 4 * nl) = v;
+    for (int i = 0; i < 16; ++i) {
+      const int r = (i >> 2) * 8 + kb * 4 + (i & 3);
+      const f4v v = {acc[mb][0][i], acc[mb][1][i], acc[mb][2][i], acc[mb][3][i]};
+      *reinterpret_cast<f4v*>(red + (size_t)wv * REGION + r * kTileN + 4 * nl) = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int r = 4 * wv + 2 * kb + j;
+      const int m = mb * 32 + r;
+      f4v v = *reinterpret_cast<const f4v*>(red + r * kTileN + 4 * nl);
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w)
+        v += *reinterpret_cast<const f4v*>(red + (size_t)w * REGION + r * kTileN + 4 * nl);
+      if (m < a.M && n_out < a.N) {
+        f4v o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = sc[e] * (v[e] * 16777216.f) - zr[e] * rs[mb][j];
+        f4v* dst = reinterpret_cast<f4v*>(a.out + (size_t)m * a.N + n_out);
+        if (a.flags & HQ_FLAG_ACCUMULATE) { const f4v old = *dst; o += old; }
+        *dst = o;
       }
-  };
-  constexpr int H = kWaves / 2;
-  if (wv >= H) put(wv - H);
-  __syncthreads();
-  if (wv < H) {
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int m = mb * 32 + (i >> 2) * 8 + kb * 4 + (i & 3);
-        const f4v v = *reinterpret_cast<const f4v*>(red + (size_t)wv * REGION + m * kTileN + 4 * nl);
-        acc[mb][0][i] += v.x; acc[mb][1][i] += v.y; acc[mb][2][i] += v.z; acc[mb][3][i] += v.w;
-      }
-  }
-  __syncthreads();
-  if (wv < H) put(wv);
-  __syncthreads();
-  // every wave finishes Mpad/kWaves rows: half wave kb takes every other row, lane -> four columns
-#pragma unroll
-  for (int r = kb; r < ROWS_PER_WAVE; r += 2) {
-    const int m = wv * ROWS_PER_WAVE + r;
-    const float rs = __shfl(rs_lane, r);  // every lane takes part (the row sum lives in lane r)
-    if (m < a.M && n_out < a.N) {
-      f4v v = *reinterpret_cast<const f4v*>(red + m * kTileN + 4 * nl);
-#pragma unroll
-      for (int region = 1; region < H; ++region)
-        v += *reinterpret_cast<const f4v*>(red + (size_t)region * REGION + m * kTileN + 4 * nl);
-      f4v o;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = sc[e] * (v[e] * 16777216.f) - zr[e] * rs;
-      f4v* dst = reinterpret_cast<f4v*>(a.out + (size_t)m * a.N + n_out);
-      if (a.flags & HQ_FLAG_ACCUMULATE) { const f4v old = *dst; o += old; }
-      *dst = o;
     }
   }
 }
@@ -269,7 +260,7 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
 template <int MB>
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   constexpr int Mpad = 32 * MB;
-  const size_t smem = (size_t)(kWaves / 2) * Mpad * kTileN * 4;  // reduction regions
+  const size_t smem = (size_t)kWaves * 32 * kTileN * 4;  // one [32][128] fp32 region per wave
   static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_gemm_kernel<MB>),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (attr != hipSuccess) return (int)attr;
