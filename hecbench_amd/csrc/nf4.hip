@@ -97,6 +97,50 @@ __global__ __launch_bounds__(256) void dequant4_kernel(const uint32_t* __restric
   }
 }
 
+// Persistent variant of the main path (MODE 0 only): a workgroup walks chunks of 256*U words with
+// the next chunk's loads in flight while the current chunk is converted and stored, so the read and
+// the write streams overlap in time.
+template <int U>
+__global__ __launch_bounds__(256) void dequant4_pipelined_kernel(const uint32_t* __restrict__ packed,
+                                                                const float* __restrict__ absmax,
+                                                                u4v* __restrict__ out, int64_t nwords, int shift,
+                                                                int table) {
+  __shared__ float tab[16];
+  if (threadIdx.x < 16) tab[threadIdx.x] = table ? c_fp4[threadIdx.x] : c_nf4[threadIdx.x];
+  const int64_t chunk_words = 256 * U;
+  const int64_t nchunks = (nwords + chunk_words - 1) / chunk_words;
+  uint32_t w[U], wn[U];
+  float am[U], amn[U];
+  auto load = [&](int64_t chunk, uint32_t (&ww)[U], float (&aa)[U]) {
+    const int64_t base = chunk * chunk_words + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = min(base + u * 256, nwords - 1);  // clamped: a duplicate is loaded, never stored
+      ww[u] = packed[i];
+      aa[u] = absmax[(i * 8) >> shift];
+    }
+  };
+  int64_t chunk = blockIdx.x;
+  if (chunk < nchunks) load(chunk, w, am);
+  __syncthreads();
+  for (; chunk < nchunks; chunk += gridDim.x) {
+    const int64_t next = chunk + gridDim.x;
+    if (next < nchunks) load(next, wn, amn);
+    const int64_t base = chunk * chunk_words + threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int64_t i = base + u * 256;
+      uint32_t o[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) o[b] = deq_pair(tab, (w[u] >> (8 * b)) & 255u, am[u], am[u]);
+      const u4v ov = {o[0], o[1], o[2], o[3]};
+      if (i < nwords) __builtin_nontemporal_store(ov, out + i);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) { w[u] = wn[u]; am[u] = amn[u]; }
+  }
+}
+
 // Tail / odd sizes: one element per thread.
 __global__ __launch_bounds__(256) void dequant4_tail_kernel(const uint8_t* __restrict__ packed,
                                                            const float* __restrict__ absmax,
@@ -141,7 +185,19 @@ extern "C" int hq_dequant_nf4(const uint8_t* packed, const float* absmax, void* 
   if (mode == MM)                                                                                            \
     hipLaunchKernelGGL((dequant4_kernel<U, MM, NT>), dim3((unsigned)blocks), dim3(256), 0, stream, pw, absmax, \
                        (u4v*)out_fp16, nwords, blocksize, shift, table);
+    // Pipelined variant, four workgroups per CU: measured 7.5 us against 7.8 us at 4096x4096 and 26.2
+    // against 27.1 us at 2^26 elements, but 4 % slower at 2^30, so it is kept to the mid sizes.
+    int pipe = hq_env_int("HQ_NF4_PIPE", -1);
+    if (pipe < 0) pipe = (nwords >= (1 << 19) && nwords <= (1 << 25)) ? 4 : 0;
+    if (mode == 0 && pipe > 0) {
+      constexpr int PU = 4;
+      const int64_t nch = (nwords + 256 * PU - 1) / (256 * PU);
+      const int64_t grid = std::min<int64_t>((int64_t)dev->cus * pipe, nch);
+      hipLaunchKernelGGL((dequant4_pipelined_kernel<PU>), dim3((unsigned)grid), dim3(256), 0, stream, pw, absmax,
+                         (u4v*)out_fp16, nwords, shift, table);
+    } else {
     HQ_NF4_LAUNCH(0) HQ_NF4_LAUNCH(1) HQ_NF4_LAUNCH(2)
+    }
 #undef HQ_NF4_LAUNCH
     rc = hq_launch_status();
     if (rc != HQ_OK) return rc;

@@ -16,7 +16,7 @@ def _run(hq, packed, absmax, n, blocksize, table=0):
 
 
 @pytest.mark.parametrize("table", [0, 1])
-@pytest.mark.parametrize("n,blocksize", [(4096 * 4096, 64), (1 << 20, 128), (1 << 16, 4096), (96, 32),
+@pytest.mark.parametrize("n,blocksize", [(4096 * 4096, 64), (4096 * 1100 + 8 * 37 + 3, 64), ((1 << 22) + 8, 256), (1 << 20, 128), (1 << 16, 4096), (96, 32),
                                          (100000, 64), (99999, 64), (31, 2), (4096, 16), (2048, 24), (64, 64)])
 def test_bit_exact(hq, oracle, n, blocksize, table):
     packed, absmax = oa.make_nf4_problem(n + blocksize + table, n, blocksize)
