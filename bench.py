@@ -229,10 +229,33 @@ def bench_others(steps, warmup):
     out["mxfp4_qdq_4096x4096_f16"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
                                       "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
     del src, dst
+    # quantVLLM at its default run size: 4096 tokens of 5137 fp16 activations -> int8 (rotate 12 x 63 MB)
+    tk, hd = 4096, 5137
+    nb = 12
+    xs = [(torch.randint(-300, 700, (tk, hd), device=dev, generator=g)).half() for _ in range(nb)]
+    qo = [torch.empty(tk, hd, dtype=torch.int8, device=dev) for _ in range(nb)]
+    scl = torch.empty(tk, device=dev)
+    azp = torch.empty(tk, dtype=torch.int32, device=dev)
+    args = [(vp(xs[i]), vp(qo[i])) for i in range(nb)]
+    psc, paz = vp(scl), vp(azp)
+    b = 3.0 * tk * hd
+    for name, call in (
+            ("int8_quant_static_4096x5137_f16",
+             lambda i: check(lib.hq_int8_quant_static(args[i][0], 1, args[i][1], tk, hd, ctypes.c_float(0.1), 0, 0, stream))),
+            ("int8_quant_static_azp_4096x5137_f16",
+             lambda i: check(lib.hq_int8_quant_static(args[i][0], 1, args[i][1], tk, hd, ctypes.c_float(0.1), 1, 3, stream))),
+            ("int8_quant_dynamic_4096x5137_f16",
+             lambda i: check(lib.hq_int8_quant_dynamic(args[i][0], 1, args[i][1], psc, None, tk, hd, stream))),
+            ("int8_quant_dynamic_azp_4096x5137_f16",
+             lambda i: check(lib.hq_int8_quant_dynamic(args[i][0], 1, args[i][1], psc, paz, tk, hd, stream)))):
+        secs = _time_loop(call, nb, steps, warmup)
+        out[name] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
+                     "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
+    del xs, qo
     # the quantBnB benchmark's own kernel at its default size: 16,777,216 floats -> 8-bit codes (rotate 8 x 84 MB)
     nq = 16777216
     nb = 8
-    code = torch.linspace(-1.0, 1.0, 256, device=dev)  # any sorted 256-entry table costs the same to search
+    code = hq.dynamic_map().to(dev)  # the table the reference quantises with
     As = [torch.randn(nq, device=dev, generator=g) for _ in range(nb)]
     qs = [torch.empty(nq, dtype=torch.uint8, device=dev) for _ in range(nb)]
     secs = _time_loop(lambda i: hq.quantize_dynamic8(code, As[i], out=qs[i]), nb, st, 5)

@@ -6,18 +6,25 @@
 // src/quantVLLM-cuda/utils.h).  Bit-exact contract: fp32 IEEE division, round to nearest
 // even, saturation, exactly as the reference's host loops (src/quantVLLM-cuda/reference.h).
 //
-// One workgroup per token.  A lane converts eight consecutive elements per trip (128-bit
-// loads for fp16 / bf16, two for fp32) into one packed 64-bit store.  The dynamic variants
-// reduce max |x| (or min and max) with cross-lane butterflies and one LDS exchange, and
-// keep the row in registers between the two passes when it fits.
+// HBM-bound: 3 bytes per fp16 / bf16 element, 5 per fp32 element.  The tensor is cut into units of
+// eight consecutive elements on a grid anchored at element 0 of the tensor, not of the row, so that a
+// unit is one aligned 128-bit load (two for fp32) and one 64-bit store whatever the hidden size is
+// (the reference's run size is 5137); a unit that straddles a row boundary is masked.
+//   static : no row structure at all, a flat grid-stride loop over the units.
+//   dynamic: a wave per row up to 1536 elements, a workgroup per row beyond; the row stays in registers
+//            between the max / min pass and the quantise pass (one read of x, up to 10240 elements),
+//            and the next row is already being loaded meanwhile.
+// The division by a scale shared by many elements is done as a multiplication by its reciprocal
+// wherever that provably rounds to the same integer (the product is further from a tie than its error
+// bound, or saturates either way); the other lanes divide.
 #include "hq_internal.h"
 
 namespace {
 
-__device__ __forceinline__ float to_f32(float v) { return v; }
-__device__ __forceinline__ float to_f32(_Float16 v) { return (float)v; }
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u2v __attribute__((ext_vector_type(2)));
+
 struct bf16_t { uint16_t bits; };  // bfloat16 = the upper half of an fp32
-__device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float((uint32_t)v.bits << 16); }
 
 // src/quantVLLM-cuda/utils.h:9-24
 __device__ __forceinline__ int float_to_int8_rn(float x) {
@@ -25,167 +32,419 @@ __device__ __forceinline__ int float_to_int8_rn(float x) {
   dst = dst < -128.f ? -128.f : (127.f < dst ? 127.f : dst);
   return (int)dst;
 }
-// src/quantVLLM-cuda/utils.h:26-50
+// src/quantVLLM-cuda/utils.h:26-50: round to nearest even, saturating at the int32 range.  The
+// hardware conversion saturates by itself (and turns a NaN into 0); it is written as an instruction
+// because the C conversion of an out-of-range value is undefined.
 __device__ __forceinline__ int float_to_int32_rn(float x) {
   const float dst = rintf(x);
-  if (dst >= 2147483648.f) return 2147483647;
-  if (dst <= -2147483648.f) return -2147483647 - 1;
-  return (int)dst;
+  int r;
+  asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(dst));
+  return r;
 }
 // src/quantVLLM-cuda/utils.h:52-61 (saturating add of the zero point happens in int32)
 __device__ __forceinline__ int int32_to_int8(int x) { return x < -128 ? -128 : (127 < x ? 127 : x); }
 
-constexpr int kThreads = 256;
-constexpr int kVec = 8;       // elements per lane per trip
-constexpr int kKeep = 4;      // trips kept in registers by the dynamic kernels (rows up to 8192)
+constexpr int kVec = 8;  // elements per unit
+
+// One unit of raw data: 16 bytes of fp16 / bf16 or 32 bytes of fp32.
+template <typename T> struct Raw { u4v w[sizeof(T) == 4 ? 2 : 1]; };
 
 template <typename T>
-__device__ __forceinline__ void load8(const T* p, float (&v)[kVec], bool vec_ok, int valid) {
-  if (vec_ok && valid == kVec) {
-    T tmp[kVec];
-    if (sizeof(T) == 2) {
-      *reinterpret_cast<uint4*>(tmp) = *reinterpret_cast<const uint4*>(p);
-    } else {
-      reinterpret_cast<uint4*>(tmp)[0] = reinterpret_cast<const uint4*>(p)[0];
-      reinterpret_cast<uint4*>(tmp)[1] = reinterpret_cast<const uint4*>(p)[1];
-    }
+__device__ __forceinline__ Raw<T> load_unit(const T* __restrict__ base, int64_t unit) {
+  Raw<T> r;
+  const u4v* p = reinterpret_cast<const u4v*>(base + unit * kVec);
 #pragma unroll
-    for (int i = 0; i < kVec; ++i) v[i] = to_f32(tmp[i]);
-  } else {
+  for (int i = 0; i < (int)(sizeof(T) == 4 ? 2 : 1); ++i) r.w[i] = __builtin_nontemporal_load(p + i);
+  return r;
+}
+// A unit that reaches past the end of the tensor: element by element, zeros beyond.
+template <typename T>
+__device__ __forceinline__ Raw<T> load_unit_tail(const T* __restrict__ base, int64_t unit, int64_t total) {
+  Raw<T> r;
+  T tmp[kVec];
 #pragma unroll
-    for (int i = 0; i < kVec; ++i) v[i] = i < valid ? to_f32(p[i]) : 0.f;
+  for (int i = 0; i < kVec; ++i) {
+    const int64_t e = unit * kVec + i;
+    tmp[i] = e < total ? base[e] : T{};
   }
+  __builtin_memcpy(&r, tmp, sizeof(r));
+  return r;
+}
+__device__ __forceinline__ void unpack(const Raw<float>& r, float (&v)[kVec]) {
+#pragma unroll
+  for (int i = 0; i < kVec; ++i) v[i] = __uint_as_float(r.w[i >> 2][i & 3]);
+}
+__device__ __forceinline__ void unpack(const Raw<_Float16>& r, float (&v)[kVec]) {
+#pragma unroll
+  for (int i = 0; i < kVec; ++i)
+    v[i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.w[0][i >> 1] >> (16 * (i & 1))));
+}
+__device__ __forceinline__ void unpack(const Raw<bf16_t>& r, float (&v)[kVec]) {
+#pragma unroll
+  for (int i = 0; i < kVec; ++i)
+    v[i] = __uint_as_float((i & 1) ? (r.w[0][i >> 1] & 0xffff0000u) : (r.w[0][i >> 1] << 16));
 }
 
-__device__ __forceinline__ void store8(int8_t* p, const int (&q)[kVec], bool vec_ok, int valid) {
-  if (vec_ok && valid == kVec) {
-    uint2 w;
+// Makes the compiler forget what it knows about a unit's bits, so that the values converted for the
+// first pass are not kept alive (at twice the registers of the raw data) for the second.
+template <typename T>
+__device__ __forceinline__ void forget(Raw<T>& r) {
+#pragma unroll
+  for (int i = 0; i < (int)(sizeof(T) == 4 ? 2 : 1); ++i)
+    asm volatile("" : "+v"(r.w[i]));
+}
+
+// Stores elements [lo, hi) of a unit's eight results; all eight as one 64-bit store.
+__device__ __forceinline__ void store_unit(int8_t* __restrict__ out, int64_t unit, const int (&q)[kVec], int lo, int hi,
+                                           bool aligned) {
+  int8_t* p = out + unit * kVec;
+  if (lo == 0 && hi == kVec && aligned) {
+    u2v w;
     w.x = (uint32_t)(q[0] & 255) | ((uint32_t)(q[1] & 255) << 8) | ((uint32_t)(q[2] & 255) << 16) |
           ((uint32_t)(q[3] & 255) << 24);
     w.y = (uint32_t)(q[4] & 255) | ((uint32_t)(q[5] & 255) << 8) | ((uint32_t)(q[6] & 255) << 16) |
           ((uint32_t)(q[7] & 255) << 24);
-    *reinterpret_cast<uint2*>(p) = w;
-  } else {
+    __builtin_nontemporal_store(w, reinterpret_cast<u2v*>(p));
+  } else if (aligned) {
+    // a unit shared with the neighbouring row: the fewest naturally aligned pieces that cover [lo, hi)
+    // (a store instruction costs the same whatever it carries, and the other lanes wait for it)
+    uint32_t w[2];
+    w[0] = (uint32_t)(q[0] & 255) | ((uint32_t)(q[1] & 255) << 8) | ((uint32_t)(q[2] & 255) << 16) |
+           ((uint32_t)(q[3] & 255) << 24);
+    w[1] = (uint32_t)(q[4] & 255) | ((uint32_t)(q[5] & 255) << 8) | ((uint32_t)(q[6] & 255) << 16) |
+           ((uint32_t)(q[7] & 255) << 24);
 #pragma unroll
-    for (int i = 0; i < kVec; ++i)
-      if (i < valid) p[i] = (int8_t)q[i];
-  }
-}
-
-// Block-wide reduction of (a: max, b: min) through one LDS exchange.
-__device__ __forceinline__ void block_max_min(float& a, float& b, float* lds) {
+    for (int d = 0; d < 2; ++d) {
+      const bool whole = lo <= 4 * d && hi >= 4 * d + 4;
+      if (whole) reinterpret_cast<uint32_t*>(p)[d] = w[d];
 #pragma unroll
-  for (int m = 32; m > 0; m >>= 1) {
-    a = fmaxf(a, __shfl_xor(a, m));
-    b = fminf(b, __shfl_xor(b, m));
-  }
-  const int wv = threadIdx.x >> 6;
-  if ((threadIdx.x & 63) == 0) { lds[wv] = a; lds[8 + wv] = b; }
-  __syncthreads();
-#pragma unroll
-  for (int w = 0; w < kThreads / 64; ++w) { a = fmaxf(a, lds[w]); b = fminf(b, lds[8 + w]); }
-}
-
-template <typename T, bool AZP>
-__global__ __launch_bounds__(kThreads) void static_quant_kernel(const T* __restrict__ in, int8_t* __restrict__ out,
-                                                               float scale, int azp, int hidden, int vec_ok) {
-  const int64_t token = blockIdx.x;
-  in += token * hidden;
-  out += token * hidden;
-  for (int e0 = threadIdx.x * kVec; e0 < hidden; e0 += kThreads * kVec) {
-    const int valid = min(kVec, hidden - e0);
-    float v[kVec];
-    int q[kVec];
-    load8(in + e0, v, vec_ok, valid);
-#pragma unroll
-    for (int i = 0; i < kVec; ++i)
-      q[i] = AZP ? int32_to_int8(float_to_int32_rn(v[i] / scale) + azp) : float_to_int8_rn(v[i] / scale);
-    store8(out + e0, q, vec_ok, valid);
-  }
-}
-
-template <typename T, bool AZP>
-__global__ __launch_bounds__(kThreads) void dynamic_quant_kernel(const T* __restrict__ in, int8_t* __restrict__ out,
-                                                                float* __restrict__ scales, int32_t* __restrict__ azps,
-                                                                int hidden, int vec_ok) {
-  __shared__ float lds[16];
-  const int64_t token = blockIdx.x;
-  in += token * hidden;
-  out += token * hidden;
-  float keep[kKeep][kVec];
-  // reference initial values: max starts at FLT_MIN (smallest positive normal), min at FLT_MAX
-  // (reference.h:71-72); the symmetric variant starts its absmax at 0 (reference.h:43)
-  float mx = AZP ? 1.17549435e-38f : 0.f, mn = 3.40282347e+38f;
-  int trip = 0;
-  for (int e0 = threadIdx.x * kVec; e0 < hidden; e0 += kThreads * kVec, ++trip) {
-    const int valid = min(kVec, hidden - e0);
-    float v[kVec];
-    load8(in + e0, v, vec_ok, valid);
-#pragma unroll
-    for (int i = 0; i < kVec; ++i) {
-      if (i < valid) {
-        if (AZP) { mx = fmaxf(mx, v[i]); mn = fminf(mn, v[i]); }
-        else mx = fmaxf(mx, fabsf(v[i]));
+      for (int h = 0; h < 2; ++h) {
+        const int b = 4 * d + 2 * h;
+        const bool half = !whole && lo <= b && hi >= b + 2;
+        if (half) reinterpret_cast<uint16_t*>(p)[2 * d + h] = (uint16_t)(w[d] >> (16 * h));
+        if (!whole && !half) {
+          if (lo <= b && hi > b) p[b] = (int8_t)q[b];
+          if (lo <= b + 1 && hi > b + 1) p[b + 1] = (int8_t)q[b + 1];
+        }
       }
-      if (trip < kKeep) keep[trip < kKeep ? trip : 0][i] = v[i];
     }
-  }
-  block_max_min(mx, mn, lds);
-  float scale_val, mul = 0.f;
-  int azp_val = 0;
-  if (AZP) {
-    scale_val = (mx - mn) / 255.0f;
-    azp_val = (int)rintf(-128.0f - mn / scale_val);
   } else {
-    scale_val = mx / 127.0f;
-    mul = 127.0f / mx;
-  }
-  if (threadIdx.x == 0) {
-    scales[token] = scale_val;
-    if (AZP) azps[token] = azp_val;
-  }
-  trip = 0;
-  for (int e0 = threadIdx.x * kVec; e0 < hidden; e0 += kThreads * kVec, ++trip) {
-    const int valid = min(kVec, hidden - e0);
-    float v[kVec];
-    int q[kVec];
-    if (trip < kKeep) {
-#pragma unroll
-      for (int i = 0; i < kVec; ++i) v[i] = keep[trip < kKeep ? trip : 0][i];
-    } else {
-      load8(in + e0, v, vec_ok, valid);
-    }
 #pragma unroll
     for (int i = 0; i < kVec; ++i)
-      q[i] = AZP ? int32_to_int8(float_to_int32_rn(v[i] / scale_val) + azp_val) : float_to_int8_rn(v[i] * mul);
-    store8(out + e0, q, vec_ok, valid);
+      if (i >= lo && i < hi) p[i] = (int8_t)q[i];
   }
 }
 
-template <typename T>
-int launch_static(const T* in, int8_t* out, int64_t tokens, int hidden, float scale, int has_azp, int azp, int vec_ok,
-                  hipStream_t stream) {
-  if (has_azp)
-    hipLaunchKernelGGL((static_quant_kernel<T, true>), dim3((unsigned)tokens), dim3(kThreads), 0, stream, in, out, scale,
-                       azp, hidden, vec_ok);
-  else
-    hipLaunchKernelGGL((static_quant_kernel<T, false>), dim3((unsigned)tokens), dim3(kThreads), 0, stream, in, out, scale,
-                       azp, hidden, vec_ok);
-  return hq_launch_status();
+// Division by a scale that many elements share.  y = v * (1 / s) differs from the rounded quotient by
+// at most 2 ulp (half an ulp each for the reciprocal, the product and the quotient itself, rounded up),
+// so both round to the same integer unless y is within 2^-21 |y| of a tie; where the result saturates
+// the quotient need not be known at all.  The reciprocal must be a normal number for that bound.
+struct Divisor {
+  float s, r;
+  bool usable;
+  __device__ __forceinline__ explicit Divisor(float scale) : s(scale), r(1.0f / scale) {
+    const float a = fabsf(scale);
+    usable = a >= 0x1p-100f && a <= 0x1p100f;
+  }
+};
+
+// float_to_int8_rn(v / s) or, with AZP, int32_to_int8(float_to_int32_rn(v / s) + azp), for eight values.
+template <bool AZP>
+__device__ __forceinline__ void quantise8(const float (&v)[kVec], const Divisor& d, int azp, int (&q)[kVec]) {
+  bool exact = !d.usable;
+  float y[kVec];
+#pragma unroll
+  for (int i = 0; i < kVec; ++i) {
+    y[i] = v[i] * d.r;
+    const float dist = fabsf(y[i] - rintf(y[i]));  // distance to the nearest integer
+    // false for a NaN and for |y| >= 2^20; the constant margin covers quotients too small for a relative bound
+    const bool clear = fmaf(fabsf(y[i]), 0x1p-21f, dist) < 0.5f - 0x1p-20f;
+    // without a zero point everything beyond +-129 saturates whichever way it rounds
+    exact |= AZP ? !clear : !(clear || fabsf(y[i]) > 130.f);
+  }
+  if (__builtin_amdgcn_ballot_w64(exact)) {
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) y[i] = v[i] / d.s;
+  }
+#pragma unroll
+  for (int i = 0; i < kVec; ++i) q[i] = AZP ? int32_to_int8(float_to_int32_rn(y[i]) + azp) : float_to_int8_rn(y[i]);
 }
+
+// ---- static scale: elementwise over the whole tensor ---------------------------------------------
+constexpr int kStaticUnroll = 2;
+
+template <typename T, bool AZP>
+__global__ __launch_bounds__(256) void static_quant_kernel(const T* __restrict__ in, int8_t* __restrict__ out,
+                                                          float scale, int azp, int64_t total, int aligned) {
+  const Divisor d(scale);
+  const int64_t units = (total + kVec - 1) / kVec;
+  const int64_t full = aligned ? total / kVec : 0;  // units loaded whole: inside the tensor, pointers aligned
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t u0 = (int64_t)blockIdx.x * 256 + threadIdx.x; u0 < units; u0 += stride * kStaticUnroll) {
+    Raw<T> raw[kStaticUnroll];
+#pragma unroll
+    for (int k = 0; k < kStaticUnroll; ++k) {
+      const int64_t u = u0 + k * stride;
+      if (u < full) raw[k] = load_unit(in, u);
+      else if (u < units) raw[k] = load_unit_tail(in, u, total);
+      else raw[k] = Raw<T>{};
+    }
+#pragma unroll
+    for (int k = 0; k < kStaticUnroll; ++k) {
+      const int64_t u = u0 + k * stride;
+      float v[kVec];
+      int q[kVec];
+      unpack(raw[k], v);
+      quantise8<AZP>(v, d, azp, q);
+      if (u < units) store_unit(out, u, q, 0, (int)min((int64_t)kVec, total - u * kVec), aligned);
+    }
+  }
+}
+
+// ---- dynamic scale: LANES threads per row --------------------------------------------------------
+// Maximum of a[r] and minimum of b[r], r < R, over the LANES threads of a row.
+template <int LANES, int R>
+__device__ __forceinline__ void rows_max_min(float (&a)[R], float (&b)[R], float* lds) {
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 32; m > 0; m >>= 1) {
+      a[r] = fmaxf(a[r], __shfl_xor(a[r], m));
+      b[r] = fminf(b[r], __shfl_xor(b[r], m));
+    }
+  if (LANES > 64) {  // the rows span the workgroup: one exchange for all of them
+    const int wv = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) { lds[8 * r + wv] = a[r]; lds[8 * r + 4 + wv] = b[r]; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int w = 0; w < LANES / 64; ++w) { a[r] = fmaxf(a[r], lds[8 * r + w]); b[r] = fminf(b[r], lds[8 * r + 4 + w]); }
+  }
+}
+
+constexpr int kMaxRows = 3;
+
+// LANES threads per row (a wave, or the workgroup), so 256 / LANES row slots per workgroup, and R rows
+// in turn per slot and trip.  KEEP units per thread and row stay in registers between the max / min
+// pass and the quantise pass; a longer row streams the rest twice.  The next trip's rows are requested
+// as soon as this trip's have been scanned, so their loads are in flight during the reduction, the
+// quantisation and the stores: R is chosen so that this is enough data to cover the memory latency.
+// VEC: both pointers are aligned and the tensor is a whole number of units, so every unit is loaded whole.
+template <typename T, bool AZP, int LANES, int KEEP, int R, bool VEC>
+__global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict__ in, int8_t* __restrict__ out,
+                                                           float* __restrict__ scales, int32_t* __restrict__ azps,
+                                                           int64_t tokens, int hidden) {
+  constexpr bool aligned = VEC;
+  __shared__ float lds[8 * kMaxRows];
+  const int lane = threadIdx.x % LANES;
+  const int64_t total = tokens * hidden;
+  // the loop bounds are uniform over the wave (LANES == 64) or the workgroup
+  const int64_t slot = LANES == 64 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
+  const int64_t slots = LANES == 64 ? (int64_t)gridDim.x * 4 : gridDim.x;
+  auto fetch = [&](int64_t u) { return VEC ? load_unit(in, u) : load_unit_tail(in, u, total); };
+  // A row's units, and the multiple of 64 at or before its first: lanes are laid over the units from
+  // there, so that a wave's loads and stores cover whole 128-byte lines of the output (256 of the
+  // input) except at the row's ends.
+  struct Row { int64_t g0, u_first, u_end, u_base; };
+  auto row_of = [&](int64_t token) {
+    Row w;
+    w.g0 = token * hidden;
+    w.u_first = w.g0 / kVec;
+    w.u_end = (w.g0 + hidden + kVec - 1) / kVec;
+    w.u_base = w.u_first & ~(int64_t)63;
+    return w;
+  };
+  auto load_row = [&](int64_t token, Raw<T> (&buf)[KEEP]) {
+    const Row w = row_of(token);
+#pragma unroll
+    for (int k = 0; k < KEEP; ++k) {
+      const int64_t u = w.u_base + lane + (int64_t)k * LANES;
+      // whole units are loaded without a branch, so that the loads stay one straight run the waits can
+      // count; a unit outside the row repeats the row's first or last
+      if (VEC) buf[k] = load_unit(in, min(max(u, w.u_first), w.u_end - 1));
+      else if (u >= w.u_first && u < w.u_end) buf[k] = fetch(u);
+    }
+  };
+  Raw<T> keep[R][KEEP], ahead[R][KEEP];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    if (slot + r * slots < tokens) load_row(slot + r * slots, keep[r]);
+  for (int64_t first = slot; first < tokens; first += slots * R) {
+    float mx[R], mn[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      // reference initial values: max starts at FLT_MIN (smallest positive normal), min at FLT_MAX
+      // (reference.h:71-72); the symmetric variant starts its absmax at 0 (reference.h:43)
+      mx[r] = AZP ? 1.17549435e-38f : 0.f;
+      mn[r] = 3.40282347e+38f;
+      const int64_t token = first + r * slots;
+      if (token >= tokens) continue;
+      const Row w = row_of(token);
+      const int head = (int)(w.g0 - w.u_first * kVec);  // elements of the first unit that belong to the row before
+      auto scan = [&](const Raw<T>& raw, int64_t u) {
+        float v[kVec];
+        unpack(raw, v);
+        const int rel = (int)(u - w.u_first) * kVec - head;  // row position of the unit's element 0
+        const int lo = max(-rel, 0), hi = min(hidden - rel, kVec);
+        if (lo == 0 && hi == kVec) {  // all but the row's first and last unit
+#pragma unroll
+          for (int i = 0; i < kVec; ++i) {
+            if (AZP) { mx[r] = fmaxf(mx[r], v[i]); mn[r] = fminf(mn[r], v[i]); }
+            else mx[r] = fmaxf(mx[r], fabsf(v[i]));
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < kVec; ++i)
+            if (i >= lo && i < hi) {
+              if (AZP) { mx[r] = fmaxf(mx[r], v[i]); mn[r] = fminf(mn[r], v[i]); }
+              else mx[r] = fmaxf(mx[r], fabsf(v[i]));
+            }
+        }
+      };
+      const int trips = (int)((w.u_end - w.u_base + LANES - 1) / LANES);
+#pragma unroll
+      for (int k = 0; k < KEEP; ++k) {
+        const int64_t u = w.u_base + lane + (int64_t)k * LANES;
+        if (u >= w.u_first && u < w.u_end) scan(keep[r][k], u);
+      }
+      for (int k = KEEP; k < trips; ++k) {
+        const int64_t u = w.u_base + lane + (int64_t)k * LANES;
+        if (u >= w.u_first && u < w.u_end) scan(fetch(u), u);
+      }
+    }
+    // the next trip's loads go out here, behind nothing this trip still waits for
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t token = first + (R + r) * slots;
+      if (token < tokens) load_row(token, ahead[r]);
+    }
+    rows_max_min<LANES, R>(mx, mn, lds);
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int64_t token = first + r * slots;
+      if (token >= tokens) continue;
+      const Row w = row_of(token);
+      const int head = (int)(w.g0 - w.u_first * kVec);
+      float scale_val, mul = 0.f;
+      int azp_val = 0;
+      if (AZP) {
+        scale_val = (mx[r] - mn[r]) / 255.0f;
+        azp_val = (int)rintf(-128.0f - mn[r] / scale_val);
+      } else {
+        scale_val = mx[r] / 127.0f;
+        mul = 127.0f / mx[r];
+      }
+      if (lane == 0) {
+        scales[token] = scale_val;
+        if (AZP) azps[token] = azp_val;
+      }
+      const Divisor d(scale_val);
+      auto emit = [&](Raw<T> raw, int64_t u) {
+        float v[kVec];
+        int q[kVec];
+        forget(raw);
+        unpack(raw, v);
+        if (AZP) {
+          quantise8<true>(v, d, azp_val, q);
+        } else {
+#pragma unroll
+          for (int i = 0; i < kVec; ++i) q[i] = float_to_int8_rn(v[i] * mul);
+        }
+        const int rel = (int)(u - w.u_first) * kVec - head;
+        store_unit(out, u, q, max(-rel, 0), min(hidden - rel, kVec), aligned);
+      };
+      const int trips = (int)((w.u_end - w.u_base + LANES - 1) / LANES);
+#pragma unroll
+      for (int k = 0; k < KEEP; ++k) {
+        const int64_t u = w.u_base + lane + (int64_t)k * LANES;
+        if (u >= w.u_first && u < w.u_end) emit(keep[r][k], u);
+      }
+      for (int k = KEEP; k < trips; ++k) {
+        const int64_t u = w.u_base + lane + (int64_t)k * LANES;
+        if (u >= w.u_first && u < w.u_end) emit(fetch(u), u);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int k = 0; k < KEEP; ++k) keep[r][k] = ahead[r][k];
+    if (LANES > 64) __syncthreads();  // the exchange buffer is reused by the next trip
+  }
+}
+
+// The 128-bit loads and 64-bit stores need both base pointers on their grid; other pointers are served
+// element by element.
+__host__ inline int pointers_aligned(const void* in, const void* out) {
+  return !((uintptr_t)in & 15) && !((uintptr_t)out & 7);
+}
+
 template <typename T>
-int launch_dynamic(const T* in, int8_t* out, float* scales, int32_t* azps, int64_t tokens, int hidden, int vec_ok,
-                   hipStream_t stream) {
-  if (azps)
-    hipLaunchKernelGGL((dynamic_quant_kernel<T, true>), dim3((unsigned)tokens), dim3(kThreads), 0, stream, in, out, scales,
-                       azps, hidden, vec_ok);
+int launch_static(const T* in, int8_t* out, int64_t tokens, int hidden, float scale, int has_azp, int azp,
+                  const HqDevice* dev, hipStream_t stream) {
+  const int aligned = pointers_aligned(in, out);
+  const int64_t total = tokens * hidden;
+  const int64_t units = (total + kVec - 1) / kVec;
+  int64_t blocks = (units + 256 * kStaticUnroll - 1) / (256 * kStaticUnroll);
+  const int64_t cap = (int64_t)dev->cus * 32;  // grid-stride beyond that
+  if (blocks > cap) blocks = cap;
+  if (has_azp)
+    hipLaunchKernelGGL((static_quant_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream, in, out, scale, azp,
+                       total, aligned);
   else
-    hipLaunchKernelGGL((dynamic_quant_kernel<T, false>), dim3((unsigned)tokens), dim3(kThreads), 0, stream, in, out,
-                       scales, azps, hidden, vec_ok);
+    hipLaunchKernelGGL((static_quant_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, stream, in, out, scale, azp,
+                       total, aligned);
   return hq_launch_status();
 }
 
-int check_common(const void* x, int x_dtype, const int8_t* out, int64_t tokens, int hidden, int* vec_ok) {
+template <typename T, bool AZP, bool VEC>
+void launch_dynamic_vec(const T* in, int8_t* out, float* scales, int32_t* azps, int64_t tokens, int hidden,
+                        const HqDevice* dev, hipStream_t stream) {
+  // short rows get a wave each, the others the workgroup; the units a thread must keep pick the kernel,
+  // and shorter rows go several to a trip
+  const bool wave_rows = hidden <= 64 * kVec * 3;
+  const int lanes = wave_rows ? 64 : 256;
+  const int span = (hidden + kVec - 1) / kVec + 1 + 63;  // units from the 64-unit boundary before a ragged row to its end
+  const int need = (span + lanes - 1) / lanes;
+  const int64_t groups = wave_rows ? (tokens + 3) / 4 : tokens;
+  const dim3 grid((unsigned)std::min<int64_t>(groups, (int64_t)dev->cus * hq_env_int("HQ_ACTQ_GROUPS", 8))), block(256);
+#define HQ_ROWS(LANES, KEEP, R)                                                                                   \
+  hipLaunchKernelGGL((dynamic_quant_kernel<T, AZP, LANES, KEEP, R, VEC>), grid, block, 0, stream, in, out, scales, \
+                     azps, tokens, hidden)
+  if (wave_rows) {
+    if (need <= 2) HQ_ROWS(64, 2, 3);
+    else if (need <= 3) HQ_ROWS(64, 3, 2);
+    else HQ_ROWS(64, 5, 1);
+  } else {
+    if (need <= 2) HQ_ROWS(256, 2, 3);
+    else if (need <= 3) HQ_ROWS(256, 3, 2);
+    else HQ_ROWS(256, 5, 1);
+  }
+#undef HQ_ROWS
+}
+
+template <typename T, bool AZP>
+void launch_dynamic_azp(const T* in, int8_t* out, float* scales, int32_t* azps, int64_t tokens, int hidden,
+                        const HqDevice* dev, hipStream_t stream) {
+  if (pointers_aligned(in, out) && (tokens * hidden) % kVec == 0)
+    launch_dynamic_vec<T, AZP, true>(in, out, scales, azps, tokens, hidden, dev, stream);
+  else
+    launch_dynamic_vec<T, AZP, false>(in, out, scales, azps, tokens, hidden, dev, stream);
+}
+
+template <typename T>
+int launch_dynamic(const T* in, int8_t* out, float* scales, int32_t* azps, int64_t tokens, int hidden,
+                   const HqDevice* dev, hipStream_t stream) {
+  if (azps) launch_dynamic_azp<T, true>(in, out, scales, azps, tokens, hidden, dev, stream);
+  else launch_dynamic_azp<T, false>(in, out, scales, azps, tokens, hidden, dev, stream);
+  return hq_launch_status();
+}
+
+int check_common(const void* x, int x_dtype, const int8_t* out, int64_t tokens, int hidden) {
   if (tokens < 0 || hidden <= 0) return HQ_ERR_BAD_SHAPE;
   if (x_dtype != HQ_DTYPE_F32 && x_dtype != HQ_DTYPE_F16 && x_dtype != HQ_DTYPE_BF16) return HQ_ERR_BAD_ENUM;
   if (tokens == 0) return HQ_OK;
@@ -193,7 +452,6 @@ int check_common(const void* x, int x_dtype, const int8_t* out, int64_t tokens, 
   if (tokens > 0x7fffffff) return HQ_ERR_TOO_LARGE;
   const int esz = x_dtype == HQ_DTYPE_F32 ? 4 : 2;
   if ((uintptr_t)x & (esz - 1)) return HQ_ERR_MISALIGNED;
-  *vec_ok = !((uintptr_t)x & 15) && !((uintptr_t)out & 7) && hidden % kVec == 0;
   return HQ_OK;
 }
 
@@ -202,24 +460,22 @@ int check_common(const void* x, int x_dtype, const int8_t* out, int64_t tokens, 
 extern "C" int hq_int8_quant_static(const void* x, int x_dtype, int8_t* out, int64_t num_tokens, int hidden_size,
                                     float scale, int has_azp, int32_t azp, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
-  int vec_ok = 0;
-  int rc = check_common(x, x_dtype, out, num_tokens, hidden_size, &vec_ok);
+  int rc = check_common(x, x_dtype, out, num_tokens, hidden_size);
   if (rc != HQ_OK || num_tokens == 0) return rc;
   const HqDevice* dev = nullptr;
   rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
   if (x_dtype == HQ_DTYPE_F32)
-    return launch_static((const float*)x, out, num_tokens, hidden_size, scale, has_azp, azp, vec_ok, stream);
+    return launch_static((const float*)x, out, num_tokens, hidden_size, scale, has_azp, azp, dev, stream);
   if (x_dtype == HQ_DTYPE_F16)
-    return launch_static((const _Float16*)x, out, num_tokens, hidden_size, scale, has_azp, azp, vec_ok, stream);
-  return launch_static((const bf16_t*)x, out, num_tokens, hidden_size, scale, has_azp, azp, vec_ok, stream);
+    return launch_static((const _Float16*)x, out, num_tokens, hidden_size, scale, has_azp, azp, dev, stream);
+  return launch_static((const bf16_t*)x, out, num_tokens, hidden_size, scale, has_azp, azp, dev, stream);
 }
 
 extern "C" int hq_int8_quant_dynamic(const void* x, int x_dtype, int8_t* out, float* scales, int32_t* azp,
                                      int64_t num_tokens, int hidden_size, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
-  int vec_ok = 0;
-  int rc = check_common(x, x_dtype, out, num_tokens, hidden_size, &vec_ok);
+  int rc = check_common(x, x_dtype, out, num_tokens, hidden_size);
   if (rc != HQ_OK || num_tokens == 0) return rc;
   if (!scales) return HQ_ERR_NULL_POINTER;
   if (((uintptr_t)scales & 3) || ((uintptr_t)azp & 3)) return HQ_ERR_MISALIGNED;
@@ -227,8 +483,8 @@ extern "C" int hq_int8_quant_dynamic(const void* x, int x_dtype, int8_t* out, fl
   rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
   if (x_dtype == HQ_DTYPE_F32)
-    return launch_dynamic((const float*)x, out, scales, azp, num_tokens, hidden_size, vec_ok, stream);
+    return launch_dynamic((const float*)x, out, scales, azp, num_tokens, hidden_size, dev, stream);
   if (x_dtype == HQ_DTYPE_F16)
-    return launch_dynamic((const _Float16*)x, out, scales, azp, num_tokens, hidden_size, vec_ok, stream);
-  return launch_dynamic((const bf16_t*)x, out, scales, azp, num_tokens, hidden_size, vec_ok, stream);
+    return launch_dynamic((const _Float16*)x, out, scales, azp, num_tokens, hidden_size, dev, stream);
+  return launch_dynamic((const bf16_t*)x, out, scales, azp, num_tokens, hidden_size, dev, stream);
 }

@@ -93,6 +93,24 @@ def dequant_4bit(packed, absmax, n_elems, blocksize, table=NF4, out=None):
     return out
 
 
+def dynamic_map():
+    """The signed dynamic 8-bit map of bitsandbytes (7 exponent bits), 256 sorted fp32 values in [-1, 1]: the
+    table the reference ships as a literal (src/quantBnB-cuda/code.h).  Returns a CPU tensor."""
+    import numpy as np
+    f32 = np.float32
+    vals = []
+    for i in range(7):
+        items = (1 << i) + 1
+        step = (f32(1.0) - f32(0.1)) / f32(items - 1)
+        b = [f32(0.1) + step * f32(j) if j < items // 2 else f32(1.0) - step * f32(items - 1 - j) for j in range(items)]
+        sc = f32(10.0 ** (-6 + i))
+        for j in range(items - 1):
+            mean = (b[j] + b[j + 1]) / f32(2.0)
+            vals += [sc * mean, -(sc * mean)]
+    vals += [f32(0.0), f32(1.0)]
+    return torch.from_numpy(np.sort(np.array(vals, dtype=f32)))
+
+
 def quantize_dynamic8(code, A, out=None):
     _dev(code, A, out)
     if out is None:

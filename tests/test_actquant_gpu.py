@@ -33,6 +33,79 @@ def test_static_and_dynamic_bit_exact(hq, oracle, tokens, hidden, dtype):
         assert np.array_equal(got.cpu().numpy(), want), with_azp
 
 
+@pytest.mark.parametrize("dtype,tokens,hidden", [("f16", 2100, 5137), ("bf16", 2100, 1001), ("f32", 2100, 8192),
+                                                 ("f16", 2049, 8185), ("f32", 2200, 13), ("f16", 2051, 1),
+                                                 ("f32", 2050, 777), ("f16", 300, 9000), ("f32", 5, 41001)])
+def test_ragged_rows_wave_and_group_paths(hq, oracle, dtype, tokens, hidden):
+    """Enough rows for the wave-per-row kernels, hidden sizes that leave every row unaligned, and rows beyond
+    what a wave or a workgroup keeps in registers."""
+    import torch
+    x = _act_inputs(dtype, tokens, hidden, tokens * 3 + hidden)
+    dx = _dev(x)
+    for azp in (None, -7):
+        got = hq.static_scaled_int8_quant(dx, 0.37, azp)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy(), oracle.int8_quant_static(x, 0.37, azp)), azp
+    for with_azp in (False, True):
+        got, gs, gz = hq.dynamic_scaled_int8_quant(dx, with_azp)
+        torch.cuda.synchronize()
+        want, ws, wz = oracle.int8_quant_dynamic(x, with_azp)
+        assert np.array_equal(gs.cpu().numpy(), ws)
+        if with_azp:
+            assert np.array_equal(gz.cpu().numpy(), wz)
+        assert np.array_equal(got.cpu().numpy(), want), with_azp
+
+
+@pytest.mark.parametrize("scale", [0.1, 0.25, 0.3, 1.0 / 3.0, 7.0, 1e-3, 123.456, 2.0 ** -100, 2.0 ** 100, 2.0 ** -101,
+                                   2.0 ** 101, 1e-40, 3e38, -0.5])
+def test_static_division_ties_and_extreme_scales(hq, oracle, scale):
+    """Inputs whose quotient by the scale sits on, or one float beside, a rounding tie or the saturation
+    edges, and scales for which the reciprocal is not usable: the result must be that of the true
+    division.  (NaN quotients are left out: converting them to an integer is undefined in the reference.)"""
+    import torch
+    s = np.float32(scale)
+    k = np.arange(-140, 141, dtype=np.float64)
+    with np.errstate(all="ignore"):
+        ties = ((k + 0.5) * np.float64(s)).astype(np.float32)
+        ints = (k * np.float64(s)).astype(np.float32)
+        base = np.concatenate([ties, ints])
+        x = np.concatenate([base, np.nextafter(base, np.float32(np.inf)), np.nextafter(base, np.float32(-np.inf)),
+                            np.array([0.0, -0.0, np.inf, -np.inf, 3e38, -3e38, 1e-45, 1e30, -1e30], np.float32),
+                            np.random.default_rng(3).standard_normal(3000).astype(np.float32) * np.float32(abs(scale)) * 60])
+    x = np.ascontiguousarray(np.resize(x, (4, x.size // 4)))
+    dx = _dev(x)
+    for azp in (None, 0, 54, -100, 2000000, -2000000):
+        if azp is not None:  # int32 overflow of quotient + zero point is undefined in the reference as well
+            with np.errstate(all="ignore"):
+                x = np.where(np.abs(x.astype(np.float64) / np.float64(s)) < 2.0e9, x, np.float32(0))
+            dx = _dev(x)
+        got = hq.static_scaled_int8_quant(dx, float(s), azp)
+        torch.cuda.synchronize()
+        want = oracle.int8_quant_static(x, float(s), azp)
+        bad = np.flatnonzero(got.cpu().numpy().ravel() != want.ravel())
+        assert bad.size == 0, (scale, azp, x.ravel()[bad[:6]], got.cpu().numpy().ravel()[bad[:6]], want.ravel()[bad[:6]])
+
+
+def test_unaligned_pointers(hq, oracle):
+    """Views that start one element into an allocation: served element by element, same results."""
+    import torch
+    x = _act_inputs("f16", 9, 1001, 5)
+    flat = torch.zeros(x.size + 8, dtype=torch.float16, device="cuda:0")
+    dx = flat[1:1 + x.size].view(9, 1001)
+    dx.copy_(_dev(x))
+    assert dx.data_ptr() % 16 != 0
+    assert np.array_equal(hq.static_scaled_int8_quant(dx, 0.1, 3).cpu().numpy(), oracle.int8_quant_static(x, 0.1, 3))
+    got, gs, gz = hq.dynamic_scaled_int8_quant(dx, True)
+    want, ws, wz = oracle.int8_quant_dynamic(x, True)
+    assert np.array_equal(got.cpu().numpy(), want) and np.array_equal(gs.cpu().numpy(), ws)
+    obuf = torch.zeros(x.size + 8, dtype=torch.int8, device="cuda:0")
+    o = obuf[3:3 + x.size].view(9, 1001)
+    got = hq.static_scaled_int8_quant(_dev(x), 0.1, None, out=o)
+    torch.cuda.synchronize()
+    assert np.array_equal(o.cpu().numpy(), oracle.int8_quant_static(x, 0.1, None))
+    assert int(obuf[:3].abs().sum()) == 0 and int(obuf[3 + x.size:].abs().sum()) == 0
+
+
 def test_reference_fixture(hq, oracle):
     """The reference main's own input: rand() % 1000 - 300, scale 0.1, azp 54 (main.cu:186-236)."""
     import torch

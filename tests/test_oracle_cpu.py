@@ -227,6 +227,11 @@ def test_dynamic_map_close_to_reference_table(o):
     assert np.all(np.abs(o.dynamic_map() - code) <= 2 * np.spacing(np.abs(code)))
 
 
+def test_package_dynamic_map_equals_oracle(o):
+    import hecbench_amd as hq
+    assert np.array_equal(hq.dynamic_map().numpy(), o.dynamic_map())
+
+
 # ------------------------------------------------------------------ LUT-GEMM
 
 @pytest.mark.parametrize("fx,N,K,NB", [("ref_lut_fixture_256x256x3", 256, 256, 3),
