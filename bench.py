@@ -26,7 +26,7 @@ ROWS = 3 * K // 32
 ALGO_BYTES = ROWS * N * 4 + 2 * N * 4 + K * 4 + N * 4   # weights + scale/zero + x + y = 17,056,768
 # HBM bytes per launch of the matvec kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what
 # the same counter reads for a plain 256 MiB device copy (profiles/q3_matvec_4096x11008.txt).
-Q3_TRAFFIC_BYTES = 17267235
+Q3_TRAFFIC_BYTES = 17267237
 
 
 def _time_loop(fn, n_buffers, steps, warmup):
