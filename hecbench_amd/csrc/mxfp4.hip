@@ -91,19 +91,27 @@ template <bool BF16>
 __global__ __launch_bounds__(256) void mxfp4_qdq_kernel(const u4v* __restrict__ in, u4v* __restrict__ out,
                                                        int64_t units) {
   const int64_t stride = (int64_t)gridDim.x * 256 * kUnroll;
-  for (int64_t base = (int64_t)blockIdx.x * 256 * kUnroll + threadIdx.x; base < units; base += stride) {
-    u4v raw[kUnroll];
+  u4v raw[kUnroll], ahead[kUnroll];
+  auto load = [&](int64_t base, u4v (&dst)[kUnroll]) {
 #pragma unroll
     for (int k = 0; k < kUnroll; ++k) {
       const int64_t u = base + k * 256;
-      raw[k] = in[u < units ? u : base];
+      dst[k] = __builtin_nontemporal_load(in + (u < units ? u : base));
     }
+  };
+  int64_t base = (int64_t)blockIdx.x * 256 * kUnroll + threadIdx.x;
+  if (base < units) load(base, raw);
+  for (; base < units; base += stride) {
+    // the next trip's loads are in flight while this one is converted and stored
+    if (base + stride < units) load(base + stride, ahead);
 #pragma unroll
     for (int k = 0; k < kUnroll; ++k) {
       const int64_t u = base + k * 256;
       const u4v res = qdq_unit<BF16>(raw[k]);
       if (u < units) __builtin_nontemporal_store(res, out + u);
     }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) raw[k] = ahead[k];
   }
 }
 
@@ -121,7 +129,7 @@ extern "C" int hq_mxfp4_qdq(const void* in, void* out, int64_t n_elems, int dtyp
   if (rc != HQ_OK) return rc;
   const int64_t units = n_elems / 8;
   int64_t blocks = (units + 256 * kUnroll - 1) / (256 * kUnroll);
-  const int64_t cap = (int64_t)dev->cus * 32;  // grid-stride beyond that
+  const int64_t cap = (int64_t)dev->cus * 32;  // grid-stride beyond that, the next trip's loads issued ahead
   if (blocks > cap) blocks = cap;
   if (dtype == HQ_DTYPE_BF16)
     hipLaunchKernelGGL(mxfp4_qdq_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream,

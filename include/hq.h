@@ -165,8 +165,10 @@ int hq_quantize_4bit(const void* x, int x_dtype, uint8_t* packed, float* absmax,
  *   dynamic: azp == NULL: scales[t] = max|x_t| / 127, out = sat8(rne(x * (127 / max|x_t|)))
  *            azp != NULL: scales[t] = (max_t - min_t) / 255, azp[t] = rne(-128 - min_t / scales[t]),
  *                         out = sat8(sat32(rne(x / scales[t])) + azp[t])
- * All arithmetic is fp32 IEEE (true division, round to nearest even): bit-exact with the
- * reference host loops (src/quantVLLM-cuda/reference.h:1-93).  Replaces
+ * Results are those of fp32 IEEE arithmetic (true division, round to nearest even): bit-exact with
+ * the reference host loops (src/quantVLLM-cuda/reference.h:1-93) wherever those are defined (a NaN
+ * quotient, or a quotient plus zero point beyond int32, is undefined there).  Any element alignment
+ * is accepted; x 16-byte and out 8-byte aligned take the vector path at every hidden size.  Replaces
  * static_scaled_int8_quant / dynamic_scaled_int8_quant, src/quantVLLM-hip/main.cu:133-168.
  */
 int hq_int8_quant_static(const void* x, int x_dtype, int8_t* out, int64_t num_tokens, int hidden_size,
