@@ -132,6 +132,7 @@ struct GemmArgs {
 
 template <int MB>  // 32-row blocks of activations
 __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
+  constexpr int Mpad = 32 * MB;
   extern __shared__ u4v lds[];  // used by the final reduction only
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -284,7 +285,7 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
   for (int m0 = 0; m0 < M; m0 += 64) {
     const int Mb = M - m0 < 64 ? M - m0 : 64;
     const int MB = Mb > 32 ? 2 : 1;
-    // const int Mpad = 32 * MB;
+    const int Mpad = 32 * MB;
     const _Float16* A = reinterpret_cast<const _Float16*>(x) + (size_t)m0 * K;
     hipLaunchKernelGGL(q3_gemm_prep, dim3(Gpad / 4 + Mpad), dim3(256), 0, stream, A, Ap, rowsum, Mb, K, Mpad,
                        Gpad);
