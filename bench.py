@@ -299,6 +299,12 @@ def cpu_others():
                               "sample": "1024 of 16384 rows, scaled x16"}
     bits = rng.standard_normal(4096 * 4096).astype(np.float16).view(np.uint16)
     out["mxfp4_qdq_4096x4096_f16"] = {"cpu_us": timed(lambda: o.mxfp4_qdq(bits, False)) * 1e6, "sample": "1 full call"}
+    xa8 = rng.integers(-300, 700, (512, 5137)).astype(np.float16)
+    o.int8_quant_static(xa8[:1], 0.1)  # the oracle builds its fp16 conversion table on first use
+    out["int8_quant_static_4096x5137_f16"] = {"cpu_us": timed(lambda: o.int8_quant_static(xa8, 0.1)) * 8 * 1e6,
+                                              "sample": "512 of 4096 tokens, scaled x8"}
+    out["int8_quant_dynamic_azp_4096x5137_f16"] = {"cpu_us": timed(lambda: o.int8_quant_dynamic(xa8, True)) * 8 * 1e6,
+                                                   "sample": "512 of 4096 tokens, scaled x8"}
     # 8-bit quantiser: the reference's own host function where oracle/_ref holds it, else the oracle's restatement
     A = rng.standard_normal(1 << 21).astype(np.float32)
     q = np.zeros(A.size, np.uint8)
