@@ -127,3 +127,24 @@ def test_empty_and_bad_arguments(hq):
     assert hq.static_scaled_int8_quant(x, 0.1).numel() == 0
     with pytest.raises(ValueError):
         hq.static_scaled_int8_quant(torch.zeros((2, 2), dtype=torch.int32, device="cuda:0"), 0.1)
+
+
+def test_full_size_error_bound(hq):
+    """The reference's run size (4096 tokens of 5137) without the oracle: the dequantised values of the
+    dynamic quantisers lie within half a step of the input, every row uses the full range, and the
+    static quantiser agrees with the dynamic one when given a row's own scale."""
+    import torch
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev); g.manual_seed(11)
+    x = (torch.randn(4096, 5137, device=dev, generator=g) * 3).half()
+    xf = x.float()
+    q, s, _ = hq.dynamic_scaled_int8_quant(x)
+    assert np.array_equal(s.cpu().numpy(), xf.abs().amax(dim=1).cpu().numpy() / np.float32(127.0))  # true division
+    assert float((q.float() * s[:, None] - xf).abs().div(s[:, None]).max()) <= 0.5 + 1e-3
+    assert int(q.abs().amax(dim=1).min()) == 127
+    qa, sa, za = hq.dynamic_scaled_int8_quant(x, True)
+    assert float(((qa.float() - za[:, None].float()) * sa[:, None] - xf).abs().div(sa[:, None]).max()) <= 1.0 + 1e-3
+    assert int(qa.amax(dim=1).min()) >= 126 and int(qa.amin(dim=1).max()) <= -127
+    row = 1234
+    qs = hq.static_scaled_int8_quant(x[row:row + 1].contiguous(), float(sa[row]), int(za[row]))
+    assert torch.equal(qs[0], qa[row])

@@ -101,3 +101,22 @@ def test_vs_reference_kernel(hq, oracle):
     y = hq.quantize_dynamic8(dcode, dA)
     torch.cuda.synchronize()
     assert torch.equal(y, out)
+
+
+def test_full_size_round_trip(hq):
+    """At the benchmark's size, without the oracle: every table value quantises to its own index (the
+    dynamic map is strictly increasing), and an input between two entries to one of the two."""
+    import torch
+    dev = torch.device("cuda:0")
+    code = hq.dynamic_map().to(dev)
+    n = 16777216
+    g = torch.Generator(device=dev); g.manual_seed(5)
+    idx = torch.randint(0, 256, (n,), device=dev, generator=g)
+    out = hq.quantize_dynamic8(code, code[idx])
+    assert torch.equal(out.long(), idx)
+    x = torch.empty(n, device=dev).uniform_(-0.99, 0.99, generator=g)
+    q = hq.quantize_dynamic8(code, x).long()
+    lo = torch.searchsorted(code, x, right=True) - 1          # code[lo] <= x < code[lo + 1]
+    assert bool(((q == lo) | (q == lo + 1)).all())
+    nearest = torch.where((x - code[lo]).abs() <= (code[(lo + 1).clamp(max=255)] - x).abs(), lo, lo + 1)
+    assert float((q != nearest).float().mean()) < 1e-4        # they differ on exact ties only
