@@ -245,28 +245,35 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict_
   // the loop bounds are uniform over the wave (LANES == 64) or the workgroup
   const int64_t slot = LANES == 64 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
   const int64_t slots = LANES == 64 ? (int64_t)gridDim.x * 4 : gridDim.x;
-  auto fetch = [&](int64_t u) { return VEC ? load_unit(in, u) : load_unit_tail(in, u, total); };
   // A row's units, and the multiple of 64 at or before its first: lanes are laid over the units from
   // there, so that a wave's loads and stores cover whole 128-byte lines of the output (256 of the
-  // input) except at the row's ends.
-  struct Row { int64_t g0, u_first, u_end, u_base; };
+  // input) except at the row's ends.  Everything per row is uniform: base pointers at that multiple of
+  // 64, and 32-bit unit numbers j relative to it (valid in [first, end)).
+  struct Row { const T* in; int8_t* out; int64_t ubase; int first, end, head; };
   auto row_of = [&](int64_t token) {
     Row w;
-    w.g0 = token * hidden;
-    w.u_first = w.g0 / kVec;
-    w.u_end = (w.g0 + hidden + kVec - 1) / kVec;
-    w.u_base = w.u_first & ~(int64_t)63;
+    const int64_t g0 = token * hidden;
+    const int64_t u_first = g0 / kVec;
+    w.ubase = u_first & ~(int64_t)63;
+    w.first = (int)(u_first - w.ubase);
+    w.end = (int)((g0 + hidden + kVec - 1) / kVec - w.ubase);
+    w.head = (int)(g0 - u_first * kVec);  // elements of the first unit that belong to the row before
+    w.in = in + w.ubase * kVec;
+    w.out = out + w.ubase * kVec;
     return w;
+  };
+  auto fetch = [&](const Row& w, int j) {
+    return VEC ? load_unit(w.in, j) : load_unit_tail(in, w.ubase + j, total);
   };
   auto load_row = [&](int64_t token, Raw<T> (&buf)[KEEP]) {
     const Row w = row_of(token);
 #pragma unroll
     for (int k = 0; k < KEEP; ++k) {
-      const int64_t u = w.u_base + lane + (int64_t)k * LANES;
+      const int j = lane + k * LANES;
       // whole units are loaded without a branch, so that the loads stay one straight run the waits can
       // count; a unit outside the row repeats the row's first or last
-      if (VEC) buf[k] = load_unit(in, min(max(u, w.u_first), w.u_end - 1));
-      else if (u >= w.u_first && u < w.u_end) buf[k] = fetch(u);
+      if (VEC) buf[k] = load_unit(w.in, min(max(j, w.first), w.end - 1));
+      else if (j >= w.first && j < w.end) buf[k] = fetch(w, j);
     }
   };
   Raw<T> keep[R][KEEP], ahead[R][KEEP];
@@ -284,11 +291,10 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict_
       const int64_t token = first + r * slots;
       if (token >= tokens) continue;
       const Row w = row_of(token);
-      const int head = (int)(w.g0 - w.u_first * kVec);  // elements of the first unit that belong to the row before
-      auto scan = [&](const Raw<T>& raw, int64_t u) {
+      auto scan = [&](const Raw<T>& raw, int j) {
         float v[kVec];
         unpack(raw, v);
-        const int rel = (int)(u - w.u_first) * kVec - head;  // row position of the unit's element 0
+        const int rel = (j - w.first) * kVec - w.head;  // row position of the unit's element 0
         const int lo = max(-rel, 0), hi = min(hidden - rel, kVec);
         if (lo == 0 && hi == kVec) {  // all but the row's first and last unit
 #pragma unroll
@@ -305,16 +311,12 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict_
             }
         }
       };
-      const int trips = (int)((w.u_end - w.u_base + LANES - 1) / LANES);
 #pragma unroll
       for (int k = 0; k < KEEP; ++k) {
-        const int64_t u = w.u_base + lane + (int64_t)k * LANES;
-        if (u >= w.u_first && u < w.u_end) scan(keep[r][k], u);
+        const int j = lane + k * LANES;
+        if (j >= w.first && j < w.end) scan(keep[r][k], j);
       }
-      for (int k = KEEP; k < trips; ++k) {
-        const int64_t u = w.u_base + lane + (int64_t)k * LANES;
-        if (u >= w.u_first && u < w.u_end) scan(fetch(u), u);
-      }
+      for (int j = lane + KEEP * LANES; j < w.end; j += LANES) scan(fetch(w, j), j);
     }
     // the next trip's loads go out here, behind nothing this trip still waits for
 #pragma unroll
@@ -329,7 +331,6 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict_
       const int64_t token = first + r * slots;
       if (token >= tokens) continue;
       const Row w = row_of(token);
-      const int head = (int)(w.g0 - w.u_first * kVec);
       float scale_val, mul = 0.f;
       int azp_val = 0;
       if (AZP) {
@@ -344,7 +345,7 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict_
         if (AZP) azps[token] = azp_val;
       }
       const Divisor d(scale_val);
-      auto emit = [&](Raw<T> raw, int64_t u) {
+      auto emit = [&](Raw<T> raw, int j) {
         float v[kVec];
         int q[kVec];
         forget(raw);
@@ -355,19 +356,15 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict_
 #pragma unroll
           for (int i = 0; i < kVec; ++i) q[i] = float_to_int8_rn(v[i] * mul);
         }
-        const int rel = (int)(u - w.u_first) * kVec - head;
-        store_unit(out, u, q, max(-rel, 0), min(hidden - rel, kVec), aligned);
+        const int rel = (j - w.first) * kVec - w.head;
+        store_unit(w.out, j, q, max(-rel, 0), min(hidden - rel, kVec), aligned);
       };
-      const int trips = (int)((w.u_end - w.u_base + LANES - 1) / LANES);
 #pragma unroll
       for (int k = 0; k < KEEP; ++k) {
-        const int64_t u = w.u_base + lane + (int64_t)k * LANES;
-        if (u >= w.u_first && u < w.u_end) emit(keep[r][k], u);
+        const int j = lane + k * LANES;
+        if (j >= w.first && j < w.end) emit(keep[r][k], j);
       }
-      for (int k = KEEP; k < trips; ++k) {
-        const int64_t u = w.u_base + lane + (int64_t)k * LANES;
-        if (u >= w.u_first && u < w.u_end) emit(fetch(u), u);
-      }
+      for (int j = lane + KEEP * LANES; j < w.end; j += LANES) emit(fetch(w, j), j);
     }
 #pragma unroll
     for (int r = 0; r < R; ++r)
