@@ -1,13 +1,11 @@
-// Test infrastructure: the reference host loops of quantVLLM
-// (src/quantVLLM-cuda/reference.h and utils.h, HeCBench tree) behind C entry points.
-#include <hip/hip_runtime.h>
-#include <hip/hip_fp16.h>
-#include <hip/hip_bf16.h>
-#include <cmath>
+// Test infrastructure: the reference host loops of quantVLLM (src/quantVLLM-cuda/reference.h and
+// utils.h, HeCBench tree) and its device kernels (src/quantVLLM-hip/main.cu) behind C entry points.
+// The reference's device kernels and their launchers (src/quantVLLM-hip/main.cu) come in with it.
 #include <cstdint>
 #include <limits>
-#include "utils.h"
-#include "reference.h"
+#define main hecbench_quantvllm_hip_main
+#include "main.cu"  // pulls in utils.h and reference.h
+#undef main
 
 #define EXPORT extern "C" __attribute__((visibility("default")))
 
@@ -33,4 +31,19 @@ EXPORT void ref_int8_quant_dynamic(const void* x, int dtype, int8_t* out, float*
   if (dtype == 0) run_dynamic<float>(x, out, scales, azp, tokens, hidden);
   else if (dtype == 1) run_dynamic<__half>(x, out, scales, azp, tokens, hidden);
   else run_dynamic<__hip_bfloat16>(x, out, scales, azp, tokens, hidden);
+}
+
+// The device launchers of src/quantVLLM-hip/main.cu:140-168 (default stream; azp == 0 selects the
+// kernels without a zero point, as there).
+EXPORT void ref_hip_int8_quant_static(const void* x, int dtype, int8_t* out, long tokens, int hidden, float scale,
+                                      int azp) {
+  if (dtype == 0) static_scaled_int8_quant<float>(out, (const float*)x, hidden, (int)tokens, scale, azp);
+  else if (dtype == 1) static_scaled_int8_quant<__half>(out, (const __half*)x, hidden, (int)tokens, scale, azp);
+  else static_scaled_int8_quant<__hip_bfloat16>(out, (const __hip_bfloat16*)x, hidden, (int)tokens, scale, azp);
+}
+EXPORT void ref_hip_int8_quant_dynamic(const void* x, int dtype, int8_t* out, float* scales, int32_t* azp,
+                                       long tokens, int hidden) {
+  if (dtype == 0) dynamic_scaled_int8_quant<float>(out, (const float*)x, hidden, (int)tokens, scales, azp);
+  else if (dtype == 1) dynamic_scaled_int8_quant<__half>(out, (const __half*)x, hidden, (int)tokens, scales, azp);
+  else dynamic_scaled_int8_quant<__hip_bfloat16>(out, (const __hip_bfloat16*)x, hidden, (int)tokens, scales, azp);
 }

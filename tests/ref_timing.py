@@ -124,6 +124,31 @@ def main():
     print(f"mxfp4 fp16 n={nel}: reference kernel "
           f"{timeit(lambda: ref.ref_mxfp4_qdq(vp(src), vp(dst), ctypes.c_int(nel), ctypes.c_int(0), None), 20):.1f} us, "
           f"libhq {timeit(lambda: hq.mxfp4_qdq(src, out=dst), 20):.1f} us")
+    del src, dst
+    # quantVLLM at the reference's run size (4096 tokens of 5137 fp16), inputs rotated over 12 tensors
+    if hasattr(ref, "ref_hip_int8_quant_static"):
+        tk, hd = 4096, 5137
+        xs = [torch.randint(-300, 700, (tk, hd), device=dev, generator=g).half() for _ in range(12)]
+        q = torch.empty(tk, hd, dtype=torch.int8, device=dev)
+        sc = torch.empty(tk, device=dev)
+        zp = torch.empty(tk, dtype=torch.int32, device=dev)
+        lib = hq._lib.load()
+        it = [0]
+
+        def nxt():
+            it[0] += 1
+            return xs[it[0] % len(xs)]
+        cl = ctypes.c_long
+        for name, rf, of in (
+                ("static", lambda: ref.ref_hip_int8_quant_static(vp(nxt()), 1, vp(q), cl(tk), hd, cf(0.1), 0),
+                 lambda: lib.hq_int8_quant_static(vp(nxt()), 1, vp(q), tk, hd, 0.1, 0, 0, None)),
+                ("static azp", lambda: ref.ref_hip_int8_quant_static(vp(nxt()), 1, vp(q), cl(tk), hd, cf(0.1), 54),
+                 lambda: lib.hq_int8_quant_static(vp(nxt()), 1, vp(q), tk, hd, 0.1, 1, 54, None)),
+                ("dynamic", lambda: ref.ref_hip_int8_quant_dynamic(vp(nxt()), 1, vp(q), vp(sc), None, cl(tk), hd),
+                 lambda: lib.hq_int8_quant_dynamic(vp(nxt()), 1, vp(q), vp(sc), None, tk, hd, None)),
+                ("dynamic azp", lambda: ref.ref_hip_int8_quant_dynamic(vp(nxt()), 1, vp(q), vp(sc), vp(zp), cl(tk), hd),
+                 lambda: lib.hq_int8_quant_dynamic(vp(nxt()), 1, vp(q), vp(sc), vp(zp), tk, hd, None))):
+            print(f"int8 quant {name} {tk}x{hd} fp16: reference kernel {timeit(rf, 200):.1f} us, libhq {timeit(of, 200):.1f} us")
 
 
 if __name__ == "__main__":

@@ -148,3 +148,33 @@ def test_full_size_error_bound(hq):
     row = 1234
     qs = hq.static_scaled_int8_quant(x[row:row + 1].contiguous(), float(sa[row]), int(za[row]))
     assert torch.equal(qs[0], qa[row])
+
+
+@pytest.mark.parametrize("dtype,code", [("f32", 0), ("f16", 1), ("bf16", 2)])
+def test_vs_reference_device_kernels(hq, dtype, code):
+    """The reference's own device kernels (src/quantVLLM-hip/main.cu), compiled into oracle/_ref, on the same
+    device buffers: byte-for-byte equal, like the reference's own memcmp against its host loops."""
+    import ctypes
+    import torch
+    from tests import oracle_api as oa
+    ref = oa.load_ref_hip()
+    if ref is None or not hasattr(ref, "ref_hip_int8_quant_static"):
+        pytest.skip("oracle/_ref/libhecref_hip.so without the quantVLLM device kernels")
+    tokens, hidden = 257, 5137
+    x = _dev(_act_inputs(dtype, tokens, hidden, 17 + code))
+    vp = lambda t: None if t is None else ctypes.c_void_p(t.data_ptr())
+    for azp in (0, 54):
+        want = torch.empty(tokens, hidden, dtype=torch.int8, device="cuda:0")
+        ref.ref_hip_int8_quant_static(vp(x), code, vp(want), ctypes.c_long(tokens), hidden, ctypes.c_float(0.1), azp)
+        torch.cuda.synchronize()
+        assert torch.equal(hq.static_scaled_int8_quant(x, 0.1, azp if azp else None), want), azp
+    for with_azp in (False, True):
+        want = torch.empty(tokens, hidden, dtype=torch.int8, device="cuda:0")
+        ws = torch.empty(tokens, device="cuda:0")
+        wz = torch.empty(tokens, dtype=torch.int32, device="cuda:0") if with_azp else None
+        ref.ref_hip_int8_quant_dynamic(vp(x), code, vp(want), vp(ws), vp(wz), ctypes.c_long(tokens), hidden)
+        torch.cuda.synchronize()
+        got, gs, gz = hq.dynamic_scaled_int8_quant(x, with_azp)
+        assert torch.equal(gs, ws) and torch.equal(got, want), with_azp
+        if with_azp:
+            assert torch.equal(gz, wz)
