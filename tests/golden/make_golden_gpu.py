@@ -9,6 +9,8 @@ data only: seeded inputs and the outputs the reference's own kernels produce for
                                (src/gemv-hip/kernels.h:66-311), 256 x 256, blocks (16, 4)
   q3_reference_kernels.npz     VecQuant3MatMulKernel and ...Faster (src/quant3MatMul-hip/kernels.h:12-169)
   aqlm_reference_kernel.npz    Code1x16MatVec (src/quantAQLM-hip/main.cu:29-101)
+  quantvllm_reference_kernels.npz  the four int8 quantisation kernels (src/quantVLLM-hip/main.cu:11-131)
+  kquantize_reference_kernel.npz   kQuantize (src/quantBnB-hip/main.cu:90-130) with the table of code.h
 """
 import ctypes
 import os
@@ -102,6 +104,45 @@ def main():
     torch.cuda.synchronize()
     np.savez_compressed(os.path.join(out_dir, "aqlm_reference_kernel.npz"), codes=codes, used_entries=used,
                         used_values=vals, x=xa, y=ya.cpu().numpy(), sizes=np.array([128, 256, 0, 0], np.int32))
+
+    # ---- quantVLLM: the four device kernels on fp32 / fp16 / bf16 rows of 200 (fractions, the reference
+    # main's integers, ties of x / 0.1), and kQuantize on normal draws plus every table entry and midpoint
+    if hasattr(ref, "ref_hip_int8_quant_static"):
+        from tests.test_oracle_cpu import _act_inputs
+        fix = {}
+        tokens, hidden = 24, 200
+        for name, code in (("f32", 0), ("f16", 1), ("bf16", 2)):
+            x = _act_inputs(name, tokens, hidden, 900 + code)
+            dx = (x if isinstance(x, torch.Tensor) else torch.from_numpy(x)).to(dev)
+            fix[f"x_{name}"] = (dx.view(torch.int16).cpu().numpy().view(np.uint16) if code == 2 else dx.cpu().numpy())
+            for azp in (0, 54):
+                q = torch.empty(tokens, hidden, dtype=torch.int8, device=dev)
+                ref.ref_hip_int8_quant_static(vp(dx), code, vp(q), ctypes.c_long(tokens), hidden, ctypes.c_float(0.1), azp)
+                torch.cuda.synchronize()
+                fix[f"static_{name}_azp{azp}"] = q.cpu().numpy()
+            for with_azp in (0, 1):
+                q = torch.empty(tokens, hidden, dtype=torch.int8, device=dev)
+                sc = torch.empty(tokens, device=dev)
+                zp = torch.empty(tokens, dtype=torch.int32, device=dev)
+                ref.ref_hip_int8_quant_dynamic(vp(dx), code, vp(q), vp(sc), vp(zp) if with_azp else None,
+                                               ctypes.c_long(tokens), hidden)
+                torch.cuda.synchronize()
+                fix[f"dynamic_{name}_azp{with_azp}"] = q.cpu().numpy()
+                fix[f"dynamic_{name}_azp{with_azp}_scales"] = sc.cpu().numpy()
+                if with_azp:
+                    fix[f"dynamic_{name}_azp1_zero_points"] = zp.cpu().numpy()
+        np.savez_compressed(os.path.join(out_dir, "quantvllm_reference_kernels.npz"), **fix)
+    ref.ref_hip_code_table.restype = ctypes.POINTER(ctypes.c_float)
+    code = np.ctypeslib.as_array(ref.ref_hip_code_table(), shape=(256,)).copy()
+    mids = ((code[:-1].astype(np.float64) + code[1:]) / 2).astype(np.float32)
+    A = np.concatenate([rng.standard_normal(20000).astype(np.float32), code, mids,
+                        np.nextafter(mids, np.float32(2)), np.nextafter(mids, np.float32(-2)),
+                        np.array([-5, 5, 0, -0.0, 1e-30, -1e-30, np.inf, -np.inf], np.float32)])
+    dA, dcode = torch.from_numpy(A).to(dev), torch.from_numpy(code).to(dev)
+    qo = torch.zeros(A.size, dtype=torch.uint8, device=dev)
+    ref.ref_kquantize(vp(dcode), vp(dA), vp(qo), ctypes.c_long(A.size), None)
+    torch.cuda.synchronize()
+    np.savez_compressed(os.path.join(out_dir, "kquantize_reference_kernel.npz"), code=code, A=A, out=qo.cpu().numpy())
     print("wrote fixtures to", out_dir)
 
 

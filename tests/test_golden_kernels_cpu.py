@@ -64,3 +64,25 @@ def test_aqlm_restatement_is_bit_identical_to_reference_kernel(o):
     assert np.array_equal(y16.view(np.uint16), g["y"].view(np.uint16))
     y_exact, y64 = o.aqlm_matvec(g["codes"], cb, None, g["x"], tuple(int(v) for v in g["sizes"]), 65536, mode=0)
     assert rel_err(g["y"], y64, FLOOR_F16) <= TOL_F16_ACC
+
+
+def test_int8_quantisers_equal_reference_kernels(o):
+    import torch
+    g = _load("quantvllm_reference_kernels.npz")
+    for name in ("f32", "f16", "bf16"):
+        x = g[f"x_{name}"]
+        if name == "bf16":
+            x = torch.from_numpy(x.view(np.int16).copy()).view(torch.bfloat16)
+        for azp in (0, 54):
+            assert np.array_equal(o.int8_quant_static(x, 0.1, azp if azp else None), g[f"static_{name}_azp{azp}"])
+        for with_azp in (0, 1):
+            q, sc, zp = o.int8_quant_dynamic(x, bool(with_azp))
+            assert np.array_equal(q, g[f"dynamic_{name}_azp{with_azp}"])
+            assert np.array_equal(sc, g[f"dynamic_{name}_azp{with_azp}_scales"])
+            if with_azp:
+                assert np.array_equal(zp, g[f"dynamic_{name}_azp1_zero_points"])
+
+
+def test_quantize_dynamic8_equals_reference_kernel(o):
+    g = _load("kquantize_reference_kernel.npz")
+    assert np.array_equal(o.quantize_dynamic8(g["code"], g["A"]), g["out"])
