@@ -5,8 +5,9 @@
 //
 //   y[n] = sum_k x[k] * ( q_bias[k/G][n] + sum_b alpha[k/G][b][n] * s(k,b,n) )
 //
-// Two kernels.  Shapes with group size % 128 == 0 and N % 64 == 0 run on the matrix cores
-// (bcq_mfma_kernel below: the packed bits themselves are the fp8 operands, no tables).
+// Shapes with N % 64 == 0 and a group size that is a multiple of 128, 64 or 32 run on the matrix cores
+// (bcq_mfma_kernel and bcq_mfma_grouped_kernel below: the packed bits themselves are the operands, no
+// tables).
 // Every other shape runs the table kernel: for every 8-element sub-vector of x the 256
 // signed sums sum_j (+-x[j]) are tabulated once per workgroup in LDS (fp32 entries), and
 // each byte of a packed bit-plane word becomes one table lookup.  A workgroup owns a tile of columns
@@ -438,6 +439,246 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
   }
 }
 
+// ---- group sizes 64 and 32 --------------------------------------------------------------------------
+// A 128-element quad then spans GS = 2 or 4 alpha / bias groups, so one sum per quad is not enough.  The
+// B operand gets a row per (group, digit): row 4g + d holds digit d at the K positions of group g and zeros
+// elsewhere (GS * 4 <= 16 MFMA columns), and a second operand holds a row of ones per group for the bit
+// counts; both are zeroed once, their constant parts written once, and only the digit bytes are rewritten
+// per round.  Every MFMA column then carries one group's sum, is scaled by that group's alpha (lane column
+// c takes the alpha of group c / 4), and the groups are added when the digits are combined at the end.
+constexpr int kGroupedQuadBytes = 20 * 128;  // sixteen digit rows and up to four rows of ones
+constexpr int kGroupedRedBytes = 20 * 64 * 4;  // a wave's final sums: twenty columns of 64 outputs
+
+template <int NB, int GS, int QUADS, int WAVES, bool BIAS>
+__global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a) {
+  constexpr int kWaveBytes = QUADS * kGroupedQuadBytes > kGroupedRedBytes ? QUADS * kGroupedQuadBytes : kGroupedRedBytes;
+  extern __shared__ float lds[];
+  char* xs = reinterpret_cast<char*>(lds);  // [waves][kWaveBytes]: operands in the loop, the final sums after it
+  float* poison_w = reinterpret_cast<float*>(xs + WAVES * kWaveBytes);  // [waves]
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int c = lane & 15, kb = lane >> 4;
+  const int tile = blockIdx.x;
+  const int nquads = a.K >> 7;
+  const size_t n0 = (size_t)tile * 64;
+  const uint32_t col_off = 4u * c;
+  const uint32_t acol = 16u * kb;
+  const int cg = min(c >> 2, GS - 1);  // the group whose sums this lane's MFMA column carries
+  char* xs_w = xs + wv * kWaveBytes;
+  // staging role of a lane, as in bcq_mfma_kernel; its four activations lie in group sg of the quad
+  const int st = lane >> 5, sa = (lane >> 3) & 3, sp = (lane >> 1) & 3, sh = lane & 1;
+  const int e0 = 8 * sp + 4 * sh;
+  const int s_quarter = 2 * (sa & 1) + (e0 >> 4), s_byte = 16 * (sa >> 1) + (e0 & 15);
+  const int sg = (sa * GS) >> 2;
+  constexpr int SP = (QUADS + 1) / 2;
+
+  v8i ones;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) ones[r] = r < 4 ? 0x11111111 : 0;
+  // zero both operands of every quad, then the rows of ones: dword w of a row sits in lane quarter w / 8
+  // at bytes 4 (w % 8), which are MFMA K indices 64 (byte / 16) + 16 quarter + byte % 16
+  {
+    const u4v zero = {0u, 0u, 0u, 0u};
+    for (int i = lane; i < QUADS * kGroupedQuadBytes / 16; i += 64) reinterpret_cast<u4v*>(xs_w)[i] = zero;
+    if (lane < 32) {
+      const int k0 = 64 * ((lane & 7) >> 2) + 16 * (lane >> 3);
+      const int grp = (k0 * GS) >> 7;
+#pragma unroll
+      for (int t = 0; t < QUADS; ++t)
+        *reinterpret_cast<uint32_t*>(xs_w + t * kGroupedQuadBytes + (16 + grp) * 128 + lane * 4) = 0x01010101u;
+    }
+  }
+
+  float tot[4][4], totp[4][4];  // digit columns and bit counts, alpha applied
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) tot[q][i] = totp[q][i] = 0.f;
+  float poison = 0.f;
+
+  for (int q0 = wv * QUADS; q0 < nquads; q0 += WAVES * QUADS) {
+    float xv[SP][4];
+    u4v wq[QUADS][NB];
+#pragma unroll
+    for (int sp_ = 0; sp_ < SP; ++sp_) {
+      const int quad = min(q0 + min(2 * sp_ + st, QUADS - 1), nquads - 1);
+      const _Float16* xp = a.x + (size_t)quad * 128 + 32 * sa + 16 * sh + sp;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xv[sp_][j] = (float)xp[4 * j];
+    }
+#pragma unroll
+    for (int t = 0; t < QUADS; ++t) {
+      const int quad = min(q0 + t, nquads - 1);
+      const uint32_t* wp = a.bW + ((size_t)(4 * quad + kb) * NB) * a.N + n0 + col_off;
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+        wq[t][b] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wp + (size_t)b * a.N));
+    }
+    Half16 al[QUADS][NB], bi[QUADS];
+#pragma unroll
+    for (int t = 0; t < QUADS; ++t) {
+      const int g = min(q0 + t, nquads - 1) * GS + cg;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) al[t][b] = load_half16(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
+      if (BIAS) bi[t] = load_half16(a.qbias + (size_t)g * a.N + n0 + acol);
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int sp_ = 0; sp_ < SP; ++sp_) {
+      const int t = 2 * sp_ + st;
+      const bool live = t < QUADS && q0 + t < nquads;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (!live) xv[sp_][j] = 0.f;
+        poison = fmaf(xv[sp_][j], 0.f, poison);
+        amax = fmaxf(amax, fabsf(xv[sp_][j]));
+      }
+    }
+    const float xmax = wave_max(amax);
+    int E = 13 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
+    E = xmax > 0.f ? max(-120, min(120, E)) : 0;
+    const float scaleE = __uint_as_float((uint32_t)(E + 127) << 23);
+#pragma unroll
+    for (int sp_ = 0; sp_ < SP; ++sp_) {
+      uint32_t ev[4], od[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t u = (uint32_t)((int)rintf(xv[sp_][j] * scaleE) + 0x8888);
+        ev[j] = u & 0x0f0fu;
+        od[j] = (u >> 4) & 0x0f0fu;
+      }
+      const uint32_t pe = __builtin_amdgcn_perm(ev[1], ev[0], 0x05010400u);
+      const uint32_t qe = __builtin_amdgcn_perm(ev[3], ev[2], 0x05010400u);
+      const uint32_t po = __builtin_amdgcn_perm(od[1], od[0], 0x05010400u);
+      const uint32_t qo = __builtin_amdgcn_perm(od[3], od[2], 0x05010400u);
+      const uint32_t dg[4] = {__builtin_amdgcn_perm(qe, pe, 0x05040100u), __builtin_amdgcn_perm(qo, po, 0x05040100u),
+                              __builtin_amdgcn_perm(qe, pe, 0x07060302u), __builtin_amdgcn_perm(qo, po, 0x07060302u)};
+      const int t = 2 * sp_ + st;
+      if (t < QUADS) {
+        char* dst = xs_w + t * kGroupedQuadBytes + (4 * sg) * 128 + s_quarter * 32 + s_byte;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(dst + d * 128) = dg[d];
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    float run[4][4], runp[4][4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) run[q][i] = runp[q][i] = 0.f;
+#pragma unroll
+    for (int t = 0; t < QUADS; ++t) {
+      if (q0 + t >= nquads) break;  // wave-uniform
+      // digit rows: MFMA column c reads row c (rows past 4 GS stay zero and are never used);
+      // rows of ones: column c reads its group's
+      const u4v* bp = reinterpret_cast<const u4v*>(xs_w + t * kGroupedQuadBytes + c * 128 + kb * 32);
+      const u4v* pp = reinterpret_cast<const u4v*>(xs_w + t * kGroupedQuadBytes + (16 + cg) * 128 + kb * 32);
+      const u4v b0 = bp[0], b1 = bp[1], p0 = pp[0], p1 = pp[1];
+      const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+      const v8i P = {(int)p0.x, (int)p0.y, (int)p0.z, (int)p0.w, (int)p1.x, (int)p1.y, (int)p1.z, (int)p1.w};
+      const f4 dsum = mfma_fp4_fp8(ones, B, f4{0.f, 0.f, 0.f, 0.f});
+      const f4 psum = mfma_fp4_fp8(ones, P, f4{0.f, 0.f, 0.f, 0.f});
+      const f4 init = {-0.5f * dsum[0], -0.5f * dsum[1], -0.5f * dsum[2], -0.5f * dsum[3]};
+      const f4 initp = {-0.5f * psum[0], -0.5f * psum[1], -0.5f * psum[2], -0.5f * psum[3]};
+      if (BIAS) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            run[q][i] = fmaf(bi[t].get(4 * i + q), 0.5f * dsum[i], run[q][i]);
+            runp[q][i] = fmaf(bi[t].get(4 * i + q), 0.5f * psum[i], runp[q][i]);
+          }
+      }
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const uint32_t words[4] = {wq[t][b].x, wq[t][b].y, wq[t][b].z, wq[t][b].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v8i A = unpack_bits_fp4(words[q]);
+          const f4 acc = mfma_fp4_fp8(A, B, init);
+          const f4 accp = mfma_fp4_fp8(A, P, initp);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float al_n = al[t][b].get(4 * i + q);
+            run[q][i] = fmaf(al_n, acc[i], run[q][i]);
+            runp[q][i] = fmaf(al_n, accp[i], runp[q][i]);
+          }
+        }
+      }
+    }
+    const float descale = __uint_as_float((uint32_t)(127 - E) << 23);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        tot[q][i] = fmaf(run[q][i], descale, tot[q][i]);
+        totp[q][i] = fmaf(runp[q][i], descale, totp[q][i]);
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+  }
+  // ---- combine digits, groups and waves: the wave's operand area now takes its sums -----------------
+  {
+    const float wp = wave_sum(poison);
+    if (lane == 0) poison_w[wv] = wp;
+  }
+  float* red_w = reinterpret_cast<float*>(xs_w);  // [20][64]: rows 4g + d digits, rows 16 + g bit counts
+  if (c < 4 * GS) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red_w[c * 64 + 16 * kb + 4 * i + q] = tot[q][i];
+  }
+  if (c < 4 * GS && (c & 3) == 0) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red_w[(16 + (c >> 2)) * 64 + 16 * kb + 4 * i + q] = totp[q][i];
+  }
+  __syncthreads();
+  const int n = tile * 64 + tid;
+  if (tid < 64 && n < a.N) {
+    float v = 0.f;
+    for (int w = 0; w < WAVES; ++w) {
+      const float* rw = reinterpret_cast<const float*>(xs + w * kWaveBytes) + tid;
+#pragma unroll
+      for (int g = 0; g < GS; ++g) {
+        const float* rg = rw + 4 * g * 64;
+        v += (((rg[192] * 16.f + rg[128]) * 16.f + rg[64]) * 16.f + rg[0]) - 34952.f * rw[(16 + g) * 64];
+      }
+      v += poison_w[w];
+    }
+    a.y[n] = (_Float16)(v * 2048.f);
+  }
+}
+
+template <int NB, int GS, int QUADS>
+int launch_bcq_grouped(const LutArgs& a, hipStream_t stream) {
+  constexpr int WAVES = 8;
+  constexpr int kWaveBytes = QUADS * kGroupedQuadBytes > kGroupedRedBytes ? QUADS * kGroupedQuadBytes : kGroupedRedBytes;
+  const size_t smem = (size_t)WAVES * kWaveBytes + (size_t)WAVES * 4;
+  const int ntiles = a.N / 64;
+  if (a.qbias)
+    hipLaunchKernelGGL((bcq_mfma_grouped_kernel<NB, GS, QUADS, WAVES, true>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
+  else
+    hipLaunchKernelGGL((bcq_mfma_grouped_kernel<NB, GS, QUADS, WAVES, false>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
+  return hq_launch_status();
+}
+template <int GS>
+int launch_bcq_grouped_nb(const LutArgs& a, hipStream_t stream) {
+  switch (a.nb) {  // quads per wave per round, bounded by the register budget
+    case 1: return launch_bcq_grouped<1, GS, 2>(a, stream);
+    case 2: return launch_bcq_grouped<2, GS, 2>(a, stream);
+    case 3: return launch_bcq_grouped<3, GS, 2>(a, stream);
+    case 4: return launch_bcq_grouped<4, GS, 2>(a, stream);
+    case 5: return launch_bcq_grouped<5, GS, 1>(a, stream);
+    case 6: return launch_bcq_grouped<6, GS, 1>(a, stream);
+    case 7: return launch_bcq_grouped<7, GS, 1>(a, stream);
+    default: return launch_bcq_grouped<8, GS, 1>(a, stream);
+  }
+}
+
 // Eight waves per workgroup (two per SIMD, up to 256 VGPRs each): sixteen-wave variants
 // spill and measured slower.
 template <int NB, int QUADS>
@@ -467,6 +708,15 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
   int rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
 
+  const bool mfma_ok = N % 64 == 0 && K % 128 == 0 && !((uintptr_t)bW & 15) && !((uintptr_t)alpha & 15) &&
+                       !((uintptr_t)q_bias & 15) && hq_env_int("HQ_LUT_PATH", 1) == 1;
+  if (mfma_ok && (group_size == 64 || group_size == 32)) {
+    LutArgs a;
+    a.bW = bW; a.alpha = (const _Float16*)alpha; a.qbias = (const _Float16*)q_bias;
+    a.x = (const _Float16*)x; a.y = (_Float16*)y; a.partial = nullptr; a.counters = nullptr;
+    a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = K; a.nsplit = 1;
+    return group_size == 64 ? launch_bcq_grouped_nb<2>(a, stream) : launch_bcq_grouped_nb<4>(a, stream);
+  }
   if (group_size % 128 == 0 && N % 64 == 0 && !((uintptr_t)bW & 15) && !((uintptr_t)alpha & 15) &&
       !((uintptr_t)q_bias & 15) && hq_env_int("HQ_LUT_PATH", 1) == 1) {
     LutArgs a;

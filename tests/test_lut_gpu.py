@@ -25,7 +25,12 @@ def _run(hq, bW, alpha, qbias, x, group):
     (4096, 16384, 3, 128, True, 1), (4096, 16384, 3, 128, False, 2), (1024, 4096, 8, 128, False, 3),
     (1024, 4096, 4, 128, False, 4), (512, 130, 3, 64, False, 5), (96, 64, 1, 32, False, 6),
     (2048, 1001, 2, 2048, False, 7), (1536, 256, 3, 512, False, 8), (640, 192, 5, 128, False, 9),
-    (8192, 64, 7, 256, False, 10), (384, 128, 6, 384, False, 11)])
+    (8192, 64, 7, 256, False, 10), (384, 128, 6, 384, False, 11),
+    # group sizes 64 and 32: the grouped matrix-core kernel (N % 64 == 0, K % 128 == 0), every plane count
+    (4096, 16384, 3, 64, False, 12), (4096, 4096, 3, 32, False, 13), (1024, 256, 1, 32, False, 14),
+    (2048, 128, 2, 64, True, 15), (1152, 192, 4, 32, False, 16), (640, 64, 5, 64, False, 17),
+    (896, 128, 6, 32, False, 18), (512, 320, 7, 64, False, 19), (1280, 64, 8, 32, False, 20),
+    (128, 64, 3, 32, False, 21), (192, 64, 3, 64, False, 22)])
 def test_vs_oracle(hq, oracle, monkeypatch, path, K, N, nb, group, zero_bias, seed):
     monkeypatch.setenv("HQ_LUT_PATH", str(path))
     bW, alpha, qbias, x = oa.make_lut_problem(seed, K, N, nb, group, zero_bias)
