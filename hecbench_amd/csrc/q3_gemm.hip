@@ -12,12 +12,12 @@
 // (q3_recipe.h).  The factor 2^pos of each operand slot is folded into the
 // activations by a small pre-pass that also reorders them into operand-slot order
 // ([k-group][mfma j][row][8 halves]) and computes the row sums for the zero term.
-// The main kernel streams the weights once: a workgroup (8 waves) owns 128 output
-// columns and all of K and walks K in steps of 16 k-groups; each wave owns two
+// The main kernel streams the weights once: a workgroup (4 waves, one per SIMD) owns 128
+// output columns and all of K and walks K in steps of 8 k-groups; each wave owns two
 // k-groups of a step, loads their activation slices (from L2) and packed rows (from
-// HBM) straight into registers one step ahead, and multiplies 2 k-groups x 128
+// HBM) straight into registers three steps ahead, and multiplies 2 k-groups x 128
 // columns x 64 rows per step with 32x32x16 fp16 MFMAs (fp32 accumulate).  There is
-// no LDS traffic and no barrier in the loop.  The eight waves' accumulators are
+// no LDS traffic and no barrier in the loop.  The four waves' accumulators are
 // summed through LDS at the end and scale/zero are applied once per output.
 #include "hq_internal.h"
 #include "q3_recipe.h"
@@ -30,10 +30,12 @@ typedef float f4v __attribute__((ext_vector_type(4)));
 typedef float f2v __attribute__((ext_vector_type(2)));
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 
-constexpr int kChunk = 16;      // the pre-pass pads K to a multiple of this many k-groups
-constexpr int kWaves = 8;       // two per SIMD
-constexpr int kStepGroups = 16; // k-groups a workgroup consumes per step (two per wave)
-constexpr int kTileN = 128;  // output columns per workgroup
+constexpr int kWaves = 4;       // one per SIMD, up to 512 registers each
+constexpr int kStepGroups = 8;  // k-groups a workgroup consumes per step (two per wave)
+constexpr int kDeep = 3;        // steps of operands in flight ahead of the one being multiplied
+constexpr int kBufs = kDeep + 1;
+constexpr int kChunk = kStepGroups * kBufs;  // the pre-pass pads K to a multiple of this many k-groups
+constexpr int kTileN = 128;     // output columns per workgroup
 
 
 // ---- pre-pass: activations -> operand-slot order, scaled by 2^-pos; row sums ----------------
@@ -130,33 +132,36 @@ struct GemmArgs {
   unsigned flags;
 };
 
+// ---- main kernel -----------------------------------------------------------------------------------
+// One wave per SIMD with up to 512 registers (the accumulators of 64 rows x 128 columns take 128 of them,
+// in the accumulation registers), kDeep steps of operands in flight.  The buffers rotate by unrolling,
+// never by copying: a register move out of a buffer whose load is still in flight would wait for it.
+// (Two waves per SIMD with one step in flight measured 38.4 us at M=64, K=8192, N=28672 against 36.2; the
+// depth itself, 2 to 5 steps, changes little: what a workgroup moves through its CU's L1 - all of the
+// re-ordered activations, 1 MB, next to 0.4 MB of weights - bounds the loop, not the latency.)
 template <int MB>  // 32-row blocks of activations
 __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
   constexpr int Mpad = 32 * MB;
   extern __shared__ u4v lds[];  // used by the final reduction only
-
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int nl = lane & 31, kb = lane >> 5;
   const int G = a.K >> 5;
-  const int nsteps = a.Gpad / kStepGroups;
+  const int nsteps = a.Gpad / kStepGroups;  // a multiple of kBufs: Gpad is a multiple of 32 k-groups
   const int col0 = blockIdx.x * kTileN;
-  const int col = min(col0 + 4 * nl, a.N - 4);  // out-of-range columns re-read valid data, never stored
+  const int col = min(col0 + 4 * nl, a.N - 4);
   const size_t row_stride = (size_t)a.N;
-
-  // what the epilogue needs, fetched while the first operands are on their way
   const int n_out = col0 + 4 * nl;
   f4v sc = {0.f, 0.f, 0.f, 0.f}, zr = {0.f, 0.f, 0.f, 0.f};
-  if (n_out < a.N) {  // N % 4 == 0: the four columns are in range together
+  if (n_out < a.N) {
     sc = *reinterpret_cast<const f4v*>(a.scales + n_out);
     zr = *reinterpret_cast<const f4v*>(a.zeros + n_out);
   }
-  // In the final reduction a wave finishes rows 4*wv .. 4*wv+3 of every 32-row block: half wave kb takes
-  // rows 4*wv + 2*kb and 4*wv + 2*kb + 1, lane nl four adjacent columns.
-  float rs[MB][2];
+  // final reduction: a wave finishes rows 8*wv .. 8*wv+7 of every 32-row block, half wave kb four of them
+  float rs[MB][4];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) rs[mb][j] = a.rowsum[mb * 32 + 4 * wv + 2 * kb + j];
+    for (int j = 0; j < 4; ++j) rs[mb][j] = a.rowsum[mb * 32 + 8 * wv + 4 * kb + j];
 
   f16v acc[MB][4];
 #pragma unroll
@@ -166,11 +171,6 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[mb][q][i] = 0.f;
 
-  // A wave owns k-groups 2*wv + kb of every step of kStepGroups k-groups and loads its
-  // operands straight into registers, one step ahead: the activations of one k-group (4 MFMA K-steps x MB row
-  // blocks, 16 bytes per lane each, 512 contiguous bytes per half wave) and three packed
-  // weight rows.  No LDS and no barrier in the loop: waves drift apart, so one wave's loads
-  // overlap the other waves' MFMAs.
   const u4v* ap_lane = a.Ap + (size_t)((2 * wv + kb) * 4) * Mpad + nl;
   auto load_step = [&](int t, u4v (&A)[4][MB], uint32_t (&wr)[3][4]) {
     const int g = min(t * kStepGroups + 2 * wv + kb, G - 1);  // padded groups: any valid weights, zero activations
@@ -185,51 +185,44 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) A[j][mb] = ap_lane[(size_t)t * (kStepGroups * 4 * Mpad) + j * Mpad + mb * 32];
   };
-
-  u4v Acur[4][MB], Anext[4][MB];
-  uint32_t wcur[3][4], wnext[3][4];
-  load_step(0, Acur, wcur);
-
-  for (int t = 0; t < nsteps; ++t) {
-    // All of the next step's loads are issued before this step's MFMAs, so they have the
-    // whole step to arrive (the last trip re-reads its own step instead of branching).
-    load_step(min(t + 1, nsteps - 1), Anext, wnext);
-    __builtin_amdgcn_sched_barrier(0);
+  auto compute = [&](const u4v (&A)[4][MB], const uint32_t (&wr)[3][4]) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       uint32_t f[16];
-      unpack16(wcur[0][q], wcur[1][q], wcur[2][q], f);
+      unpack16(wr[0][q], wr[1][q], wr[2][q], f);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const u4v bv = {f[4 * j], f[4 * j + 1], f[4 * j + 2], f[4 * j + 3]};
         const h8 B = __builtin_bit_cast(h8, bv);
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          acc[mb][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, Acur[j][mb]), B, acc[mb][q], 0, 0, 0);
+          acc[mb][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, A[j][mb]), B, acc[mb][q], 0, 0, 0);
       }
     }
-    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  u4v Ab[kBufs][4][MB];
+  uint32_t wb[kBufs][3][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+  for (int b = 0; b < kDeep; ++b) load_step(min(b, nsteps - 1), Ab[b], wb[b]);
+  for (int t0 = 0; t0 < nsteps; t0 += kBufs) {
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) Acur[j][mb] = Anext[j][mb];
-#pragma unroll
-    for (int j = 0; j < 3; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) wcur[j][q] = wnext[j][q];
+    for (int b = 0; b < kBufs; ++b) {
+      // step t0 + b is multiplied from buffer b while step t0 + b + kDeep goes into the buffer freed one
+      // step ago (the last trips re-read the last step instead of branching)
+      load_step(min(t0 + b + kDeep, nsteps - 1), Ab[(b + kDeep) % kBufs], wb[(b + kDeep) % kBufs]);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(Ab[b], wb[b]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
   __syncthreads();
 
-  // ---- sum the waves' accumulators through LDS, one 32-row block at a time -------------------
-  // D[row][col = nl]: register i of a lane holds row (i/4)*8 + kb*4 + i%4 of its 32-row block;
-  // the four accumulators q of a lane are four adjacent output columns 4*nl + q.  Every wave writes
-  // its block to its own region ([32][128] floats), then every wave sums four rows over the eight
-  // regions, applies scale / zero and stores them: all waves are busy in both phases.
   float* red = reinterpret_cast<float*>(lds);
   constexpr int REGION = 32 * kTileN;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    if (mb) __syncthreads();  // the previous block has been read
+    if (mb) __syncthreads();
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int r = (i >> 2) * 8 + kb * 4 + (i & 3);
@@ -238,8 +231,8 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
     }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int r = 4 * wv + 2 * kb + j;
+    for (int j = 0; j < 4; ++j) {
+      const int r = 8 * wv + 4 * kb + j;
       const int m = mb * 32 + r;
       f4v v = *reinterpret_cast<const f4v*>(red + r * kTileN + 4 * nl);
 #pragma unroll
@@ -259,7 +252,7 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
 
 template <int MB>
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
-  const size_t smem = (size_t)kWaves * 32 * kTileN * 4;  // one [32][128] fp32 region per wave
+  const size_t smem = (size_t)kWaves * 32 * kTileN * 4;
   static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_gemm_kernel<MB>),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (attr != hipSuccess) return (int)attr;
