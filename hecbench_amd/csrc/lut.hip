@@ -161,12 +161,13 @@ __global__ __launch_bounds__(256) void lut_gemv_kernel(LutArgs a) {
                          __HIP_MEMORY_SCOPE_AGENT);
   }
   if (a.nsplit > 1) {
-    // Split-K arrival counting with relaxed device-scope atomics only: the barrier
-    // waits for this workgroup's write-through partial stores to be acknowledged
-    // before the counter is bumped; the last workgroup to arrive adds the partials in
+    // Split-K arrival counting with relaxed device-scope atomics only: every wave waits
+    // for its write-through partial stores to be acknowledged, then the barrier, then
+    // the counter is bumped; the last workgroup to arrive adds the partials in
     // split order.  Full release/acquire fences would write back and invalidate the
     // whole L2 of the XCD on every workgroup and cost tens of microseconds per call.
     unsigned* s_last = reinterpret_cast<unsigned*>(lds + kTables * 256);
+    __builtin_amdgcn_s_waitcnt(0);  // the stores above are acknowledged (a barrier alone does not wait for them)
     __syncthreads();
     if (tid == 0)
       *s_last = (__hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==

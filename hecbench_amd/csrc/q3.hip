@@ -355,14 +355,15 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     }
   }
   if (a.nsplit > 1) {
-    // Arrival counting with relaxed device-scope atomics only.  The barrier waits for
-    // this workgroup's partial-sum stores to be acknowledged (they are write-through,
-    // so acknowledged means visible device-wide) before the counter is bumped; the last
+    // Arrival counting with relaxed device-scope atomics only.  Every wave waits for its
+    // partial-sum stores to be acknowledged (they are write-through, so acknowledged means
+    // visible device-wide), then the barrier, then the counter is bumped; the last
     // workgroup to arrive reads every partial with device-coherent loads and adds them
     // in split order, so the result does not depend on the arrival order.  Full
     // release/acquire fences are avoided on purpose: on this multi-XCD part they write
     // back and invalidate the whole L2 and cost tens of microseconds per call.
     __shared__ unsigned s_last;
+    __builtin_amdgcn_s_waitcnt(0);  // the stores above are acknowledged (a barrier alone does not wait for them)
     __syncthreads();
     if (tid == 0) {
       const unsigned old = __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
