@@ -1,16 +1,22 @@
 #!/usr/bin/env python3
-"""Benchmark of the GPTQ 3-bit matvec (K=4096, N=11008, fp32 activations) on one
-MI355X: achieved HBM GB/s (algorithmic bytes / time per call) and microseconds per
-call, with weights rotated over more than 512 MB of distinct buffers so that no
-call is served from the 256 MB Infinity Cache.
+"""Benchmark of the weight-only quantized-inference kernels on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--all]
+Headline (the fields `metric`, `value`, `ms_per_step`, `roofline`): the GPTQ 3-bit matvec K=4096, N=11008
+with fp32 activations - achieved HBM GB/s (algorithmic bytes / time per call) and microseconds per call,
+weights rotated over more than 512 MB of distinct buffers so that no call is served from the 256 MB
+Infinity Cache.  The same line carries, under `configs`, the other four benchmark configurations (NF4
+dequantisation, LUT-GEMM, AQLM, batched 3-bit GEMM), each timed the same way with its own roofline object.
 
-Prints ONE JSON line.  A step is one hq_q3_matvec call (one kernel launch)."""
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--windows R] [--no-cpu] [--all]
+
+A step is one library call.  After W warm-up calls, R windows of exactly K back-to-back calls are enqueued
+with a HIP event between windows (on the stream the kernels are launched on); `ms_per_step` is the MEDIAN
+window divided by K, the fastest and slowest windows are reported next to it.  Prints ONE JSON line."""
 import argparse
 import ctypes
 import json
 import os
+import re
 import sys
 import time
 
@@ -24,31 +30,55 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 K, N = 4096, 11008
 ROWS = 3 * K // 32
 ALGO_BYTES = ROWS * N * 4 + 2 * N * 4 + K * 4 + N * 4   # weights + scale/zero + x + y = 17,056,768
-# HBM bytes per launch of the matvec kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by what
-# the same counter reads for a plain 256 MiB device copy (profiles/q3_matvec_4096x11008.txt).
-Q3_TRAFFIC_BYTES = 17267237
 
 
-def _time_loop(fn, n_buffers, steps, warmup):
-    """Event-timed back-to-back launches on torch's current stream (the stream the
-    kernels are enqueued on).  Returns seconds for `steps` calls."""
+def profile_traffic(name):
+    """HBM bytes per launch of the dominant kernel of a configuration: FETCH_SIZE + WRITE_SIZE from two
+    rocprofv3 --pmc runs, each scaled by what the same counter reads for a plain 256 MiB device copy, as
+    recorded in profiles/<name>.txt.  None when the summary is missing."""
+    try:
+        text = open(os.path.join(ROOT, "profiles", name + ".txt")).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic \(fetched \+ written\) per launch: (\d+) bytes", text)
+    return int(m.group(1)) if m else None
+
+
+def _windows_for(steps, windows):
+    if windows:
+        return max(1, windows)
+    # short windows are noisier: more of them (always an odd count, at least 11)
+    return max(11, min(201, (20000 // max(steps, 1)) | 1))
+
+
+def _time_windows(fn, n_buffers, steps, warmup, windows):
+    """R windows of `steps` back-to-back calls on torch's current stream (the stream the kernels are
+    enqueued on), a HIP event between windows, one synchronisation at the end.  Returns the sorted list of
+    seconds per window."""
     import torch
     for i in range(warmup):
         fn(i % n_buffers)
     torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(steps):
-        fn(i % n_buffers)
-    e1.record()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(windows + 1)]
+    k = 0
+    ev[0].record()
+    for w in range(windows):
+        for _ in range(steps):
+            fn(k % n_buffers)
+            k += 1
+        ev[w + 1].record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3
+    return sorted(ev[w].elapsed_time(ev[w + 1]) * 1e-3 for w in range(windows))
 
 
-def bench_q3(steps, warmup, hot=False):
+def _summary(secs, steps):
+    """median / fastest / slowest window as microseconds per call"""
+    med = secs[len(secs) // 2]
+    return med / steps * 1e6, secs[0] / steps * 1e6, secs[-1] / steps * 1e6
+
+
+def bench_q3(steps, warmup, windows, hot=False):
     import torch
-    import hecbench_amd as hq
     from hecbench_amd import _lib
     dev = torch.device("cuda:0")
     lib = _lib.load()
@@ -71,8 +101,118 @@ def bench_q3(steps, warmup, hot=False):
         if rc:
             raise RuntimeError(lib.hq_strerror(rc).decode())
 
-    secs = _time_loop(call, n_buf, steps, warmup)
+    secs = _time_windows(call, n_buf, steps, warmup, windows)
     return secs, dict(x=x, scales=scales, zeros=zeros, mat0=mats[0], y=y, call=call)
+
+
+def _roofline_hbm(algo_bytes, us, profile):
+    gbs = algo_bytes / us / 1e3
+    return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": profile_traffic(profile)}
+
+
+def bench_configs(steps, warmup, windows):
+    """Configurations 0, 2, 3 and 4 of the benchmark: microseconds per call (median window), algorithmic GB/s
+    and the roofline object of each; inputs rotated over more than 512 MB so that every call reads HBM."""
+    import torch
+    from hecbench_amd import _lib
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(99)
+    lib = _lib.load()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {}
+
+    def vp(t):
+        return ctypes.c_void_p(t.data_ptr())
+
+    def check(rc):
+        if rc:
+            raise RuntimeError(lib.hq_strerror(rc).decode())
+
+    def entry(name, workload, algo_bytes, secs, st, profile, **extra):
+        us, lo, hi = _summary(secs, st)
+        e = {"workload": workload, "us_per_call": round(us, 3), "us_per_call_min": round(lo, 3),
+             "us_per_call_max": round(hi, 3), "steps": st, "windows": len(secs),
+             "algorithmic_bytes_per_call": algo_bytes, "GBps": round(algo_bytes / us / 1e3, 1),
+             "roofline": _roofline_hbm(algo_bytes, us, profile)}
+        e.update(extra)
+        out[name] = e
+        return us
+
+    # config 0: NF4 dequant 4096x4096, blocksize 64 (rotate 14 x 43 MB)
+    n = 4096 * 4096
+    nb = 14
+    packed = [torch.randint(0, 256, (n // 2,), dtype=torch.uint8, device=dev, generator=g) for _ in range(nb)]
+    absmax = [torch.empty(n // 64, device=dev).uniform_(0.5, 2.0, generator=g) for _ in range(nb)]
+    outs = [torch.empty(n, dtype=torch.float16, device=dev) for _ in range(nb)]
+    args = [(vp(packed[i]), vp(absmax[i]), vp(outs[i])) for i in range(nb)]
+    secs = _time_windows(lambda i: check(lib.hq_dequant_nf4(args[i][0], args[i][1], args[i][2], n, 64, 0, stream)),
+                         nb, steps, warmup, windows)
+    entry("0_nf4_dequant_4096x4096", "NF4 dequant 4096x4096, blocksize 64, fp16 out, 14 rotated buffer sets (602 MB)",
+          n // 2 + n // 64 * 4 + 64 + n * 2, secs, steps, "nf4_dequant_4096x4096", dtype="f32 multiply -> f16")
+    del packed, absmax, outs
+    # config 2: LUT-GEMM K=4096 N=16384 q=3 G=128 (rotate 20 x 29 MB)
+    Kl, Nl = 4096, 16384
+    nb = 20
+    bW = [torch.randint(-2 ** 31, 2 ** 31 - 1, (Kl // 32, 3, Nl), dtype=torch.int32, device=dev, generator=g)
+          for _ in range(nb)]
+    alpha = [(torch.randn(Kl // 128, 3, Nl, device=dev, generator=g) * 0.02).abs().half() for _ in range(nb)]
+    qb = torch.zeros(Kl // 128, Nl, dtype=torch.float16, device=dev)
+    xl = torch.randn(Kl, device=dev, generator=g).half()
+    yl = torch.empty(Nl, dtype=torch.float16, device=dev)
+    args = [(vp(bW[i]), vp(alpha[i])) for i in range(nb)]
+    pq, px, py = vp(qb), vp(xl), vp(yl)
+    secs = _time_windows(lambda i: check(lib.hq_lut_gemv(args[i][0], args[i][1], pq, px, py, Kl, Nl, 3, 128, stream)),
+                         nb, steps, warmup, windows)
+    entry("2_lut_gemv_4096x16384_q3", "LUT-GEMM K=4096 N=16384, 3 bit planes, group 128, 20 rotated weight sets (566 MB)",
+          Kl // 32 * 3 * Nl * 4 + Kl // 128 * 3 * Nl * 2 + Kl // 128 * Nl * 2 + Kl * 2 + Nl * 2, secs, steps,
+          "lut_gemv_4096x16384_q3", dtype="f16 in, exact integer sums, f32 alpha, f16 out")
+    del bW, alpha
+    # config 3: AQLM 4096x4096 (rotate 128 x 4 MB of codes; the 1 MB code book is shared)
+    Ma, Ka = 4096, 4096
+    nb = 128
+    codes = [torch.randint(-32768, 32768, (Ma, Ka // 8), dtype=torch.int16, device=dev, generator=g)
+             for _ in range(nb)]
+    cb = (torch.randn(65536, 8, device=dev, generator=g) * 0.05).half()
+    sc = torch.empty(Ma, device=dev).uniform_(0.5, 1.5, generator=g).half()
+    xa = torch.randn(Ka, device=dev, generator=g).half()
+    ya = torch.empty(Ma, dtype=torch.float16, device=dev)
+    args = [vp(c) for c in codes]
+    pcb, psc, pxa, pya = vp(cb), vp(sc), vp(xa), vp(ya)
+    sizes = (ctypes.c_int * 4)(Ma, 0, 0, 0)
+    secs = _time_windows(lambda i: check(lib.hq_aqlm_matvec(args[i], pcb, psc, pxa, pya, Ma, Ka, sizes, 65536, stream)),
+                         nb, steps, warmup, windows)
+    us = entry("3_aqlm_4096x4096", "AQLM 1x16 M=4096 K=4096, one code book, 128 rotated code sets (537 MB)",
+               Ma * Ka // 8 * 2 + 65536 * 16 + 3 * Ka * 2, secs, steps, "aqlm_matvec_4096x4096",
+               dtype="f16 in, f32 sums, f16 out")
+    out["3_aqlm_4096x4096"]["gather_GBps"] = round(Ma * Ka // 8 * 16 / us / 1e3, 1)   # 16-byte code-book gathers (L2)
+    del codes
+    # config 4: batched GPTQ 3-bit GEMM M=64 K=8192 N=28672 (rotate 7 x 88 MB)
+    Mg, Kg, Ng = 64, 8192, 28672
+    nb = 7
+    mats = [torch.randint(-2 ** 31, 2 ** 31 - 1, (3 * Kg // 32, Ng), dtype=torch.int32, device=dev, generator=g)
+            for _ in range(nb)]
+    sg = torch.empty(Ng, device=dev).uniform_(0.005, 0.02, generator=g)
+    zg = sg * torch.randint(3, 5, (Ng,), device=dev, generator=g).float()
+    Ag = torch.randn(Mg, Kg, device=dev, generator=g).half()
+    og = torch.empty(Mg, Ng, device=dev)
+    pA, psg, pzg, pog = vp(Ag), vp(sg), vp(zg), vp(og)
+    pm = [vp(m) for m in mats]
+    st = max(10, min(steps, 500))
+    secs = _time_windows(lambda i: check(lib.hq_q3_matvec(pA, 1, pm[i], psg, pzg, pog, Kg, Ng, Mg, 0, stream)),
+                         nb, st, min(warmup, 50), windows)
+    fl = 2.0 * Mg * Kg * Ng
+    us = entry("4_q3_gemm_64x8192x28672", "batched GPTQ 3-bit GEMM M=64 K=8192 N=28672, fp16 activations, 7 rotated "
+               "weight buffers (617 MB); one call = activation pre-pass + main kernel",
+               3 * Kg // 32 * Ng * 4 + 2 * Ng * 4 + Mg * Kg * 2 + Mg * Ng * 4, secs, st, "q3_gemm_64x8192x28672",
+               dtype="f16 MFMA, f32 accumulate")
+    tf = fl / us / 1e6
+    out["4_q3_gemm_64x8192x28672"]["roofline_mfma"] = {"bound": "mfma", "achieved": round(tf, 1),
+                                                       "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                                       "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None}
+    del mats, Ag, og
+    return out
 
 
 def cpu_baseline_q3(state, budget_s=12.0):
@@ -114,15 +254,16 @@ def cpu_baseline_q3(state, budget_s=12.0):
             "gpu_vs_oracle_max_rel_err": err}
 
 
-def bench_others(steps, warmup):
-    """Microseconds per call and algorithmic GB/s of the other configurations."""
+def bench_others(steps, warmup, windows):
+    """The kernels of the neighbouring benchmarks (gemv, mxfp4, quantVLLM, quantBnB): microseconds per call
+    (median window) and algorithmic GB/s."""
     import numpy as np
     import torch
     import hecbench_amd as hq
     from hecbench_amd import _lib
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev)
-    g.manual_seed(99)
+    g.manual_seed(199)
     out = {}
     # raw C-ABI calls with prepared arguments: the Python wrappers cost as much as the short kernels take
     lib = _lib.load()
@@ -135,72 +276,10 @@ def bench_others(steps, warmup):
         if rc:
             raise RuntimeError(lib.hq_strerror(rc).decode())
 
-    # config 0: NF4 dequant 4096x4096, blocksize 64 (rotate 14 x 43 MB)
-    n = 4096 * 4096
-    nb = 14
-    packed = [torch.randint(0, 256, (n // 2,), dtype=torch.uint8, device=dev, generator=g) for _ in range(nb)]
-    absmax = [torch.empty(n // 64, device=dev).uniform_(0.5, 2.0, generator=g) for _ in range(nb)]
-    outs = [torch.empty(n, dtype=torch.float16, device=dev) for _ in range(nb)]
-    args = [(vp(packed[i]), vp(absmax[i]), vp(outs[i])) for i in range(nb)]
-    secs = _time_loop(lambda i: check(lib.hq_dequant_nf4(args[i][0], args[i][1], args[i][2], n, 64, 0, stream)),
-                      nb, steps, warmup)
-    b = n // 2 + n // 64 * 4 + 64 + n * 2
-    out["nf4_dequant_4096x4096"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
-                                    "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
-    del packed, absmax, outs
-    # config 2: LUT-GEMM K=4096 N=16384 q=3 G=128 (rotate 20 x 29 MB)
-    Kl, Nl = 4096, 16384
-    nb = 20
-    bW = [torch.randint(-2 ** 31, 2 ** 31 - 1, (Kl // 32, 3, Nl), dtype=torch.int32, device=dev, generator=g)
-          for _ in range(nb)]
-    alpha = [(torch.randn(Kl // 128, 3, Nl, device=dev, generator=g) * 0.02).abs().half() for _ in range(nb)]
-    qb = torch.zeros(Kl // 128, Nl, dtype=torch.float16, device=dev)
-    xl = torch.randn(Kl, device=dev, generator=g).half()
-    yl = torch.empty(Nl, dtype=torch.float16, device=dev)
-    args = [(vp(bW[i]), vp(alpha[i])) for i in range(nb)]
-    pq, px, py = vp(qb), vp(xl), vp(yl)
-    secs = _time_loop(lambda i: check(lib.hq_lut_gemv(args[i][0], args[i][1], pq, px, py, Kl, Nl, 3, 128, stream)),
-                      nb, steps, warmup)
-    b = Kl // 32 * 3 * Nl * 4 + Kl // 128 * 3 * Nl * 2 + Kl // 128 * Nl * 2 + Kl * 2 + Nl * 2
-    out["lut_gemv_4096x16384_q3"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
-                                     "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS}
-    del bW, alpha
-    # config 3: AQLM 4096x4096 (rotate 128 x 4 MB of codes; the 1 MB code book is shared)
-    Ma, Ka = 4096, 4096
-    nb = 128
-    codes = [torch.randint(-32768, 32768, (Ma, Ka // 8), dtype=torch.int16, device=dev, generator=g)
-             for _ in range(nb)]
-    cb = (torch.randn(65536, 8, device=dev, generator=g) * 0.05).half()
-    sc = torch.empty(Ma, device=dev).uniform_(0.5, 1.5, generator=g).half()
-    xa = torch.randn(Ka, device=dev, generator=g).half()
-    ya = torch.empty(Ma, dtype=torch.float16, device=dev)
-    args = [vp(c) for c in codes]
-    pcb, psc, pxa, pya = vp(cb), vp(sc), vp(xa), vp(ya)
-    sizes = (ctypes.c_int * 4)(Ma, 0, 0, 0)
-    secs = _time_loop(lambda i: check(lib.hq_aqlm_matvec(args[i], pcb, psc, pxa, pya, Ma, Ka, sizes, 65536, stream)),
-                      nb, steps, warmup)
-    b = Ma * Ka // 8 * 2 + 65536 * 16 + 3 * Ka * 2
-    out["aqlm_4096x4096"] = {"us": secs / steps * 1e6, "GBps": b * steps / secs / 1e9,
-                             "frac_hbm": b * steps / secs / 1e9 / HBM_PEAK_GBS,
-                             "gather_GBps": (Ma * Ka // 8 * 16) * steps / secs / 1e9}
-    # config 4: batched GPTQ 3-bit GEMM M=64 K=8192 N=28672 (rotate 7 x 88 MB)
-    Mg, Kg, Ng = 64, 8192, 28672
-    nb = 7
-    mats = [torch.randint(-2 ** 31, 2 ** 31 - 1, (3 * Kg // 32, Ng), dtype=torch.int32, device=dev, generator=g)
-            for _ in range(nb)]
-    sg = torch.empty(Ng, device=dev).uniform_(0.005, 0.02, generator=g)
-    zg = sg * torch.randint(3, 5, (Ng,), device=dev, generator=g).float()
-    Ag = torch.randn(Mg, Kg, device=dev, generator=g).half()
-    og = torch.empty(Mg, Ng, device=dev)
-    st = max(50, steps // 4)
-    secs = _time_loop(lambda i: hq.q3_gemm(Ag, mats[i], sg, zg, out=og), nb, st, 10)
-    b = 3 * Kg // 32 * Ng * 4 + 2 * Ng * 4 + Mg * Kg * 2 + Mg * Ng * 4
-    fl = 2.0 * Mg * Kg * Ng
-    out["q3_gemm_64x8192x28672"] = {"us": secs / st * 1e6, "GBps": b * st / secs / 1e9,
-                                    "frac_hbm": b * st / secs / 1e9 / HBM_PEAK_GBS,
-                                    "TFLOPs": fl * st / secs / 1e12,
-                                    "frac_mfma_f16": fl * st / secs / 1e12 / MFMA_F16_PEAK_TFLOPS}
-    del mats, Ag, og
+    def _time_loop(fn, n_buffers, st, wu):
+        secs = _time_windows(fn, n_buffers, st, wu, windows)
+        return secs[len(secs) // 2]
+
     # next rows: dense / int8 / int4 gemv at the reference's run size 16384 x 16384 (the weight buffers are
     # rotated so that at least 512 MB of distinct data passes between two uses of a buffer) and mxfp4
     # quantise-dequantise of 4096 x 4096 fp16 elements (rotate 16 x 67 MB)
@@ -353,10 +432,13 @@ def reference_quantbnb_omp():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--windows", type=int, default=0,
+                    help="timed windows of --steps calls (default: 11, more when --steps is small)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--all", action="store_true", help="also time the other configurations")
+    ap.add_argument("--no-configs", action="store_true", help="time the headline configuration only")
+    ap.add_argument("--all", action="store_true", help="also time the kernels of the neighbouring benchmarks")
     ap.add_argument("--no-hot", action="store_true", help="skip the hot-cache (single buffer) timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 20 plain device copies of 256 MiB (reference point for rocprofv3 "
@@ -366,6 +448,9 @@ def main():
         print("bench.py measures one GPU: this path has no collective and every box here has one GPU; "
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.steps < 1 or args.warmup < 0:
+        print("--steps must be >= 1 and --warmup >= 0", file=sys.stderr)
+        sys.exit(2)
     import torch
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (no CPU path exists for the product kernels)", file=sys.stderr)
@@ -373,6 +458,7 @@ def main():
     import hecbench_amd as hq
     hq.init()
     info = hq.device_info()
+    windows = _windows_for(args.steps, args.windows)
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_()
@@ -382,10 +468,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    secs, state = bench_q3(args.steps, args.warmup)
-    us = secs / args.steps * 1e6
-    gbs = ALGO_BYTES / (secs / args.steps) / 1e9
-    hot_secs = None if args.no_hot else bench_q3(args.steps, args.warmup, hot=True)[0]
+    secs, state = bench_q3(args.steps, args.warmup, windows)
+    us, us_min, us_max = _summary(secs, args.steps)
+    gbs = ALGO_BYTES / us / 1e3
+    hot_us = None if args.no_hot else _summary(bench_q3(args.steps, args.warmup, windows, hot=True)[0], args.steps)[0]
     result = {
         "metric": "achieved HBM GB/s: GPTQ-3bit matvec 4096x11008 (algorithmic bytes / time per call)",
         "value": round(gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -393,24 +479,37 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "GPTQ 3-bit matvec K=4096 N=11008 batch 1, fp32 x, weights rotated over 34 "
                                "distinct 16.9 MB buffers (575 MB)", "algorithmic_bytes_per_call": ALGO_BYTES},
+        "windows": windows, "ms_per_step_min": round(us_min * 1e-3, 6), "ms_per_step_max": round(us_max * 1e-3, 6),
+        "timing": f"median of {windows} windows of {args.steps} back-to-back calls, HIP events on the launch stream",
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
-        "effective_fp16_weight_GBps": round(K * N * 2 / (secs / args.steps) / 1e9, 1),
-        "hot_cache_us_per_call": None if hot_secs is None else round(hot_secs / args.steps * 1e6, 3),
+        "effective_fp16_weight_GBps": round(K * N * 2 / us / 1e3, 1),
+        "hot_cache_us_per_call": None if hot_us is None else round(hot_us, 3),
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": Q3_TRAFFIC_BYTES},
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": profile_traffic("q3_matvec_4096x11008")},
         "device": info,
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_q3(state)
+    del state
+    if not args.no_configs:
+        # the other four benchmark configurations: a few thousand calls each at most
+        st = max(1, min(args.steps, 1000))
+        result["configs"] = bench_configs(st, min(args.warmup, 100), _windows_for(st, args.windows))
     if args.all:
-        result["other_configs"] = bench_others(max(200, args.steps // 8), 50)
+        st = max(20, min(args.steps // 4, 500))
+        result["other_kernels"] = bench_others(st, 20, 11)
         if not args.no_cpu:
-            for name, cpu in cpu_others().items():
-                result["other_configs"][name]["cpu_serial"] = {"us": round(cpu["cpu_us"], 1), "cores": 1,
-                                                               "kind": cpu.get("kind", "port"),
-                                                               "sample": cpu["sample"]}
-                if "reference_omp" in cpu:
-                    result["other_configs"][name]["cpu_reference_omp"] = cpu["reference_omp"]
+            cpu = cpu_others()
+            for name, c in cpu.items():
+                tgt = result["other_kernels"].get(name)
+                if tgt is None and not args.no_configs:
+                    tgt = next((v for k, v in result["configs"].items() if k[2:] == name), None)
+                if tgt is None:
+                    continue
+                tgt["cpu_serial"] = {"us": round(c["cpu_us"], 1), "cores": 1, "kind": c.get("kind", "port"),
+                                     "sample": c["sample"]}
+                if "reference_omp" in c:
+                    tgt["cpu_reference_omp"] = c["reference_omp"]
     print(json.dumps(result))
 
 

@@ -16,6 +16,9 @@ _SIGNATURES = {
     "hq_abi_version": (_c.c_int, []),
     "hq_strerror": (_c.c_char_p, [_c.c_int]),
     "hq_init": (_c.c_int, []),
+    "hq_reserve_workspace": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int]),
+    "hq_shutdown": (_c.c_int, []),
+    "hq_set_tunable": (_c.c_int, [_c.c_char_p, _c.c_int, _c.c_int]),
     "hq_device_info": (_c.c_int, [_c.POINTER(_c.c_int)] * 5 + [_c.c_char_p, _c.c_int]),
     "hq_dequant_nf4": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int,
                                   _c.c_int, _c.c_void_p]),

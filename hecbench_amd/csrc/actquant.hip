@@ -408,7 +408,7 @@ void launch_dynamic_vec(const T* in, int8_t* out, float* scales, int32_t* azps, 
   const int span = (hidden + kVec - 1) / kVec + 1 + 63;  // units from the 64-unit boundary before a ragged row to its end
   const int need = (span + lanes - 1) / lanes;
   const int64_t groups = wave_rows ? (tokens + 3) / 4 : tokens;
-  const dim3 grid((unsigned)std::min<int64_t>(groups, (int64_t)dev->cus * hq_env_int("HQ_ACTQ_GROUPS", 8))), block(256);
+  const dim3 grid((unsigned)std::min<int64_t>(groups, (int64_t)dev->cus * hq_tune(HQ_TUNE_ACTQ_GROUPS, 8))), block(256);
 #define HQ_ROWS(LANES, KEEP, R)                                                                                   \
   hipLaunchKernelGGL((dynamic_quant_kernel<T, AZP, LANES, KEEP, R, VEC>), grid, block, 0, stream, in, out, scales, \
                      azps, tokens, hidden)

@@ -1,9 +1,13 @@
 // Library-wide state of libhq: device facts, per-stream workspaces, error text.
+#include <atomic>
+#include <climits>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
 #include <utility>
+#include <vector>
 
 #include "hq_internal.h"
 
@@ -11,14 +15,50 @@ namespace {
 std::mutex g_mu;
 std::map<int, HqDevice> g_devices;
 std::map<std::pair<int, hipStream_t>, HqWorkspace> g_workspaces;
+std::vector<std::pair<int, void*>> g_retired;  // outgrown buffers, freed by hq_shutdown()
 }  // namespace
 
-int hq_env_int(const char* name, int dflt) {
-  const char* v = std::getenv(name);
-  if (!v || !*v) return dflt;
-  char* end = nullptr;
-  long r = std::strtol(v, &end, 10);
-  return (end && *end == '\0') ? (int)r : dflt;
+// ---- launch-shape overrides ------------------------------------------------------------------
+// Every knob is an int that is "unset" by default.  The environment variable of the same name is
+// read ONCE (first use), hq_set_tunable() changes a knob at run time; a launch path reads a knob
+// with one relaxed atomic load, never the environment.
+namespace {
+const char* const kTunableNames[HQ_TUNE_COUNT] = {
+    "HQ_Q3_WAVES", "HQ_Q3_STEPS", "HQ_Q3_KSPLIT", "HQ_Q3_SMALL_BATCH", "HQ_LUT_PATH", "HQ_LUT_KSPLIT", "HQ_NF4_PIPE",
+    "HQ_AQLM_ROWS", "HQ_Q8_WGS", "HQ_Q8_FAST", "HQ_ACTQ_GROUPS", "HQ_SPLITK_FENCES"};
+constexpr int kUnset = INT_MIN;
+std::atomic<int> g_tunables[HQ_TUNE_COUNT];
+std::once_flag g_tunables_once;
+
+void seed_tunables_from_env() {
+  for (int i = 0; i < HQ_TUNE_COUNT; ++i) {
+    int v = kUnset;
+    const char* e = std::getenv(kTunableNames[i]);
+    if (e && *e) {
+      char* end = nullptr;
+      const long r = std::strtol(e, &end, 10);
+      if (end && *end == '\0') v = (int)r;
+    }
+    g_tunables[i].store(v, std::memory_order_relaxed);
+  }
+}
+}  // namespace
+
+int hq_tune(HqTunable id, int dflt) {
+  std::call_once(g_tunables_once, seed_tunables_from_env);
+  const int v = g_tunables[id].load(std::memory_order_relaxed);
+  return v == kUnset ? dflt : v;
+}
+
+extern "C" int hq_set_tunable(const char* name, int value, int clear) {
+  if (!name) return HQ_ERR_NULL_POINTER;
+  std::call_once(g_tunables_once, seed_tunables_from_env);
+  for (int i = 0; i < HQ_TUNE_COUNT; ++i)
+    if (std::strcmp(name, kTunableNames[i]) == 0) {
+      g_tunables[i].store(clear ? kUnset : value, std::memory_order_relaxed);
+      return HQ_OK;
+    }
+  return HQ_ERR_BAD_ENUM;
 }
 
 int hq_current_device(const HqDevice** out) {
@@ -48,23 +88,68 @@ int hq_get_workspace(hipStream_t stream, size_t need_floats, size_t need_counter
   std::lock_guard<std::mutex> lk(g_mu);
   HqWorkspace& ws = g_workspaces[std::make_pair(dev, stream)];
   if (ws.partial_floats < need_floats) {
-    size_t n = need_floats < (1u << 20) ? (1u << 20) : need_floats;
+    // grow geometrically: a stream that sees larger and larger problems allocates O(log) times
+    size_t n = ws.partial_floats ? ws.partial_floats * 2 : (size_t)1 << 20;
+    while (n < need_floats) n *= 2;
     float* p = nullptr;
     HQ_HIP_TRY(hipMalloc((void**)&p, n * sizeof(float)));
-    // The previous buffer may still be read by kernels in flight: keep it.
+    // kernels in flight may still read the previous buffer: it is kept until hq_shutdown()
+    if (ws.partial) g_retired.push_back(std::make_pair(dev, (void*)ws.partial));
     ws.partial = p;
     ws.partial_floats = n;
   }
   if (ws.ncounters < need_counters) {
-    size_t n = need_counters < (1u << 14) ? (1u << 14) : need_counters;
+    size_t n = ws.ncounters ? ws.ncounters * 2 : (size_t)1 << 14;
+    while (n < need_counters) n *= 2;
     unsigned* c = nullptr;
     HQ_HIP_TRY(hipMalloc((void**)&c, n * sizeof(unsigned)));
     HQ_HIP_TRY(hipMemset(c, 0, n * sizeof(unsigned)));
+    if (ws.counters) g_retired.push_back(std::make_pair(dev, (void*)ws.counters));
     ws.counters = c;
     ws.ncounters = n;
   }
   *out = ws;
   return HQ_OK;
+}
+
+extern "C" int hq_reserve_workspace(void* stream, int max_K, int max_N) {
+  if (max_K < 0 || max_N < 0) return HQ_ERR_BAD_SHAPE;
+  const HqDevice* d = nullptr;
+  int rc = hq_current_device(&d);
+  if (rc != HQ_OK) return rc;
+  // batched GEMM: re-ordered activations of 64 rows (128 bytes per input feature, K padded to 1024) plus
+  // the row sums and scales; split-K matvecs: at most one partial row of 64 floats per compute unit
+  const size_t kpad = ((size_t)max_K + 1023) / 1024 * 1024;
+  const size_t gemm_floats = kpad * 32 + 128;
+  const size_t tiles = ((size_t)max_N + 63) / 64;
+  const size_t split_floats = (tiles > (size_t)d->cus ? tiles : (size_t)d->cus) * 64 * 2;
+  HqWorkspace ws;
+  return hq_get_workspace((hipStream_t)stream, gemm_floats > split_floats ? gemm_floats : split_floats,
+                          tiles > 1 ? tiles : 1, &ws);
+}
+
+extern "C" int hq_shutdown(void) {
+  HQ_HIP_TRY(hipDeviceSynchronize());
+  std::lock_guard<std::mutex> lk(g_mu);
+  int cur = 0;
+  HQ_HIP_TRY(hipGetDevice(&cur));
+  int rc = HQ_OK;
+  auto release = [&](int dev, void* p) {
+    if (!p) return;
+    hipError_t e = hipSetDevice(dev);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipFree(p);
+    if (e != hipSuccess && rc == HQ_OK) rc = (int)e;
+  };
+  for (auto& kv : g_workspaces) {
+    release(kv.first.first, kv.second.partial);
+    release(kv.first.first, kv.second.counters);
+  }
+  for (auto& r : g_retired) release(r.first, r.second);
+  g_workspaces.clear();
+  g_retired.clear();
+  (void)hipSetDevice(cur);
+  return rc;
 }
 
 extern "C" int hq_abi_version(void) { return 1; }

@@ -121,7 +121,7 @@ extern "C" int hq_aqlm_matvec(const int16_t* codes, const void* codebooks, const
   for (int j = 0; j < 4; ++j) a.cb_sizes[j] = cb_a_sizes[j];
   // Rows per wave: keep at least ~8 waves per CU in flight (mirrors the CU-count
   // based sizing of the reference launcher, src/quantAQLM-hip/main.cu:108-121).
-  int rows = hq_env_int("HQ_AQLM_ROWS", 0);
+  int rows = hq_tune(HQ_TUNE_AQLM_ROWS, 0);
   if (rows != 1 && rows != 2 && rows != 4) {
     const long waves_wanted = (long)dev->cus * 8;
     rows = (M >= 4 * waves_wanted) ? 4 : (M >= 2 * waves_wanted ? 2 : 1);

@@ -6,6 +6,9 @@
 
 #include "../../include/hq.h"
 
+// internal flag bit of the split-K kernels: formal release/acquire fences in the arrival protocol
+#define HQ_FLAG_STRICT_FENCES 0x80000000u
+
 #define HQ_HIP_TRY(expr)                      \
   do {                                        \
     hipError_t hq_e_ = (expr);                \
@@ -36,10 +39,15 @@ struct HqWorkspace {
 };
 
 // Workspace of (current device, stream) holding at least the requested sizes.
-// Allocated on first use and grown on demand; never freed while the process runs.
+// Allocated on first use, grown geometrically on demand, freed by hq_shutdown().
 int hq_get_workspace(hipStream_t stream, size_t need_floats, size_t need_counters,
                      HqWorkspace* out);
 
-// Integer tuning knob from the environment (used by the benchmark drivers to
-// sweep launch shapes); returns dflt when unset or unparsable.
-int hq_env_int(const char* name, int dflt);
+// Launch-shape overrides for tests and sweeps (hq_set_tunable, or the environment variable of the
+// same name, which is read once per process).  hq_tune returns dflt while a knob is unset; it costs
+// one relaxed atomic load.
+enum HqTunable {
+  HQ_TUNE_Q3_WAVES, HQ_TUNE_Q3_STEPS, HQ_TUNE_Q3_KSPLIT, HQ_TUNE_Q3_SMALL_BATCH, HQ_TUNE_LUT_PATH, HQ_TUNE_LUT_KSPLIT,
+  HQ_TUNE_NF4_PIPE, HQ_TUNE_AQLM_ROWS, HQ_TUNE_Q8_WGS, HQ_TUNE_Q8_FAST, HQ_TUNE_ACTQ_GROUPS, HQ_TUNE_SPLITK_FENCES, HQ_TUNE_COUNT
+};
+int hq_tune(HqTunable id, int dflt);

@@ -35,6 +35,7 @@ struct LutArgs {
   int K, N, nb, G;
   int kslice;  // K elements per workgroup (multiple of 512)
   int nsplit;
+  int strict;  // formal release/acquire in the split-K arrival (HQ_SPLITK_FENCES)
 };
 
 constexpr int kStepK = 512;        // K elements tabulated per iteration
@@ -161,18 +162,20 @@ __global__ __launch_bounds__(256) void lut_gemv_kernel(LutArgs a) {
                          __HIP_MEMORY_SCOPE_AGENT);
   }
   if (a.nsplit > 1) {
-    // Split-K arrival counting with relaxed device-scope atomics only: every wave waits
-    // for its write-through partial stores to be acknowledged, then the barrier, then
-    // the counter is bumped; the last workgroup to arrive adds the partials in
-    // split order.  Full release/acquire fences would write back and invalidate the
-    // whole L2 of the XCD on every workgroup and cost tens of microseconds per call.
+    // Split-K arrival counting with relaxed device-scope atomics only (the protocol and what it rests
+    // on are spelled out at the same place in q3.hip): write-through partial stores, wait for their
+    // acknowledgement, workgroup fence + barrier, one device-scope fetch-add, and the last workgroup
+    // to arrive adds the partials in split order.  a.strict selects formal release/acquire instead.
     unsigned* s_last = reinterpret_cast<unsigned*>(lds + kTables * 256);
     __builtin_amdgcn_s_waitcnt(0);  // the stores above are acknowledged (a barrier alone does not wait for them)
     __syncthreads();
-    if (tid == 0)
-      *s_last = (__hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
-                 (unsigned)(a.nsplit - 1));
+    if (tid == 0) {
+      const unsigned old = a.strict ? __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT)
+                                    : __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *s_last = (old == (unsigned)(a.nsplit - 1));
+    }
     __syncthreads();
+    if (*s_last && a.strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     if (*s_last) {
       if (tid < 64 * CPL && n < a.N) {
         float sum = 0.f;
@@ -710,20 +713,20 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
   if (rc != HQ_OK) return rc;
 
   const bool mfma_ok = N % 64 == 0 && K % 128 == 0 && !((uintptr_t)bW & 15) && !((uintptr_t)alpha & 15) &&
-                       !((uintptr_t)q_bias & 15) && hq_env_int("HQ_LUT_PATH", 1) == 1;
+                       !((uintptr_t)q_bias & 15) && hq_tune(HQ_TUNE_LUT_PATH, 1) == 1;
   if (mfma_ok && (group_size == 64 || group_size == 32)) {
     LutArgs a;
     a.bW = bW; a.alpha = (const _Float16*)alpha; a.qbias = (const _Float16*)q_bias;
     a.x = (const _Float16*)x; a.y = (_Float16*)y; a.partial = nullptr; a.counters = nullptr;
-    a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = K; a.nsplit = 1;
+    a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = K; a.nsplit = 1; a.strict = 0;
     return group_size == 64 ? launch_bcq_grouped_nb<2>(a, stream) : launch_bcq_grouped_nb<4>(a, stream);
   }
   if (group_size % 128 == 0 && N % 64 == 0 && !((uintptr_t)bW & 15) && !((uintptr_t)alpha & 15) &&
-      !((uintptr_t)q_bias & 15) && hq_env_int("HQ_LUT_PATH", 1) == 1) {
+      !((uintptr_t)q_bias & 15) && hq_tune(HQ_TUNE_LUT_PATH, 1) == 1) {
     LutArgs a;
     a.bW = bW; a.alpha = (const _Float16*)alpha; a.qbias = (const _Float16*)q_bias;
     a.x = (const _Float16*)x; a.y = (_Float16*)y; a.partial = nullptr; a.counters = nullptr;
-    a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = K; a.nsplit = 1;
+    a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = K; a.nsplit = 1; a.strict = 0;
     switch (nbits) {  // quads per wave per round, bounded by the register budget
       case 1: return launch_bcq_mfma<1, 2>(a, stream);
       case 2: return launch_bcq_mfma<2, 2>(a, stream);
@@ -739,7 +742,7 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
   const int cpl = pair ? 2 : 1;
   const int ntiles = (N + 64 * cpl - 1) / (64 * cpl);
   // K slice per workgroup: enough workgroups to cover the CUs about twice.
-  int nsplit = hq_env_int("HQ_LUT_KSPLIT", 0);
+  int nsplit = hq_tune(HQ_TUNE_LUT_KSPLIT, 0);
   const int steps = (K + kStepK - 1) / kStepK;
   if (nsplit <= 0) {
     nsplit = (2 * dev->cus + ntiles - 1) / ntiles;
@@ -752,7 +755,7 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
   LutArgs a;
   a.bW = bW; a.alpha = (const _Float16*)alpha; a.qbias = (const _Float16*)q_bias;
   a.x = (const _Float16*)x; a.y = (_Float16*)y; a.partial = nullptr; a.counters = nullptr;
-  a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = steps_per * kStepK; a.nsplit = nsplit;
+  a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = steps_per * kStepK; a.nsplit = nsplit; a.strict = hq_tune(HQ_TUNE_SPLITK_FENCES, 0);
   if (nsplit > 1) {
     HqWorkspace ws;
     rc = hq_get_workspace(stream, (size_t)ntiles * nsplit * 64 * cpl, (size_t)ntiles, &ws);

@@ -7,8 +7,12 @@
 // shared scale is 2^(e-2) clamped to the E8M0 range (main.cu:128-132), and every element
 // becomes scale * e2m1(x / scale), where e2m1() rounds to the nearest of 0, .5, 1, 1.5, 2,
 // 3, 4, 6 (ties to the even mantissa, saturating at 6, sign kept).  Bit-exact with the
-// reference for finite inputs whose group maximum does not round to zero (there the
-// reference divides by a zero scale; this kernel writes signed zeros).
+// reference for finite inputs, with two exceptions where the reference's own arithmetic breaks down:
+// a group maximum that rounds to zero (the reference divides by a zero scale; this kernel writes signed
+// zeros), and a group maximum whose rounding to a power of two leaves the format (fp16 >= 61440, bf16 >=
+// 0x7f60: the reference takes log2 of an infinity and writes NaN for the whole group; this kernel uses the
+// scale the carry stands for, 2^14 or 2^126, and writes finite values, the maximum itself becoming
+// infinity).
 //
 // HBM-bound: 4 bytes per element.  A lane owns 8 consecutive elements (one 128-bit load, one
 // 128-bit nontemporal store), a group is 4 adjacent lanes, and the group maximum takes two

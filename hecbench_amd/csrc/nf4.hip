@@ -187,7 +187,7 @@ extern "C" int hq_dequant_nf4(const uint8_t* packed, const float* absmax, void* 
                        (u4v*)out_fp16, nwords, blocksize, shift, table);
     // Pipelined variant, four workgroups per CU: measured 7.5 us against 7.8 us at 4096x4096 and 26.2
     // against 27.1 us at 2^26 elements, but 4 % slower at 2^30, so it is kept to the mid sizes.
-    int pipe = hq_env_int("HQ_NF4_PIPE", -1);
+    int pipe = hq_tune(HQ_TUNE_NF4_PIPE, -1);
     if (pipe < 0) pipe = (nwords >= (1 << 19) && nwords <= (1 << 25)) ? 4 : 0;
     if (mode == 0 && pipe > 0) {
       constexpr int PU = 4;

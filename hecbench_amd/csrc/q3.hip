@@ -325,7 +325,10 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     }
   }
   if (lane == 0) wsum[wv] = asum_total;
-  __syncthreads();
+  // the digit rows written above are read back by this wave only: a wave-local fence, no workgroup barrier
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
   {
     const float* rw = red + (wv * 8) * kRedStride + lane;
     float h = rw[7 * kRedStride];
@@ -346,7 +349,9 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     val = fmaf(xsum, 0.f, val);  // a NaN or infinity among the activations makes the result NaN (the
                                  // fixed-point digits cannot carry it)
     if (a.nsplit == 1) {
-      a.y[n] = y_old + val;
+      // Write-through store: the result is on its way to memory at once instead of waiting in this
+      // XCD's L2 for the write-back at the end of the kernel (the last store of a kernel is exposed).
+      __hip_atomic_store(&a.y[n], y_old + val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
       // Device-coherent (write-through) store: visible to the other XCDs' workgroups
       // without flushing or invalidating this XCD's L2.
@@ -355,21 +360,30 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     }
   }
   if (a.nsplit > 1) {
-    // Arrival counting with relaxed device-scope atomics only.  Every wave waits for its
-    // partial-sum stores to be acknowledged (they are write-through, so acknowledged means
-    // visible device-wide), then the barrier, then the counter is bumped; the last
-    // workgroup to arrive reads every partial with device-coherent loads and adds them
-    // in split order, so the result does not depend on the arrival order.  Full
-    // release/acquire fences are avoided on purpose: on this multi-XCD part they write
-    // back and invalidate the whole L2 and cost tens of microseconds per call.
+    // Arrival counting.  Default protocol, relaxed device-scope atomics only:
+    //  (1) the partial sums above are device-scope atomic stores, i.e. write-through stores that are
+    //      acknowledged only once they are visible to every XCD;
+    //  (2) every wave waits for those acknowledgements (vmcnt 0);
+    //  (3) __syncthreads: a workgroup-scope fence plus barrier - the compiler moves no memory access
+    //      across it, and after it all of the workgroup's partial sums are visible device-wide;
+    //  (4) one device-scope fetch-add per workgroup, performed at the memory side;
+    //  (5) the last workgroup to arrive reads every partial with device-scope atomic loads, which
+    //      bypass the non-coherent levels, and adds them in split order (deterministic result).
+    // What this rests on is the gfx950 cache policy of device-scope atomic accesses (they do not stay
+    // in an XCD's L2).  A formal release/acquire pair at device scope writes back and invalidates the
+    // whole L2 of the XCD and costs tens of microseconds per call; HQ_FLAG_STRICT_FENCES (set from the
+    // HQ_SPLITK_FENCES knob) selects it, for checking that both give the same result.
     __shared__ unsigned s_last;
-    __builtin_amdgcn_s_waitcnt(0);  // the stores above are acknowledged (a barrier alone does not wait for them)
+    const bool strict = (a.flags & HQ_FLAG_STRICT_FENCES) != 0;
+    __builtin_amdgcn_s_waitcnt(0);  // (2): a barrier alone does not wait for outstanding stores
     __syncthreads();
     if (tid == 0) {
-      const unsigned old = __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned old = strict ? __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT)
+                                  : __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       s_last = (old == (unsigned)(a.nsplit - 1));
     }
     __syncthreads();
+    if (s_last && strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     if (s_last) {
       if (tid < 64 && n < a.N) {
         float sum = 0.f;
@@ -418,6 +432,7 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   if (!x || !qweight || !scales || !zeros || !y) return HQ_ERR_NULL_POINTER;
   if (x_dtype != HQ_DTYPE_F32 && x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
   if (flags & ~HQ_FLAG_ACCUMULATE) return HQ_ERR_BAD_ENUM;
+  if (hq_tune(HQ_TUNE_SPLITK_FENCES, 0)) flags |= HQ_FLAG_STRICT_FENCES;
   if (K <= 0 || N <= 0 || batch_M <= 0 || (K & 31) || (N & 3)) return HQ_ERR_BAD_SHAPE;
   if (((uintptr_t)qweight & 15) || ((uintptr_t)x & 15) ||  // activations are read with 128-bit loads
       ((uintptr_t)y & 3) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
@@ -436,8 +451,8 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   // walks its K range in rounds (the next round's loads are in flight during the current
   // one).  K is split across workgroups only as far as needed to give every CU a
   // workgroup: the split costs a device-scope round trip per workgroup.
-  int waves = hq_env_int("HQ_Q3_WAVES", 8);
-  int steps = hq_env_int("HQ_Q3_STEPS", 0);
+  int waves = hq_tune(HQ_TUNE_Q3_WAVES, 8);
+  int steps = hq_tune(HQ_TUNE_Q3_STEPS, 0);
   if (waves != 4 && waves != 8 && waves != 16) waves = 8;
   if (waves == 16) steps = 1;  // register budget of 16-wave workgroups
   if (steps != 1 && steps != 2 && steps != 4 && (steps != 8 || waves != 4)) {
@@ -446,7 +461,7 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   }
   const int gpr = waves * 4 * steps;  // k-groups one workgroup covers per round
   const int max_split = (G + gpr - 1) / gpr;
-  int nsplit = hq_env_int("HQ_Q3_KSPLIT", 0);
+  int nsplit = hq_tune(HQ_TUNE_Q3_KSPLIT, 0);
   if (nsplit <= 0) nsplit = dev->cus / ntiles;  // only when there are fewer tiles than half the CUs
   if (nsplit > max_split) nsplit = max_split;
   if (nsplit < 1) nsplit = 1;

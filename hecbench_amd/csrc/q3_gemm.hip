@@ -11,7 +11,9 @@
 // window of the packed string into two subnormal-fp16 MFMA operands
 // (q3_recipe.h).  The factor 2^pos of each operand slot is folded into the
 // activations by a small pre-pass that also reorders them into operand-slot order
-// ([k-group][mfma j][row][8 halves]) and computes the row sums for the zero term.
+// ([k-group][mfma j][row][8 halves]), scales every row by a power of two so that
+// the fold stays inside the fp16 normal range, and computes the row sums for the
+// zero term.
 // The main kernel streams the weights once: a workgroup (4 waves, one per SIMD) owns 128
 // output columns and all of K and walks K in steps of 8 k-groups; each wave owns two
 // k-groups of a step, loads their activation slices (from L2) and packed rows (from
@@ -38,47 +40,21 @@ constexpr int kChunk = kStepGroups * kBufs;  // the pre-pass pads K to a multipl
 constexpr int kTileN = 128;     // output columns per workgroup
 
 
-// ---- pre-pass: activations -> operand-slot order, scaled by 2^-pos; row sums ----------------
-// Ap[((g*4 + j)*Mpad + m)*8 + e] = A[m][32g + k] * 2^-pos(k) with slot(k) = 8j + e; rows >= M and
-// groups >= G hold zeros.  Blocks [0, Gpad/4): wave w of block b re-orders k-group 4b + w, lane =
-// row, so the 16-byte pieces of 64 rows form 1 KB contiguous stores.  Blocks [Gpad/4, Gpad/4 +
-// Mpad): one block per row sums the row in a fixed order (deterministic).
+// ---- pre-pass: activations -> operand-slot order, scaled by P[m] * 2^-pos; row sums ------------
+// Ap[((g*4 + j)*Mpad + m)*8 + e] = A[m][32g + k] * P[m] * 2^-pos(k) with slot(k) = 8j + e; rows >= M and
+// groups >= G hold zeros.  One block per row: it finds the row's largest magnitude and sum, picks the
+// power of two P[m] that puts the largest magnitude in [2^14, 2^15), and re-orders its row.  The 2^-pos
+// of an operand slot (pos <= 7) then leaves every entry within 2^21 of its row's largest an fp16 normal
+// number, i.e. exactly the input's mantissa; the main kernel's epilogue divides by P[m] again.  (Without
+// P[m] the slot factor alone pushed activations below 2^-7 into the fp16 subnormals.)
 __global__ __launch_bounds__(256) void q3_gemm_prep(const _Float16* __restrict__ A, _Float16* __restrict__ Ap,
-                                                   float* __restrict__ rowsum, int M, int K, int Mpad,
-                                                   int Gpad) {
+                                                   float* __restrict__ rowsum, float* __restrict__ rowinv,
+                                                   int M, int K, int Mpad, int Gpad) {
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int G = K >> 5;
-  const int nreorder = Gpad >> 2;
-  if ((int)blockIdx.x < nreorder) {
-    const int g = blockIdx.x * 4 + wv, m = lane;
-    if (m >= Mpad) return;
-    _Float16 out[32];
-#pragma unroll
-    for (int i = 0; i < 32; ++i) out[i] = (_Float16)0.f;
-    if (m < M && g < G) {
-      const u4v* src = reinterpret_cast<const u4v*>(A + (size_t)m * K + 32 * g);
-      u4v raw[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) raw[i] = src[i];
-      const _Float16* in = reinterpret_cast<const _Float16*>(raw);
-#pragma unroll
-      for (int k = 0; k < 32; ++k) {
-        // exact power-of-two scaling (subnormal results lose bits below 2^-24 only)
-        out[hq_q3::slot_of(k)] =
-            (_Float16)((float)in[k] * __uint_as_float((uint32_t)(127 - hq_q3::pos_of(k)) << 23));
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      u4v* dst = reinterpret_cast<u4v*>(Ap + ((size_t)(g * 4 + j) * Mpad + m) * 8);
-      *dst = *reinterpret_cast<const u4v*>(out + 8 * j);
-    }
-    return;
-  }
-  // one block per row: every thread's loads are independent and issued together
-  const int m = (int)blockIdx.x - nreorder;
-  __shared__ float part[4];
-  float sum = 0.f;
+  const int m = blockIdx.x;
+  __shared__ float s_sum[4], s_max[4];
+  float sum = 0.f, amax = 0.f;
   if (m < M) {
     const u4v* src = reinterpret_cast<const u4v*>(A + (size_t)m * K);
     const int n16 = K >> 3;
@@ -93,18 +69,54 @@ __global__ __launch_bounds__(256) void q3_gemm_prep(const _Float16* __restrict__
       for (int u = 0; u < 4; ++u) {
         const int i = i0 + u * 256 + (int)threadIdx.x;
         const _Float16* in = reinterpret_cast<const _Float16*>(&raw[u]);
-        float s8 = 0.f;
+        float s8 = 0.f, m8 = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) s8 += (float)in[e];
+        for (int e = 0; e < 8; ++e) {
+          s8 += (float)in[e];
+          m8 = fmaxf(m8, fabsf((float)in[e]));
+        }
         sum += i < n16 ? s8 : 0.f;
+        amax = i < n16 ? fmaxf(amax, m8) : amax;
       }
     }
   }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-  if (lane == 0) part[wv] = sum;
+  for (int off = 32; off > 0; off >>= 1) {
+    sum += __shfl_xor(sum, off);
+    amax = fmaxf(amax, __shfl_xor(amax, off));
+  }
+  if (lane == 0) { s_sum[wv] = sum; s_max[wv] = amax; }
   __syncthreads();
-  if (threadIdx.x == 0) rowsum[m] = (part[0] + part[1]) + (part[2] + part[3]);
+  amax = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+  // P = 2^(14 - floor(log2 amax)); an all-zero or non-finite row keeps P = 1 (fp16 magnitudes span 2^-24 .. 2^16)
+  const int ex = (int)((__float_as_uint(amax) >> 23) & 255u) - 127;
+  const int pe = (amax > 0.f && ex < 128) ? 14 - ex : 0;
+  if (threadIdx.x == 0) {
+    rowsum[m] = (s_sum[0] + s_sum[1]) + (s_sum[2] + s_sum[3]);
+    rowinv[m] = __uint_as_float((uint32_t)(127 - pe) << 23);
+  }
+  // second pass over the row (it is in the caches now): thread = k-group
+  for (int g = threadIdx.x; g < Gpad; g += 256) {
+    _Float16 out[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) out[i] = (_Float16)0.f;
+    if (m < M && g < G) {
+      const u4v* src = reinterpret_cast<const u4v*>(A + (size_t)m * K + 32 * g);
+      u4v raw[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) raw[i] = src[i];
+      const _Float16* in = reinterpret_cast<const _Float16*>(raw);
+#pragma unroll
+      for (int k = 0; k < 32; ++k)
+        out[hq_q3::slot_of(k)] =
+            (_Float16)((float)in[k] * __uint_as_float((uint32_t)(127 + pe - hq_q3::pos_of(k)) << 23));
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      u4v* dst = reinterpret_cast<u4v*>(Ap + ((size_t)(g * 4 + j) * Mpad + m) * 8);
+      *dst = *reinterpret_cast<const u4v*>(out + 8 * j);
+    }
+  }
 }
 
 // Sixteen two-field registers of one column's k-group (see q3_recipe.h).
@@ -125,6 +137,7 @@ struct GemmArgs {
   const uint32_t* w;
   const u4v* Ap;        // [Gpad][4][Mpad] 16-byte operand chunks
   const float* rowsum;  // [Mpad]
+  const float* rowinv;  // [Mpad] 1 / P[m]
   const float* scales;
   const float* zeros;
   float* out;           // [M][N]
@@ -157,11 +170,14 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
     zr = *reinterpret_cast<const f4v*>(a.zeros + n_out);
   }
   // final reduction: a wave finishes rows 8*wv .. 8*wv+7 of every 32-row block, half wave kb four of them
-  float rs[MB][4];
+  float rs[MB][4], ri[MB][4];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) rs[mb][j] = a.rowsum[mb * 32 + 8 * wv + 4 * kb + j];
+    for (int j = 0; j < 4; ++j) {
+      rs[mb][j] = a.rowsum[mb * 32 + 8 * wv + 4 * kb + j];
+      ri[mb][j] = a.rowinv[mb * 32 + 8 * wv + 4 * kb + j] * 16777216.f;  // 2^24: the unit of the code operands
+    }
 
   f16v acc[MB][4];
 #pragma unroll
@@ -241,7 +257,7 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
       if (m < a.M && n_out < a.N) {
         f4v o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = sc[e] * (v[e] * 16777216.f) - zr[e] * rs[mb][j];
+        for (int e = 0; e < 4; ++e) o[e] = sc[e] * (v[e] * ri[mb][j]) - zr[e] * rs[mb][j];
         f4v* dst = reinterpret_cast<f4v*>(a.out + (size_t)m * a.N + n_out);
         if (a.flags & HQ_FLAG_ACCUMULATE) { const f4v old = *dst; o += old; }
         *dst = o;
@@ -270,24 +286,25 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
   const int Gpad = (G + kChunk - 1) / kChunk * kChunk;
   const size_t ap_halves = (size_t)Gpad * 4 * 64 * 8;
   HqWorkspace ws;
-  int rc = hq_get_workspace(stream, ap_halves / 2 + 64, 1, &ws);
+  int rc = hq_get_workspace(stream, ap_halves / 2 + 128, 1, &ws);
   if (rc != HQ_OK) return rc;
   _Float16* Ap = reinterpret_cast<_Float16*>(ws.partial);
   float* rowsum = ws.partial + ap_halves / 2;
+  float* rowinv = rowsum + 64;
   // up to 64 rows per pass over the weights
   for (int m0 = 0; m0 < M; m0 += 64) {
     const int Mb = M - m0 < 64 ? M - m0 : 64;
     const int MB = Mb > 32 ? 2 : 1;
     const int Mpad = 32 * MB;
     const _Float16* A = reinterpret_cast<const _Float16*>(x) + (size_t)m0 * K;
-    hipLaunchKernelGGL(q3_gemm_prep, dim3(Gpad / 4 + Mpad), dim3(256), 0, stream, A, Ap, rowsum, Mb, K, Mpad,
-                       Gpad);
+    hipLaunchKernelGGL(q3_gemm_prep, dim3(Mpad), dim3(256), 0, stream, A, Ap, rowsum, rowinv, Mb, K, Mpad, Gpad);
     rc = hq_launch_status();
     if (rc != HQ_OK) return rc;
     GemmArgs a;
     a.w = reinterpret_cast<const uint32_t*>(qweight);
     a.Ap = reinterpret_cast<const u4v*>(Ap);
     a.rowsum = rowsum;
+    a.rowinv = rowinv;
     a.scales = scales;
     a.zeros = zeros;
     a.out = y + (size_t)m0 * N;

@@ -279,10 +279,10 @@ extern "C" int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* 
   if (rc != HQ_OK) return rc;
   const int vec_ok = !((uintptr_t)A & 15) && !((uintptr_t)out & 3);
   int64_t blocks = (n / 4 + 256 * kQuads - 1) / (256 * kQuads);  // one trip of the fast path each, or grid-stride
-  const int64_t cap = (int64_t)dev->cus * hq_env_int("HQ_Q8_WGS", 5);
+  const int64_t cap = (int64_t)dev->cus * hq_tune(HQ_TUNE_Q8_WGS, 5);
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(quantize8_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, code, A, out, n,
-                     vec_ok, hq_env_int("HQ_Q8_FAST", 1));
+                     vec_ok, hq_tune(HQ_TUNE_Q8_FAST, 1));
   return hq_launch_status();
 }

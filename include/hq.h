@@ -19,8 +19,12 @@
  *     fixed-point matrix-core paths give NaN where the reference arithmetic would give +-Inf);
  *   - the library keeps one small workspace per (device, stream) pair (split-K
  *     partial sums, arrival counters, re-ordered GEMM activations), allocated by
- *     hq_init() or by the first call that needs it; calls on different streams
- *     use different workspaces and may overlap.
+ *     hq_init() / hq_reserve_workspace() or by the first call that needs more than
+ *     is there (that call then runs hipMalloc, which fails under stream capture:
+ *     reserve first).  A workspace grows geometrically, lives until hq_shutdown()
+ *     and is used by every call on its stream: calls on different streams may
+ *     overlap, two host threads must not issue calls on the SAME stream at the
+ *     same time (the calls of one stream share the workspace in stream order).
  */
 #ifndef HQ_H
 #define HQ_H
@@ -48,7 +52,10 @@ extern "C" {
 /* flags */
 #define HQ_FLAG_ACCUMULATE 1u /* y += result (reference wrapper semantics) */
 
-/* 4-bit code books of hq_dequant_4bit */
+/* 4-bit code books of hq_dequant_nf4 / hq_quantize_4bit.
+ * NF4: the QLoRA normal-float table (checked against its quantile construction).
+ * FP4: bit 3 sign, low bits {0, 1/192, 2/3, 1, 1/3, 1/2, 1/6, 1/4} -- parity unpinned: the HeCBench
+ * tree holds no FP4 source, so the table is this library's statement of the bitsandbytes one. */
 #define HQ_TABLE_NF4 0
 #define HQ_TABLE_FP4 1
 
@@ -63,6 +70,22 @@ const char* hq_strerror(int code);
  * but calling it keeps the allocation out of the first timed call.
  * Mirrors the device query of the AQLM launcher, src/quantAQLM-hip/main.cu:108-121. */
 int hq_init(void);
+
+/* Sizes the workspace of (current device, stream) for split-K matvecs up to max_N columns and
+ * batched GEMMs up to max_K input features, so that later calls on that stream never allocate
+ * (needed before stream capture).  No counterpart in the reference. */
+int hq_reserve_workspace(void* stream, int max_K, int max_N);
+
+/* Waits for the current device, then frees every workspace the library holds on any device.
+ * Optional; the library can be used again afterwards (workspaces are re-created on demand). */
+int hq_shutdown(void);
+
+/* Launch-shape override for tests and sweeps, not part of the stable interface: name is one of
+ * HQ_Q3_WAVES, HQ_Q3_STEPS, HQ_Q3_KSPLIT, HQ_Q3_SMALL_BATCH, HQ_LUT_PATH, HQ_LUT_KSPLIT, HQ_NF4_PIPE,
+ * HQ_AQLM_ROWS, HQ_Q8_WGS, HQ_Q8_FAST, HQ_ACTQ_GROUPS, HQ_SPLITK_FENCES (an environment variable of the same name seeds
+ * the knob once per process); clear != 0 returns the knob to the library's own choice.  Results
+ * never depend on a knob beyond the documented tolerances. */
+int hq_set_tunable(const char* name, int value, int clear);
 
 /* Device facts the benchmark drivers print next to the roofline numbers.
  * Any pointer may be NULL. */
@@ -101,7 +124,10 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  *   y        : fp32 [batch_M][N]
  *   K % 32 == 0, N % 4 == 0, batch_M >= 1; qweight and x 16-byte aligned.
  * Products are accumulated in fp32 for both dtypes (the reference's fp16
- * variant accumulates 16 terms in fp16; this library is never less accurate).
+ * variant accumulates 16 terms in fp16).  batch_M > 1 pre-scales every activation
+ * row by a power of two, so accuracy does not depend on the magnitude of the
+ * activations: entries within 2^21 of their row's largest magnitude enter the
+ * matrix cores exactly, smaller ones lose low bits (those 2^32 below it vanish).
  * batch_M == 1 replaces vecquant3matmul / vecquant3matmul_faster
  * (src/quant3MatMul-hip/kernels.h:171-217) — pass HQ_FLAG_ACCUMULATE for their
  * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 and runs the
@@ -131,7 +157,7 @@ int hq_lut_gemv(const uint32_t* bW, const void* alpha_fp16, const void* q_bias_f
  * codes int16[M][K/8] (read as unsigned), codebooks fp16[..][65536][8] with
  * consecutive code books codebook_stride_int4*16 bytes apart, cb(m) = first j
  * with m < codebook_a_sizes[j].  scales_fp16 may be NULL (the reference kernel
- * applies no scale).  K % 8 == 0.  fp32 accumulation, one rounding.  Replaces
+ * applies no scale).  K % 64 == 0 (as in the reference).  fp32 accumulation, one rounding.  Replaces
  * code1x16_matvec, src/quantAQLM-hip/main.cu:103-139 (without its internal
  * synchronisation, timing and printing).
  */
@@ -201,7 +227,10 @@ int hq_gemv_int4(const uint8_t* mat_packed, const void* vec_fp16, void* res_fp16
  * mantissa of 0.75); out = scale * e2m1(in / scale) with round-to-nearest-even onto
  * {0, .5, 1, 1.5, 2, 3, 4, 6} and saturation.  dtype HQ_DTYPE_F16 or HQ_DTYPE_BF16; n_elems a
  * multiple of 32; 16-byte aligned pointers; in and out must not overlap.  Bit-exact with the reference
- * kernel for finite data.  Replaces mxfp4<T>(y, a, numel, niters), src/mxfp4-hip/main.cu:144-171
+ * kernel for finite data, except where its arithmetic breaks down: a group maximum that rounds to zero
+ * (the reference divides by zero; here signed zeros) and a finite group maximum whose power-of-two
+ * rounding leaves the format (fp16 >= 61440, bf16 >= 0x7f60: the reference writes NaN for the group;
+ * here the scale is 2^14 / 2^126 and the results are finite or infinite).  Replaces mxfp4<T>(y, a, numel, niters), src/mxfp4-hip/main.cu:144-171
  * (kernel main.cu:109-142), without its timing loop and printing.
  */
 int hq_mxfp4_qdq(const void* in, void* out, int64_t n_elems, int dtype, void* stream);

@@ -650,7 +650,8 @@ static float round_to_e2m1(float a) {
  * of 0.75 (main.cu:124-126), gives the shared scale 2^(e-2) clamped to the E8M0 range
  * (main.cu:128-132); every element is divided by it, rounded to e2m1 and multiplied back
  * (main.cu:134-141).  Groups whose rounded maximum is zero give zeros (the reference divides by a
- * zero scale there). */
+ * zero scale there); groups whose rounded maximum leaves the format use the scale 2^14 / 2^126 (the
+ * reference writes NaN there).  Both cases: parity unpinned, behaviour defined by this library. */
 void hqo_mxfp4_qdq(const uint16_t* in, uint16_t* out, int64_t n, int is_bf16) {
   const int mant = is_bf16 ? 7 : 10;
   for (int64_t g = 0; g + 32 <= n; g += 32) {
@@ -666,8 +667,16 @@ void hqo_mxfp4_qdq(const uint16_t* in, uint16_t* out, int64_t n, int is_bf16) {
       continue;
     }
     int e;
-    frexpf(bmax, &e); /* bmax = 0.5 * 2^e exactly */
-    e -= 1;
+    if ((rounded >> mant) == (is_bf16 ? 255u : 31u)) {
+      /* The rounding carried past the largest power of two of the format (group maximum >= 61440 in
+       * fp16, >= 0x7f60 in bf16, or an infinity).  The reference takes log2 of that infinity and writes
+       * NaN for the whole group (main.cu:126-141); the library's stated behaviour is the exponent the
+       * carry stands for, restated here.  Parity with the reference is deliberately given up. */
+      e = is_bf16 ? 128 : 16;
+    } else {
+      frexpf(bmax, &e); /* bmax = 0.5 * 2^e exactly */
+      e -= 1;
+    }
     int scale_exp = 127 + (e - 2 < 127 ? e - 2 : 127);
     if (scale_exp < 0) scale_exp = 0;
     float scale = ldexpf(1.f, scale_exp - 127);

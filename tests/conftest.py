@@ -26,3 +26,20 @@ def hq():
     import hecbench_amd
     hecbench_amd.init()
     return hecbench_amd
+
+
+@pytest.fixture
+def tunable():
+    """Sets launch-shape knobs of the library through hq_set_tunable and clears them afterwards."""
+    from hecbench_amd import _lib
+    lib = _lib.load()
+    touched = []
+
+    def set_(name, value):
+        rc = lib.hq_set_tunable(name.encode(), int(value), 0)
+        assert rc == 0, (name, rc)
+        touched.append(name)
+
+    yield set_
+    for name in touched:
+        lib.hq_set_tunable(name.encode(), 0, 1)

@@ -58,3 +58,18 @@ def test_argument_validation_needs_no_gpu():
     assert lib.hq_aqlm_matvec(None, None, None, None, None, 4096, 4096, None, 65536, None) == -1
     assert lib.hq_quantize_dynamic8(None, None, None, 5, None) == -1
     assert lib.hq_quantize_dynamic8(None, None, None, 0, None) == 0
+
+
+def test_tunables_need_no_gpu():
+    """Launch-shape knobs are set by name; unknown names and null pointers are rejected."""
+    from hecbench_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("libhq.so not built in this checkout")
+    lib = _lib.load()
+    for name in (b"HQ_Q3_WAVES", b"HQ_Q3_STEPS", b"HQ_Q3_KSPLIT", b"HQ_LUT_PATH", b"HQ_NF4_PIPE", b"HQ_AQLM_ROWS",
+                 b"HQ_SPLITK_FENCES"):
+        assert lib.hq_set_tunable(name, 4, 0) == 0
+        assert lib.hq_set_tunable(name, 0, 1) == 0
+    assert lib.hq_set_tunable(b"HQ_NO_SUCH_KNOB", 1, 0) == -3
+    assert lib.hq_set_tunable(None, 1, 0) == -1
+    assert lib.hq_reserve_workspace(None, -1, 0) == -2

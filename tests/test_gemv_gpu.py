@@ -70,7 +70,7 @@ def test_rejects_bad_arguments(hq):
     from hecbench_amd import HqError
     v = torch.zeros(40, dtype=torch.float16, device="cuda:0")
     with pytest.raises(HqError):
-        hq.gemv_fp16(torch.zeros(4, 36, dtype=torch.float16, device="cuda:0"), v)     # n % 8
+        hq.gemv_fp16(torch.zeros(4, 36, dtype=torch.float16, device="cuda:0"), v[:36])     # n % 8
     with pytest.raises(HqError):
         hq.gemv_int8(torch.zeros(4, 40, dtype=torch.int8, device="cuda:0"), v, 1.0, 0.0)   # n % 16
     with pytest.raises(HqError):

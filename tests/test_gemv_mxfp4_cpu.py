@@ -176,3 +176,26 @@ def test_mxfp4_vs_numpy_restatement(o, bf16):
     # idempotent: quantising a quantised tensor changes nothing
     again = from_bits(o.mxfp4_qdq(as_bits(got, bf16), bf16), bf16)
     assert np.array_equal(again, got)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_mxfp4_group_maximum_rounding_past_the_format(o, bf16):
+    """A finite group maximum whose power-of-two rounding leaves the format (fp16 >= 61440, bf16 >= 0x7f60):
+    the reference kernel rounds it to infinity, takes log2(inf) and writes NaN for the whole group
+    (src/mxfp4-hip/main.cu:126-141).  This library documents a different, finite behaviour there: the scale
+    is the power of two the carry would have produced, 2^14 (bf16: 2^126), and elements quantise against it
+    as anywhere else (the maximum itself lands on 4 * scale, which overflows to infinity)."""
+    top = 0x7f7f if bf16 else 0x7bff                       # largest finite value
+    bits = np.zeros(64, np.uint16)
+    bits[0] = top
+    bits[1] = 0x7f00 if bf16 else 0x7800                   # 2^127 | 32768: scale * 2 -> kept
+    bits[2] = (0x7e80 if bf16 else 0x7400) | 0x8000        # -2^126 | -16384: -scale -> kept
+    bits[3] = 0x7e00 if bf16 else 0x7000                   # scale / 2 -> kept (0.5 is on the grid)
+    bits[4] = 0x3f80 if bf16 else 0x3c00                   # 1.0: far below scale / 4 -> 0
+    bits[32] = 0x3f80 if bf16 else 0x3c00                  # second group, ordinary: 1.0 is kept
+    got = o.mxfp4_qdq(bits, bf16)
+    inf = 0x7f80 if bf16 else 0x7c00
+    assert got[0] == inf
+    assert got[1] == bits[1] and got[2] == bits[2] and got[3] == bits[3]
+    assert got[4] == 0 and not got[5:32].any()
+    assert got[32] == bits[32]

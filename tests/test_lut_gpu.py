@@ -31,8 +31,8 @@ def _run(hq, bW, alpha, qbias, x, group):
     (2048, 128, 2, 64, True, 15), (1152, 192, 4, 32, False, 16), (640, 64, 5, 64, False, 17),
     (896, 128, 6, 32, False, 18), (512, 320, 7, 64, False, 19), (1280, 64, 8, 32, False, 20),
     (128, 64, 3, 32, False, 21), (192, 64, 3, 64, False, 22)])
-def test_vs_oracle(hq, oracle, monkeypatch, path, K, N, nb, group, zero_bias, seed):
-    monkeypatch.setenv("HQ_LUT_PATH", str(path))
+def test_vs_oracle(hq, oracle, tunable, path, K, N, nb, group, zero_bias, seed):
+    tunable("HQ_LUT_PATH", path)
     bW, alpha, qbias, x = oa.make_lut_problem(seed, K, N, nb, group, zero_bias)
     y = _run(hq, bW, alpha, qbias, x, group)
     ref = oracle.lut_gemv_f64(bW, alpha, qbias, x, group)

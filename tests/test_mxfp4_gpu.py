@@ -62,6 +62,27 @@ def test_every_magnitude_below_saturation(hq, oracle, bf16):
         assert np.array_equal(_bits(got), oracle.mxfp4_qdq(bits, bf16))
 
 
+@pytest.mark.parametrize("bf16", [False, True])
+def test_group_maximum_rounding_past_the_format(hq, oracle, bf16):
+    """Finite groups whose maximum rounds past the largest power of two of the format: the reference kernel
+    writes NaN there (it takes log2 of an infinity); the library's documented behaviour is the finite scale
+    2^14 (bf16: 2^126), the same as the oracle's."""
+    import torch
+    rng = np.random.default_rng(5)
+    top = 0x7f7f if bf16 else 0x7bff
+    lo = 0x7f60 if bf16 else 0x7b80
+    bits = _random_bits(31, 32 * 64, bf16).reshape(-1, 32)
+    bits[:, 0] = rng.integers(lo, top + 1, bits.shape[0]).astype(np.uint16)      # every group overflows the rounding
+    bits[:, 1] = (bits[:, 0] - 0x0100) | 0x8000
+    bits = bits.reshape(-1)
+    got = _bits(hq.mxfp4_qdq(_tensor(bits, bf16)))
+    torch.cuda.synchronize()
+    want = oracle.mxfp4_qdq(bits, bf16)
+    assert np.array_equal(got, want)
+    inf = 0x7f80 if bf16 else 0x7c00
+    assert ((got & 0x7fff) <= inf).all()          # no NaN anywhere
+
+
 def test_empty_and_rejections(hq):
     import torch
     from hecbench_amd import HqError

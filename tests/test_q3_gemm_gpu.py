@@ -35,6 +35,41 @@ def test_small_shapes_vs_oracle(hq, oracle, M, K, N, seed):
     assert rel_err(y, exact, FLOOR_F16) <= 1e-4
 
 
+@pytest.mark.parametrize("scale_exp", [-16, -12, -8, 0, 4])
+def test_dynamic_range(hq, oracle, scale_exp):
+    """Accuracy must not depend on the magnitude of the activations: whole problem scaled by a power of
+    two (down to where fp16 inputs are subnormal), rows of very different magnitude in one batch, an
+    all-zero row and a row with one large outlier.  Every row is held to the bound the N(0,1) cases meet,
+    measured against that row's own RMS."""
+    M, K, N = 40, 2048, 260
+    codes, scales, zeros, A = oa.make_q3_problem(70 + scale_exp, K, N, x_dtype=np.float16, batch=M)
+    rng = np.random.default_rng(7)
+    A = A.astype(np.float32) * np.float32(2.0 ** scale_exp)
+    A[3] = 0.0                                            # an all-zero row
+    A[5] *= np.float32(2.0 ** -6)                         # rows of other magnitudes in the same batch
+    A[6] *= np.float32(2.0 ** 5)
+    A[7, 100] = np.float32(2.0 ** min(15, scale_exp + 12))   # one large outlier (4096 sigma) in a row
+    A[8] = rng.standard_normal(K).astype(np.float32) * np.float32(2.0 ** scale_exp) * \
+        np.exp2(rng.integers(-8, 1, K)).astype(np.float32)    # magnitudes spread over 2^8 inside a row
+    A = A.astype(np.float16)
+    mat = oracle.q3_pack(codes)
+    y = _run(hq, A, mat, scales, zeros)
+    exact = oracle.q3_gemm(A, mat, scales, zeros, mode=0)
+    assert np.all(y[3] == 0.0)
+    for m in range(M):
+        if m == 3:
+            continue
+        assert rel_err(y[m], exact[m]) <= 5e-3, (scale_exp, m)
+        assert rel_err(y[m], exact[m], FLOOR_F16) <= 1e-4, (scale_exp, m)
+    # a row of the batch equals the batch-1 matvec on that row
+    import torch
+    dev = torch.device("cuda:0")
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    for m in (0, 5, 7):
+        yv = hq.q3_matvec(t(A[m]), t(mat), t(scales), t(zeros)).cpu().numpy()
+        assert rel_err(y[m], yv) <= 5e-3, (scale_exp, m)
+
+
 def test_config4_sampled_columns(hq, oracle):
     """M=64, K=8192, N=28672: all outputs computed on the GPU, 384 sampled columns checked."""
     M, K, N = 64, 8192, 28672

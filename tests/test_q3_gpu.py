@@ -122,7 +122,7 @@ def test_non_finite_activations_propagate(hq, oracle):
             assert not np.isfinite(y).any(), bad
 
 
-def test_launch_shapes_match(hq, oracle, monkeypatch):
+def test_launch_shapes_match(hq, oracle, tunable):
     """Every launch shape (waves per workgroup x steps x K split; one or several
     rounds per workgroup) gives the same answer."""
     K, N = 4096, 1024
@@ -131,12 +131,16 @@ def test_launch_shapes_match(hq, oracle, monkeypatch):
     ref = oracle.q3_matvec_f64(x, mat, scales, zeros)
     for waves, steps, ks in [(8, 4, 0), (8, 2, 0), (4, 2, 1), (4, 1, 0), (16, 1, 1), (8, 4, 1), (4, 4, 2), (4, 8, 0),
                              (8, 1, 3), (8, 1, 1), (4, 1, 1)]:
-        monkeypatch.setenv("HQ_Q3_WAVES", str(waves))
-        monkeypatch.setenv("HQ_Q3_STEPS", str(steps))
-        monkeypatch.setenv("HQ_Q3_KSPLIT", str(ks))
+        tunable("HQ_Q3_WAVES", waves)
+        tunable("HQ_Q3_STEPS", steps)
+        tunable("HQ_Q3_KSPLIT", ks)
         for _ in range(2):  # twice: the arrival counters must reset themselves
             y = _run(hq, x, mat, scales, zeros)
             assert rel_err(y, ref) <= 1e-4, (waves, steps, ks)
+            if ks > 1:  # formal release/acquire fences in the split-K arrival: the same bits
+                tunable("HQ_SPLITK_FENCES", 1)
+                assert np.array_equal(_run(hq, x, mat, scales, zeros), y), (waves, steps, ks)
+                tunable("HQ_SPLITK_FENCES", 0)
 
 
 def test_rejects_bad_arguments(hq):

@@ -8,12 +8,12 @@ from tests import oracle_api as oa
 pytestmark = pytest.mark.gpu
 
 
-def test_two_streams_interleaved(hq, oracle, monkeypatch):
+def test_two_streams_interleaved(hq, oracle, tunable):
     import torch
     dev = torch.device("cuda:0")
-    monkeypatch.setenv("HQ_Q3_KSPLIT", "4")          # force the cross-workgroup reduction (workspace + counters)
-    monkeypatch.setenv("HQ_Q3_WAVES", "4")
-    monkeypatch.setenv("HQ_Q3_STEPS", "1")
+    tunable("HQ_Q3_KSPLIT", 4)          # force the cross-workgroup reduction (workspace + counters)
+    tunable("HQ_Q3_WAVES", 4)
+    tunable("HQ_Q3_STEPS", 1)
     K, N, M = 2048, 512, 24
     problems = []
     for seed in (1, 2):
