@@ -174,7 +174,9 @@ extern "C" int hq_init(void) {
   int rc = hq_current_device(&d);
   if (rc != HQ_OK) return rc;
   HqWorkspace ws;
-  return hq_get_workspace(nullptr, 1, 1, &ws);
+  rc = hq_get_workspace(nullptr, 1, 1, &ws);
+  if (rc != HQ_OK) return rc;
+  return hq_noalloc_setup();  // this device's address of the fixed scratch of hq_q3_matvec_noalloc
 }
 
 extern "C" int hq_device_info(int* compute_units, int* wavefront_size, int* lds_bytes_per_cu,

@@ -43,6 +43,21 @@ struct HqWorkspace {
 int hq_get_workspace(hipStream_t stream, size_t need_floats, size_t need_counters,
                      HqWorkspace* out);
 
+// Caller-provided scratch of the GPTQ 3-bit paths (the entry point that allocates nothing passes its
+// fixed device array here; a null pointer means "use the stream's workspace").
+struct HqQ3Scratch {
+  float* partial;          // split-K partial sums, also the batched GEMM's re-ordered activations
+  size_t partial_floats;
+  float* rows;             // 128 floats: row sums and row scales of the batched GEMM
+  unsigned* counters;      // split-K arrival counters (cleared by the call that uses them)
+  size_t ncounters;
+};
+int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const float* scales, const float* zeros,
+                      float* y, int K, int N, int batch_M, unsigned flags, hipStream_t stream,
+                      const HqQ3Scratch* fixed);
+// Resolves the current device's copy of the fixed scratch array (once per device).
+int hq_noalloc_setup(void);
+
 // Launch-shape overrides for tests and sweeps (hq_set_tunable, or the environment variable of the
 // same name, which is read once per process).  hq_tune returns dflt while a knob is unset; it costs
 // one relaxed atomic load.

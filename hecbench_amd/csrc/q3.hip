@@ -423,12 +423,26 @@ int launch_matvec(const Q3Args& a, int ntiles, hipStream_t stream) {
 }  // namespace
 
 int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros,
-                      float* y, int K, int N, int M, unsigned flags, hipStream_t stream);
+                      float* y, int K, int N, int M, unsigned flags, hipStream_t stream, const HqQ3Scratch* fixed);
+
+namespace {
+// Zeroes n words with a kernel (a memset node inside a captured graph is not an option for callers
+// that capture the stream).
+__global__ __launch_bounds__(256) void fill_zero_kernel(unsigned* p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+}  // namespace
 
 extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float* scales,
                             const float* zeros, float* y, int K, int N, int batch_M, unsigned flags,
-                            void* stream_) {
-  hipStream_t stream = (hipStream_t)stream_;
+                            void* stream) {
+  return hq_q3_matvec_impl(x, x_dtype, qweight, scales, zeros, y, K, N, batch_M, flags, (hipStream_t)stream, nullptr);
+}
+
+int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const float* scales, const float* zeros,
+                      float* y, int K, int N, int batch_M, unsigned flags, hipStream_t stream,
+                      const HqQ3Scratch* fixed) {
   if (!x || !qweight || !scales || !zeros || !y) return HQ_ERR_NULL_POINTER;
   if (x_dtype != HQ_DTYPE_F32 && x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
   if (flags & ~HQ_FLAG_ACCUMULATE) return HQ_ERR_BAD_ENUM;
@@ -442,7 +456,7 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   if (rc != HQ_OK) return rc;
   if (batch_M > 1) {
     if (x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
-    return hq_q3_gemm_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream);
+    return hq_q3_gemm_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream, fixed);
   }
 
   const int G = K / 32;
@@ -473,7 +487,17 @@ extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, 
   a.x = x; a.w = reinterpret_cast<const uint32_t*>(qweight); a.scales = scales; a.zeros = zeros;
   a.y = y; a.partial = nullptr; a.counters = nullptr; a.K = K; a.N = N; a.gpw = gpw;
   a.nsplit = nsplit; a.x_f16 = (x_dtype == HQ_DTYPE_F16); a.flags = flags;
-  if (nsplit > 1) {
+  if (nsplit > 1 && fixed) {
+    // fixed scratch shared by every call on this device: the counters start from zero by a fill kernel
+    // on the same stream (they also reset themselves, but an earlier call may have been cut short)
+    if ((size_t)ntiles * nsplit * 64 > fixed->partial_floats || (size_t)ntiles > fixed->ncounters)
+      return HQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((ntiles + 255) / 256), dim3(256), 0, stream, fixed->counters, ntiles);
+    rc = hq_launch_status();
+    if (rc != HQ_OK) return rc;
+    a.partial = fixed->partial;
+    a.counters = fixed->counters;
+  } else if (nsplit > 1) {
     HqWorkspace ws;
     rc = hq_get_workspace(stream, (size_t)ntiles * nsplit * 64, (size_t)ntiles, &ws);
     if (rc != HQ_OK) return rc;

@@ -21,6 +21,8 @@
 // columns x 64 rows per step with 32x32x16 fp16 MFMAs (fp32 accumulate).  There is
 // no LDS traffic and no barrier in the loop.  The four waves' accumulators are
 // summed through LDS at the end and scale/zero are applied once per output.
+#include <mutex>
+
 #include "hq_internal.h"
 #include "q3_recipe.h"
 
@@ -279,18 +281,28 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream) {
 }  // namespace
 
 int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                      int K, int N, int M, unsigned flags, hipStream_t stream) {
+                      int K, int N, int M, unsigned flags, hipStream_t stream, const HqQ3Scratch* fixed) {
   if (((uintptr_t)x & 15) || (K & 7)) return HQ_ERR_MISALIGNED;
   if (((uintptr_t)scales & 15) || ((uintptr_t)zeros & 15) || ((uintptr_t)y & 15)) return HQ_ERR_MISALIGNED;
   const int G = K / 32;
   const int Gpad = (G + kChunk - 1) / kChunk * kChunk;
   const size_t ap_halves = (size_t)Gpad * 4 * 64 * 8;
-  HqWorkspace ws;
-  int rc = hq_get_workspace(stream, ap_halves / 2 + 128, 1, &ws);
-  if (rc != HQ_OK) return rc;
-  _Float16* Ap = reinterpret_cast<_Float16*>(ws.partial);
-  float* rowsum = ws.partial + ap_halves / 2;
-  float* rowinv = rowsum + 64;
+  _Float16* Ap;
+  float *rowsum, *rowinv;
+  if (fixed) {
+    if (ap_halves / 2 > fixed->partial_floats) return HQ_ERR_TOO_LARGE;
+    Ap = reinterpret_cast<_Float16*>(fixed->partial);
+    rowsum = fixed->rows;
+    rowinv = fixed->rows + 64;
+  } else {
+    HqWorkspace ws;
+    int rc = hq_get_workspace(stream, ap_halves / 2 + 128, 1, &ws);
+    if (rc != HQ_OK) return rc;
+    Ap = reinterpret_cast<_Float16*>(ws.partial);
+    rowsum = ws.partial + ap_halves / 2;
+    rowinv = rowsum + 64;
+  }
+  int rc = HQ_OK;
   // up to 64 rows per pass over the weights
   for (int m0 = 0; m0 < M; m0 += 64) {
     const int Mb = M - m0 < 64 ? M - m0 : 64;
@@ -313,4 +325,58 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
     if (rc != HQ_OK) return rc;
   }
   return HQ_OK;
+}
+
+// ---- the entry point that allocates nothing ----------------------------------------------------
+// Its scratch (split-K partial sums and arrival counters of the matvec, re-ordered activations, row
+// sums and row scales of the batched GEMM) lives in a fixed device array instead of the stream's
+// workspace.  Every GPU holds its own copy of the array at its own address, resolved once per device.
+namespace {
+constexpr size_t kScratchPartialBytes = (size_t)2 << 20;  // 2 MiB: K <= 16384 batched, 8192 partial rows of 64 floats
+constexpr size_t kScratchRowBytes = 1024;                 // 128 floats used
+constexpr size_t kScratchCounterBytes = 64 * 1024 - kScratchRowBytes;
+constexpr size_t kScratchBytes = kScratchPartialBytes + kScratchRowBytes + kScratchCounterBytes;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, null until resolved
+
+int scratch_of_current_device(void** out) {
+  int dev = 0;
+  HQ_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return HQ_ERR_UNSUPPORTED_DEVICE;
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    HQ_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return HQ_OK;
+}
+}  // namespace
+
+int hq_noalloc_setup(void) {
+  void* p = nullptr;
+  return scratch_of_current_device(&p);
+}
+
+extern "C" int hq_q3_matvec_noalloc(const void* x, int x_dtype, const int32_t* qweight, const float* scales,
+                                    const float* zeros, float* y, int K, int N, int batch_M, unsigned flags,
+                                    void* stream) {
+  void* base = nullptr;
+  int rc = scratch_of_current_device(&base);
+  if (rc != HQ_OK) return rc;
+  unsigned char* b = static_cast<unsigned char*>(base);
+  HqQ3Scratch s;
+  s.partial = reinterpret_cast<float*>(b);
+  s.partial_floats = kScratchPartialBytes / sizeof(float);
+  s.rows = reinterpret_cast<float*>(b + kScratchPartialBytes);
+  s.counters = reinterpret_cast<unsigned*>(b + kScratchPartialBytes + kScratchRowBytes);
+  s.ncounters = kScratchCounterBytes / sizeof(unsigned);
+  return hq_q3_matvec_impl(x, x_dtype, qweight, scales, zeros, y, K, N, batch_M, flags, (hipStream_t)stream, &s);
 }

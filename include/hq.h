@@ -138,6 +138,23 @@ int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float
                  void* stream);
 
 /*
+ * hq_q3_matvec for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): same arguments, same kernels and bit-identical results, but the
+ * scratch the kernels need (split-K partial sums and arrival counters of the matvec, the batched
+ * path's re-ordered activations, row sums and row scales) is a fixed 2 MiB + 64 KiB array in device
+ * memory that each GPU holds from library load to process end, instead of the stream's workspace.
+ * The call runs no hipMalloc, hipFree or allocating library routine.  Limits: batch_M > 1 needs
+ * K <= 16384; a split-K matvec needs tiles * splits <= 8192 and N <= 1032192 (never exceeded while
+ * the device has at most 8192 compute units); beyond them HQ_ERR_TOO_LARGE.  All calls on one GPU
+ * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race;
+ * issue them on one stream or order them with events.  Call hq_init() once per device beforehand,
+ * outside any capture (it resolves the array's address).  No counterpart in the reference.
+ */
+int hq_q3_matvec_noalloc(const void* x, int x_dtype, const int32_t* qweight, const float* scales,
+                         const float* zeros, float* y, int K, int N, int batch_M, unsigned flags,
+                         void* stream);
+
+/*
  * LUT-GEMM binary-coded-quantisation matvec (fp16 in, fp16 out):
  *   y[n] = sum_k x[k] * ( q_bias[k/G][n] + sum_b alpha[k/G][b][n] * s(k,b,n) ),
  *   s = +1 if bit (k%32) of bW[k/32][b][n] is set, else -1
