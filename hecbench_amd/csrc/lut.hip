@@ -250,17 +250,38 @@ struct Half16 {  // sixteen fp16 values as two 128-bit loads
   h8 lo, hi;
   __device__ __forceinline__ float get(int i) const { return (float)(i < 8 ? lo[i] : hi[i - 8]); }
 };
+// The same 128-bit loads for rows that start at any element (N not a multiple of 8 or 4): the types carry
+// the element's own alignment, the hardware reads unaligned global addresses.
+typedef _Float16 h8_any __attribute__((ext_vector_type(8), aligned(2)));
+typedef uint32_t u4v_any __attribute__((ext_vector_type(4), aligned(4)));
+template <bool RAGGED>
 __device__ __forceinline__ Half16 load_half16(const _Float16* p) {
   Half16 h;
-  h.lo = reinterpret_cast<const h8*>(p)[0];
-  h.hi = reinterpret_cast<const h8*>(p)[1];
+  if (RAGGED) {
+    h.lo = reinterpret_cast<const h8_any*>(p)[0];
+    h.hi = reinterpret_cast<const h8_any*>(p)[1];
+  } else {
+    h.lo = reinterpret_cast<const h8*>(p)[0];
+    h.hi = reinterpret_cast<const h8*>(p)[1];
+  }
   return h;
 }
+template <bool RAGGED>
+__device__ __forceinline__ u4v load_words(const uint32_t* p) {
+  if (RAGGED) return *reinterpret_cast<const u4v_any*>(p);
+  return __builtin_nontemporal_load(reinterpret_cast<const u4v*>(p));
+}
 
-constexpr int kQuadBytes = 5 * 128;  // B operand rows of one quad: four digits and the ones row
+// One B operand row is 4 lane quarters x 32 B; rows start 144 B apart (9 x 16 B, an odd multiple), so the
+// 16-byte pieces that the sixteen lanes of a quarter read from up to sixteen different rows fall into
+// sixteen different bank groups (with rows 128 B apart, rows 0, 2, 4 .. shared their banks).
+constexpr int kLutRow = 144;
+constexpr int kQuadBytes = 5 * kLutRow;  // B operand rows of one quad: four digits and the ones row
 
 // NB bit planes, QUADS 128-element quads per wave per round, WAVES waves per workgroup.
-template <int NB, int QUADS, int WAVES, bool BIAS>
+// RAGGED: N is any number >= 64 and the operands have only their elements' alignment; the last tile then
+// starts at column N - 64 (it overlaps its neighbour, both write the same values to the shared columns).
+template <int NB, int QUADS, int WAVES, bool BIAS, bool RAGGED>
 __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
   extern __shared__ float lds[];
   char* xs = reinterpret_cast<char*>(lds);                             // [waves][QUADS][5 rows][4 kb][32 B]
@@ -270,8 +291,8 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
   const int c = lane & 15, kb = lane >> 4;
   const int tile = blockIdx.x;
   const int nquads = a.K >> 7;
-  const size_t n0 = (size_t)tile * 64;
-  const uint32_t col_off = 4u * c;   // first of the lane's 4 columns (N % 64 == 0: no partial tiles)
+  const size_t n0 = RAGGED ? (size_t)min(tile * 64, a.N - 64) : (size_t)tile * 64;
+  const uint32_t col_off = 4u * c;   // first of the lane's 4 columns (no partial tiles: N % 64 == 0 or RAGGED)
   const uint32_t acol = 16u * kb;    // first of the 16 columns this lane applies alpha to
   char* xs_w = xs + wv * (QUADS * kQuadBytes);
   // Staging role of a lane: 32 lanes per quad; lane (sa, sp, sh) owns the four activations
@@ -289,7 +310,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
   // row 4 of every quad is the constant one (fp8 0x01 = 2^-9, the unit of the digits)
   if (lane < 32) {
 #pragma unroll
-    for (int t = 0; t < QUADS; ++t) *reinterpret_cast<uint32_t*>(xs_w + t * kQuadBytes + 4 * 128 + lane * 4) = 0x01010101u;
+    for (int t = 0; t < QUADS; ++t) *reinterpret_cast<uint32_t*>(xs_w + t * kQuadBytes + 4 * kLutRow + lane * 4) = 0x01010101u;
   }
 
   float tot[4][4];
@@ -315,8 +336,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
       const int quad = min(q0 + t, nquads - 1);
       const uint32_t* wp = a.bW + ((size_t)(4 * quad + kb) * NB) * a.N + n0 + col_off;
 #pragma unroll
-      for (int b = 0; b < NB; ++b)
-        wq[t][b] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wp + (size_t)b * a.N));
+      for (int b = 0; b < NB; ++b) wq[t][b] = load_words<RAGGED>(wp + (size_t)b * a.N);
     }
     // alpha and bias of the round's quads: issued here so that they arrive with the words
     Half16 al[QUADS][NB], bi[QUADS];
@@ -324,8 +344,8 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
     for (int t = 0; t < QUADS; ++t) {
       const int g = (min(q0 + t, nquads - 1) * 128) / a.G;
 #pragma unroll
-      for (int b = 0; b < NB; ++b) al[t][b] = load_half16(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
-      if (BIAS) bi[t] = load_half16(a.qbias + (size_t)g * a.N + n0 + acol);
+      for (int b = 0; b < NB; ++b) al[t][b] = load_half16<RAGGED>(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
+      if (BIAS) bi[t] = load_half16<RAGGED>(a.qbias + (size_t)g * a.N + n0 + acol);
     }
     // ---- scale to 16-bit fixed point, bias, cut into nibbles, stage (wave-local) ------------
     float amax = 0.f;
@@ -366,7 +386,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
       if (t < QUADS) {
         char* dst = xs_w + t * kQuadBytes + s_quarter * 32 + s_byte;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(dst + d * 128) = dg[d];
+        for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(dst + d * kLutRow) = dg[d];
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -382,7 +402,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
     for (int t = 0; t < QUADS; ++t) {
       if (q0 + t >= nquads) break;  // wave-uniform
       // MFMA columns 5..15 are never read: they re-use the ones row
-      const u4v* bp = reinterpret_cast<const u4v*>(xs_w + t * kQuadBytes + min(c, 4) * 128 + kb * 32);
+      const u4v* bp = reinterpret_cast<const u4v*>(xs_w + t * kQuadBytes + min(c, 4) * kLutRow + kb * 32);
       const u4v b0 = bp[0], b1 = bp[1];
       const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
       // column sum of the quad (digits 0..3: sum of the nibbles; column 4: 128), in units of
@@ -428,7 +448,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
       for (int i = 0; i < 4; ++i) red[(wv * 5 + c) * 64 + 16 * kb + 4 * i + q] = tot[q][i];
   }
   __syncthreads();
-  const int n = tile * 64 + tid;
+  const int n = (int)n0 + tid;
   if (tid < 64 && n < a.N) {
     float v = 0.f;
 #pragma unroll
@@ -450,10 +470,10 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
 // counts; both are zeroed once, their constant parts written once, and only the digit bytes are rewritten
 // per round.  Every MFMA column then carries one group's sum, is scaled by that group's alpha (lane column
 // c takes the alpha of group c / 4), and the groups are added when the digits are combined at the end.
-constexpr int kGroupedQuadBytes = 20 * 128;  // sixteen digit rows and up to four rows of ones
+constexpr int kGroupedQuadBytes = 20 * kLutRow;  // sixteen digit rows and up to four rows of ones
 constexpr int kGroupedRedBytes = 20 * 64 * 4;  // a wave's final sums: twenty columns of 64 outputs
 
-template <int NB, int GS, int QUADS, int WAVES, bool BIAS>
+template <int NB, int GS, int QUADS, int WAVES, bool BIAS, bool RAGGED>
 __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a) {
   constexpr int kWaveBytes = QUADS * kGroupedQuadBytes > kGroupedRedBytes ? QUADS * kGroupedQuadBytes : kGroupedRedBytes;
   extern __shared__ float lds[];
@@ -463,7 +483,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a)
   const int c = lane & 15, kb = lane >> 4;
   const int tile = blockIdx.x;
   const int nquads = a.K >> 7;
-  const size_t n0 = (size_t)tile * 64;
+  const size_t n0 = RAGGED ? (size_t)min(tile * 64, a.N - 64) : (size_t)tile * 64;
   const uint32_t col_off = 4u * c;
   const uint32_t acol = 16u * kb;
   const int cg = min(c >> 2, GS - 1);  // the group whose sums this lane's MFMA column carries
@@ -488,7 +508,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a)
       const int grp = (k0 * GS) >> 7;
 #pragma unroll
       for (int t = 0; t < QUADS; ++t)
-        *reinterpret_cast<uint32_t*>(xs_w + t * kGroupedQuadBytes + (16 + grp) * 128 + lane * 4) = 0x01010101u;
+        *reinterpret_cast<uint32_t*>(xs_w + t * kGroupedQuadBytes + (16 + grp) * kLutRow + lane * 4) = 0x01010101u;
     }
   }
 
@@ -514,16 +534,15 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a)
       const int quad = min(q0 + t, nquads - 1);
       const uint32_t* wp = a.bW + ((size_t)(4 * quad + kb) * NB) * a.N + n0 + col_off;
 #pragma unroll
-      for (int b = 0; b < NB; ++b)
-        wq[t][b] = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wp + (size_t)b * a.N));
+      for (int b = 0; b < NB; ++b) wq[t][b] = load_words<RAGGED>(wp + (size_t)b * a.N);
     }
     Half16 al[QUADS][NB], bi[QUADS];
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
       const int g = min(q0 + t, nquads - 1) * GS + cg;
 #pragma unroll
-      for (int b = 0; b < NB; ++b) al[t][b] = load_half16(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
-      if (BIAS) bi[t] = load_half16(a.qbias + (size_t)g * a.N + n0 + acol);
+      for (int b = 0; b < NB; ++b) al[t][b] = load_half16<RAGGED>(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
+      if (BIAS) bi[t] = load_half16<RAGGED>(a.qbias + (size_t)g * a.N + n0 + acol);
     }
     float amax = 0.f;
 #pragma unroll
@@ -558,9 +577,9 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a)
                               __builtin_amdgcn_perm(qe, pe, 0x07060302u), __builtin_amdgcn_perm(qo, po, 0x07060302u)};
       const int t = 2 * sp_ + st;
       if (t < QUADS) {
-        char* dst = xs_w + t * kGroupedQuadBytes + (4 * sg) * 128 + s_quarter * 32 + s_byte;
+        char* dst = xs_w + t * kGroupedQuadBytes + (4 * sg) * kLutRow + s_quarter * 32 + s_byte;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(dst + d * 128) = dg[d];
+        for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(dst + d * kLutRow) = dg[d];
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -576,8 +595,8 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a)
       if (q0 + t >= nquads) break;  // wave-uniform
       // digit rows: MFMA column c reads row c (rows past 4 GS stay zero and are never used);
       // rows of ones: column c reads its group's
-      const u4v* bp = reinterpret_cast<const u4v*>(xs_w + t * kGroupedQuadBytes + c * 128 + kb * 32);
-      const u4v* pp = reinterpret_cast<const u4v*>(xs_w + t * kGroupedQuadBytes + (16 + cg) * 128 + kb * 32);
+      const u4v* bp = reinterpret_cast<const u4v*>(xs_w + t * kGroupedQuadBytes + c * kLutRow + kb * 32);
+      const u4v* pp = reinterpret_cast<const u4v*>(xs_w + t * kGroupedQuadBytes + (16 + cg) * kLutRow + kb * 32);
       const u4v b0 = bp[0], b1 = bp[1], p0 = pp[0], p1 = pp[1];
       const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
       const v8i P = {(int)p0.x, (int)p0.y, (int)p0.z, (int)p0.w, (int)p1.x, (int)p1.y, (int)p1.z, (int)p1.w};
@@ -641,7 +660,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a)
       for (int i = 0; i < 4; ++i) red_w[(16 + (c >> 2)) * 64 + 16 * kb + 4 * i + q] = totp[q][i];
   }
   __syncthreads();
-  const int n = tile * 64 + tid;
+  const int n = (int)n0 + tid;
   if (tid < 64 && n < a.N) {
     float v = 0.f;
     for (int w = 0; w < WAVES; ++w) {
@@ -658,43 +677,57 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a)
 }
 
 template <int NB, int GS, int QUADS>
-int launch_bcq_grouped(const LutArgs& a, hipStream_t stream) {
+int launch_bcq_grouped(const LutArgs& a, bool ragged, hipStream_t stream) {
   constexpr int WAVES = 8;
   constexpr int kWaveBytes = QUADS * kGroupedQuadBytes > kGroupedRedBytes ? QUADS * kGroupedQuadBytes : kGroupedRedBytes;
   const size_t smem = (size_t)WAVES * kWaveBytes + (size_t)WAVES * 4;
-  const int ntiles = a.N / 64;
-  if (a.qbias)
-    hipLaunchKernelGGL((bcq_mfma_grouped_kernel<NB, GS, QUADS, WAVES, true>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
-  else
-    hipLaunchKernelGGL((bcq_mfma_grouped_kernel<NB, GS, QUADS, WAVES, false>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
+  const dim3 grid((a.N + 63) / 64), block(WAVES * 64);
+#define HQ_LUT_GO(BIAS, RAG) \
+  hipLaunchKernelGGL((bcq_mfma_grouped_kernel<NB, GS, QUADS, WAVES, BIAS, RAG>), grid, block, smem, stream, a)
+  if (a.qbias) { if (ragged) HQ_LUT_GO(true, true); else HQ_LUT_GO(true, false); }
+  else { if (ragged) HQ_LUT_GO(false, true); else HQ_LUT_GO(false, false); }
+#undef HQ_LUT_GO
   return hq_launch_status();
 }
 template <int GS>
-int launch_bcq_grouped_nb(const LutArgs& a, hipStream_t stream) {
+int launch_bcq_grouped_nb(const LutArgs& a, bool ragged, hipStream_t stream) {
   switch (a.nb) {  // quads per wave per round, bounded by the register budget
-    case 1: return launch_bcq_grouped<1, GS, 2>(a, stream);
-    case 2: return launch_bcq_grouped<2, GS, 2>(a, stream);
-    case 3: return launch_bcq_grouped<3, GS, 2>(a, stream);
-    case 4: return launch_bcq_grouped<4, GS, 2>(a, stream);
-    case 5: return launch_bcq_grouped<5, GS, 1>(a, stream);
-    case 6: return launch_bcq_grouped<6, GS, 1>(a, stream);
-    case 7: return launch_bcq_grouped<7, GS, 1>(a, stream);
-    default: return launch_bcq_grouped<8, GS, 1>(a, stream);
+    case 1: return launch_bcq_grouped<1, GS, 2>(a, ragged, stream);
+    case 2: return launch_bcq_grouped<2, GS, 2>(a, ragged, stream);
+    case 3: return launch_bcq_grouped<3, GS, 2>(a, ragged, stream);
+    case 4: return launch_bcq_grouped<4, GS, 2>(a, ragged, stream);
+    case 5: return launch_bcq_grouped<5, GS, 1>(a, ragged, stream);
+    case 6: return launch_bcq_grouped<6, GS, 1>(a, ragged, stream);
+    case 7: return launch_bcq_grouped<7, GS, 1>(a, ragged, stream);
+    default: return launch_bcq_grouped<8, GS, 1>(a, ragged, stream);
   }
 }
 
 // Eight waves per workgroup (two per SIMD, up to 256 VGPRs each): sixteen-wave variants
 // spill and measured slower.
 template <int NB, int QUADS>
-int launch_bcq_mfma(const LutArgs& a, hipStream_t stream) {
+int launch_bcq_mfma(const LutArgs& a, bool ragged, hipStream_t stream) {
   constexpr int WAVES = 8;
   const size_t smem = (size_t)WAVES * QUADS * kQuadBytes + (size_t)WAVES * 5 * 64 * 4 + (size_t)WAVES * 4;
-  const int ntiles = a.N / 64;
-  if (a.qbias)
-    hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, true>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
-  else
-    hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, false>), dim3(ntiles), dim3(WAVES * 64), smem, stream, a);
+  const dim3 grid((a.N + 63) / 64), block(WAVES * 64);
+#define HQ_LUT_GO(BIAS, RAG) \
+  hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, BIAS, RAG>), grid, block, smem, stream, a)
+  if (a.qbias) { if (ragged) HQ_LUT_GO(true, true); else HQ_LUT_GO(true, false); }
+  else { if (ragged) HQ_LUT_GO(false, true); else HQ_LUT_GO(false, false); }
+#undef HQ_LUT_GO
   return hq_launch_status();
+}
+
+// Which kernel a call takes (HQ_LUT_PLAN_* in hq.h).
+int lut_plan(const void* bW, const void* alpha, const void* q_bias, int K, int N, int group_size) {
+  if (hq_tune(HQ_TUNE_LUT_PATH, 1) != 1) return HQ_LUT_PLAN_TABLE;
+  if (K % 128 != 0 || N < 64) return HQ_LUT_PLAN_TABLE;
+  const bool aligned = N % 64 == 0 && !((uintptr_t)bW & 15) && !((uintptr_t)alpha & 15) && !((uintptr_t)q_bias & 15);
+  int plan;
+  if (group_size == 64 || group_size == 32) plan = HQ_LUT_PLAN_MFMA_GROUPED;
+  else if (group_size % 128 == 0) plan = HQ_LUT_PLAN_MFMA;
+  else return HQ_LUT_PLAN_TABLE;
+  return aligned ? plan : (plan | HQ_LUT_PLAN_RAGGED);
 }
 
 }  // namespace
@@ -712,30 +745,24 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
   int rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
 
-  const bool mfma_ok = N % 64 == 0 && K % 128 == 0 && !((uintptr_t)bW & 15) && !((uintptr_t)alpha & 15) &&
-                       !((uintptr_t)q_bias & 15) && hq_tune(HQ_TUNE_LUT_PATH, 1) == 1;
-  if (mfma_ok && (group_size == 64 || group_size == 32)) {
+  const int plan = lut_plan(bW, alpha, q_bias, K, N, group_size);
+  if (plan != HQ_LUT_PLAN_TABLE) {
+    const bool ragged = (plan & HQ_LUT_PLAN_RAGGED) != 0;
     LutArgs a;
     a.bW = bW; a.alpha = (const _Float16*)alpha; a.qbias = (const _Float16*)q_bias;
     a.x = (const _Float16*)x; a.y = (_Float16*)y; a.partial = nullptr; a.counters = nullptr;
     a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = K; a.nsplit = 1; a.strict = 0;
-    return group_size == 64 ? launch_bcq_grouped_nb<2>(a, stream) : launch_bcq_grouped_nb<4>(a, stream);
-  }
-  if (group_size % 128 == 0 && N % 64 == 0 && !((uintptr_t)bW & 15) && !((uintptr_t)alpha & 15) &&
-      !((uintptr_t)q_bias & 15) && hq_tune(HQ_TUNE_LUT_PATH, 1) == 1) {
-    LutArgs a;
-    a.bW = bW; a.alpha = (const _Float16*)alpha; a.qbias = (const _Float16*)q_bias;
-    a.x = (const _Float16*)x; a.y = (_Float16*)y; a.partial = nullptr; a.counters = nullptr;
-    a.K = K; a.N = N; a.nb = nbits; a.G = group_size; a.kslice = K; a.nsplit = 1; a.strict = 0;
+    if ((plan & ~HQ_LUT_PLAN_RAGGED) == HQ_LUT_PLAN_MFMA_GROUPED)
+      return group_size == 64 ? launch_bcq_grouped_nb<2>(a, ragged, stream) : launch_bcq_grouped_nb<4>(a, ragged, stream);
     switch (nbits) {  // quads per wave per round, bounded by the register budget
-      case 1: return launch_bcq_mfma<1, 2>(a, stream);
-      case 2: return launch_bcq_mfma<2, 2>(a, stream);
-      case 3: return launch_bcq_mfma<3, 2>(a, stream);
-      case 4: return launch_bcq_mfma<4, 2>(a, stream);
-      case 5: return launch_bcq_mfma<5, 2>(a, stream);
-      case 6: return launch_bcq_mfma<6, 2>(a, stream);
-      case 7: return launch_bcq_mfma<7, 1>(a, stream);
-      default: return launch_bcq_mfma<8, 1>(a, stream);
+      case 1: return launch_bcq_mfma<1, 2>(a, ragged, stream);
+      case 2: return launch_bcq_mfma<2, 2>(a, ragged, stream);
+      case 3: return launch_bcq_mfma<3, 2>(a, ragged, stream);
+      case 4: return launch_bcq_mfma<4, 2>(a, ragged, stream);
+      case 5: return launch_bcq_mfma<5, 2>(a, ragged, stream);
+      case 6: return launch_bcq_mfma<6, 2>(a, ragged, stream);
+      case 7: return launch_bcq_mfma<7, 1>(a, ragged, stream);
+      default: return launch_bcq_mfma<8, 1>(a, ragged, stream);
     }
   }
   const bool pair = (N % 2 == 0) && !((uintptr_t)bW & 7);
@@ -773,4 +800,11 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
   if (pair) hipLaunchKernelGGL(lut_gemv_kernel<2>, dim3(ntiles * nsplit), dim3(256), smem, stream, a);
   else hipLaunchKernelGGL(lut_gemv_kernel<1>, dim3(ntiles * nsplit), dim3(256), smem, stream, a);
   return hq_launch_status();
+}
+
+extern "C" int hq_lut_gemv_plan(const uint32_t* bW, const void* alpha, const void* q_bias, int K, int N, int nbits,
+                                int group_size) {
+  if (K <= 0 || N <= 0 || nbits < 1 || nbits > 8 || group_size <= 0) return HQ_ERR_BAD_SHAPE;
+  if ((K & 31) || (group_size & 31) || (K % group_size)) return HQ_ERR_BAD_SHAPE;
+  return lut_plan(bW, alpha, q_bias, K, N, group_size);
 }

@@ -160,13 +160,25 @@ int hq_q3_matvec_noalloc(const void* x, int x_dtype, const int32_t* qweight, con
  *   s = +1 if bit (k%32) of bW[k/32][b][n] is set, else -1
  * Layouts (src/lut-gemm-hip/nQWeight_fp16.h:24-26): bW uint32[K/32][nbits][N],
  * alpha fp16[K/G][nbits][N], q_bias fp16[K/G][N] or NULL, x fp16[K], y fp16[N].
- * K % 32 == 0, G % 32 == 0, K % G == 0, 1 <= nbits <= 8.
+ * K % 32 == 0, G % 32 == 0, K % G == 0, 1 <= nbits <= 8; any N.
  * Sums are kept in fp32 and rounded to fp16 once.  Replaces
  * matmul(output, input, nqW, m), src/lut-gemm-hip/kernels.cu:27-31.
  */
 int hq_lut_gemv(const uint32_t* bW, const void* alpha_fp16, const void* q_bias_fp16,
                 const void* x_fp16, void* y_fp16, int K, int N, int nbits, int group_size,
                 void* stream);
+
+/* Which kernel hq_lut_gemv takes for a problem (pointers matter through their alignment only; nothing is
+ * launched): HQ_LUT_PLAN_TABLE, or a matrix-core plan, with HQ_LUT_PLAN_RAGGED or-ed in when N is not a
+ * multiple of 64 or an operand is not 16-byte aligned.  Negative: the HQ_ERR_* code hq_lut_gemv would return
+ * for the shape.  The reference kernel takes any N (src/lut-gemm-hip/mv_fp16.h:229-236); so do the
+ * matrix-core plans for N >= 64 and K % 128 == 0. */
+#define HQ_LUT_PLAN_TABLE 0        /* 256-entry tables per 8-element sub-vector in LDS */
+#define HQ_LUT_PLAN_MFMA 1         /* group size a multiple of 128 */
+#define HQ_LUT_PLAN_MFMA_GROUPED 2 /* group size 64 or 32 */
+#define HQ_LUT_PLAN_RAGGED 16
+int hq_lut_gemv_plan(const uint32_t* bW, const void* alpha_fp16, const void* q_bias_fp16, int K, int N,
+                     int nbits, int group_size);
 
 /*
  * AQLM 1x16 code-book matvec (fp16 in, fp16 out):

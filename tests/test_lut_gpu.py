@@ -30,7 +30,10 @@ def _run(hq, bW, alpha, qbias, x, group):
     (4096, 16384, 3, 64, False, 12), (4096, 4096, 3, 32, False, 13), (1024, 256, 1, 32, False, 14),
     (2048, 128, 2, 64, True, 15), (1152, 192, 4, 32, False, 16), (640, 64, 5, 64, False, 17),
     (896, 128, 6, 32, False, 18), (512, 320, 7, 64, False, 19), (1280, 64, 8, 32, False, 20),
-    (128, 64, 3, 32, False, 21), (192, 64, 3, 64, False, 22)])
+    (128, 64, 3, 32, False, 21), (192, 64, 3, 64, False, 22),
+    # N not a multiple of 64 (rows start at any element): the matrix-core kernels with a shifted last tile
+    (1024, 1000, 3, 128, False, 23), (512, 72, 4, 64, False, 24), (256, 65, 2, 32, True, 25),
+    (4096, 11004, 3, 128, False, 26), (384, 127, 8, 128, False, 27)])
 def test_vs_oracle(hq, oracle, tunable, path, K, N, nb, group, zero_bias, seed):
     tunable("HQ_LUT_PATH", path)
     bW, alpha, qbias, x = oa.make_lut_problem(seed, K, N, nb, group, zero_bias)
@@ -40,6 +43,47 @@ def test_vs_oracle(hq, oracle, tunable, path, K, N, nb, group, zero_bias, seed):
     # ~4e-5 of the RMS, a fifth of the fp16 output rounding): far inside the contract
     assert rel_err(y, ref, FLOOR_F16) <= 2e-3
     assert rel_err(y, ref) <= TOL_F16_ACC
+
+
+def test_plans(hq):
+    """Which kernel a shape takes, asked of the library itself: ragged shapes stay on the matrix cores."""
+    from hecbench_amd import _lib
+    lib = _lib.load()
+    TABLE, MFMA, GROUPED, RAGGED = 0, 1, 2, 16
+    a16, a4, a2 = 4096, 4100, 4098            # stand-ins for pointers of 16-, 4- and 2-byte alignment
+    plan = lambda K, N, nb, G, bw=a16, al=a16, qb=a16: lib.hq_lut_gemv_plan(bw, al, qb, K, N, nb, G)
+    assert plan(4096, 16384, 3, 128) == MFMA
+    assert plan(4096, 16384, 3, 64) == GROUPED and plan(4096, 4096, 3, 32) == GROUPED
+    assert plan(512, 130, 3, 64) == GROUPED | RAGGED
+    assert plan(2048, 1001, 2, 2048) == MFMA | RAGGED
+    assert plan(4096, 16384, 3, 128, bw=a4) == MFMA | RAGGED       # aligned shape, unaligned operand
+    assert plan(4096, 16384, 3, 128, al=a2) == MFMA | RAGGED
+    assert plan(4096, 16384, 3, 128, qb=None) == MFMA              # no bias: nothing to align
+    assert plan(96, 64, 1, 32) == TABLE                            # K % 128
+    assert plan(4096, 48, 3, 128) == TABLE                         # fewer than 64 columns
+    assert plan(1536, 256, 3, 96) == TABLE                         # group size 96
+    assert plan(4096, 16384, 9, 128) == -2
+
+
+def test_unaligned_operands(hq, oracle):
+    """Operands that start 4 (bit planes) and 2 (alpha, bias) bytes past a 16-byte boundary."""
+    import torch
+    dev = torch.device("cuda:0")
+    K, N, nb, G = 1024, 256, 3, 128
+    bW, alpha, qbias, x = oa.make_lut_problem(77, K, N, nb, G, False)
+    def shifted(a, dtype, elems):
+        buf = torch.zeros(a.size + 16, dtype=dtype, device=dev)
+        view = buf[elems:elems + a.size]
+        view.copy_(torch.from_numpy(np.ascontiguousarray(a).reshape(-1)).to(dev))
+        return view
+    dW = shifted(bW.view(np.int32), torch.int32, 1).view(K // 32, nb, N)
+    da = shifted(alpha, torch.float16, 1).view(K // G, nb, N)
+    dq = shifted(qbias, torch.float16, 3).view(K // G, N)
+    assert dW.data_ptr() % 16 == 4 and da.data_ptr() % 16 == 2
+    y = hq.lut_matmul(torch.from_numpy(x).to(dev), dW, da, dq, G)
+    torch.cuda.synchronize()
+    ref = oracle.lut_gemv_f64(bW, alpha, qbias, x, G)
+    assert rel_err(y.cpu().numpy(), ref, FLOOR_F16) <= 2e-3
 
 
 def test_no_bias_pointer(hq, oracle):
