@@ -30,6 +30,7 @@ _SIGNATURES = {
                                         _c.c_void_p, _c.c_int, _c.c_int, _c.c_int, _c.c_uint, _c.c_void_p]),
     "hq_lut_gemv": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
                                _c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.c_void_p]),
+    "hq_q3_matvec_plan": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int]),
     "hq_lut_gemv_plan": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int, _c.c_int, _c.c_int]),
     "hq_aqlm_matvec": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p,
                                   _c.c_int, _c.c_int, _c.POINTER(_c.c_int), _c.c_int, _c.c_void_p]),

@@ -425,6 +425,9 @@ int launch_matvec(const Q3Args& a, int ntiles, hipStream_t stream) {
 int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros,
                       float* y, int K, int N, int M, unsigned flags, hipStream_t stream, const HqQ3Scratch* fixed);
 
+int hq_q3_rows_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
+                      int K, int N, int M, unsigned flags, hipStream_t stream);
+
 namespace {
 // Zeroes n words with a kernel (a memset node inside a captured graph is not an option for callers
 // that capture the stream).
@@ -433,6 +436,22 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(unsigned* p, int n) {
   if (i < n) p[i] = 0u;
 }
 }  // namespace
+
+namespace {
+int q3_plan(const HqDevice* dev, int N, int batch_M) {
+  if (batch_M == 1) return HQ_Q3_PLAN_MATVEC;
+  if (batch_M <= 3 && 2 * ((N + 63) / 64) >= dev->cus && hq_tune(HQ_TUNE_Q3_SMALL_BATCH, 1) != 0)
+    return HQ_Q3_PLAN_ROWS;
+  return HQ_Q3_PLAN_GEMM;
+}
+}  // namespace
+
+extern "C" int hq_q3_matvec_plan(int K, int N, int batch_M) {
+  if (K <= 0 || N <= 0 || batch_M <= 0 || (K & 31) || (N & 3)) return HQ_ERR_BAD_SHAPE;
+  const HqDevice* dev = nullptr;
+  const int rc = hq_current_device(&dev);
+  return rc != HQ_OK ? rc : q3_plan(dev, N, batch_M);
+}
 
 extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float* scales,
                             const float* zeros, float* y, int K, int N, int batch_M, unsigned flags,
@@ -456,6 +475,11 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   if (rc != HQ_OK) return rc;
   if (batch_M > 1) {
     if (x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
+    // Batches of 2 and 3 ride on the matvec's digit kernel (one pass over the weights, no workspace)
+    // when the column tiles alone give at least every other CU a workgroup; everything else takes the
+    // batched GEMM.
+    if (q3_plan(dev, N, batch_M) == HQ_Q3_PLAN_ROWS)
+      return hq_q3_rows_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream);
     return hq_q3_gemm_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream, fixed);
   }
 
