@@ -6,7 +6,7 @@
 //   y[n] = sum_k x[k] * ( q_bias[k/G][n] + sum_b alpha[k/G][b][n] * s(k,b,n) )
 //
 // Shapes with N % 64 == 0 and a group size that is a multiple of 128, 64 or 32 run on the matrix cores
-// (bcq_mfma_kernel and bcq_mfma_grouped_kernel below: the packed bits themselves are the operands, no
+// (bcq_planes_kernel and bcq_mfma_grouped_kernel below: the packed bits themselves are the operands, no
 // tables).
 // Every other shape runs the table kernel: for every 8-element sub-vector of x the 256
 // signed sums sum_j (+-x[j]) are tabulated once per workgroup in LDS (fp32 entries), and
@@ -191,20 +191,16 @@ __global__ __launch_bounds__(256) void lut_gemv_kernel(LutArgs a) {
 
 
 // ======================================================================================
-// Matrix-core path (group size a multiple of 128, N a multiple of 64).
+// Matrix-core paths (group size a multiple of 128: bcq_planes_kernel; 64 or 32: bcq_mfma_grouped_kernel).
 //
 // sum_k s*x = 2*(sum_k bit*x - (sum_k x)/2).  An fp4 (e2m1) nibble with only its lowest bit set
 // is the number 0.5, so `(word >> p) & 0x11111111` (p = 0..3) turns a packed 32-bit word into
 // the four operand registers (32 fp4 values) of one 16x16x128 f8f6f4 MFMA: seven VALU
 // instructions per 32 weights, no table, no LDS lookup.  The activations of a round are
-// scaled to 16-bit fixed point, biased by 0x8888 and cut into four nibbles; a nibble 0..15 in
-// an otherwise zero byte is the fp8 (e4m3) number nibble * 2^-9, so the digits need no
-// conversion, only a byte transpose.  MFMA column d carries nibble d, column 4 a constant one
-// (it counts the set bits, which takes the bias out at the very end), so every product is an
-// integer and the matrix-core sums are exact.  Lane quarter kb streams k-word 4*quad + kb, so
-// one MFMA sums a whole 128-element quad of one bit plane for 16 columns (four adjacent
-// columns per lane and 128-bit load); alpha is applied to that sum in fp32, per MFMA column,
-// and the columns are combined once at the end.
+// scaled to 16-bit fixed point and cut into four nibbles; a nibble 0..15 in an otherwise zero
+// byte is the fp8 (e4m3) number nibble * 2^-9, so the digits need no conversion, only a byte
+// transpose.  Every product is an integer and the matrix-core sums are exact; alpha is applied to
+// the sums in fp32 and everything is rounded to fp16 once.
 typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
@@ -272,83 +268,155 @@ __device__ __forceinline__ u4v load_words(const uint32_t* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const u4v*>(p));
 }
 
-// One B operand row is 4 lane quarters x 32 B, rows 128 B apart.  Rows 0, 2, 4 (and 1, 3) then share LDS banks
-// and the bank-conflict counter shows it; rows 144 B apart (an odd multiple of 16 B, no two rows on the same
-// banks) were built and measured SLOWER on MI355X - 10.05 against 9.57 us at K=4096, N=16384, 3 planes - so
-// the operand reads are not what bounds the kernel and the plain layout is kept.
-constexpr int kLutRow = 128;
-constexpr int kQuadBytes = 5 * kLutRow;  // B operand rows of one quad: four digits and the ones row
+// ---- group size a multiple of 128: up to three bit planes per MFMA ---------------------------------
+// A matvec has one activation vector, so of the sixteen rows of the activation operand only the four
+// digits would be used.  The bit planes fill the rest:
+//  - the weights are the SECOND operand: lane quarter kb of MFMA m of a quad (128 elements of K) streams
+//    block j = 4m + kb of the quad's 4*P (k-word, plane) blocks, k-word j / P and plane j % P (P <= 3 planes
+//    per set; consecutive rows of bW, since the planes of a k-word are adjacent): P MFMAs cover the quad
+//    for P planes and 16 columns, four adjacent columns per lane and 128-bit load;
+//  - the digits are the FIRST operand: row 4b + d holds digit d at the K positions of the blocks of plane b
+//    and zeros elsewhere.  Result row 4b + d, column n is then plane b's sum of digit d for weight column
+//    n over the whole quad, accumulated across the P MFMAs inside the matrix core: lane (n, kb) holds the
+//    four digits of plane kb in its four result registers, combines them in registers and applies
+//    alpha[plane kb][n] ONCE per quad, set and column block.  Lane quarter 3 of the first set carries the
+//    q_bias term the same way (its rows are zero; +sum(x)/2 is added to its sum where the others get -sum(x)/2);
+//  - the digits are sign-magnitude: |x| in 16-bit fixed point cut into four nibbles, the sign in the fp8
+//    sign bit of every digit byte, so no bias has to be taken out and no bit counts are needed;
+//  - one more MFMA per quad, all-ones weights against the plain digits, gives sum(x) of the quad.
+// Per 128 x 64 x 3-plane quad a lane spends 84 instructions on operands and about 30 on everything else,
+// and loads 8 bytes of alpha.  (A kernel with one plane per MFMA - digits as MFMA columns, alpha applied
+// per MFMA, 96 bytes of alpha per lane and quad - measured 9.57 us at K=4096, N=16384, 3 planes, this one
+// 8.24 us; its loads alone take 6.9 us.)
+typedef _Float16 h4v __attribute__((ext_vector_type(4)));
+typedef _Float16 h4v_any __attribute__((ext_vector_type(4), aligned(2)));
 
-// NB bit planes, QUADS 128-element quads per wave per round, WAVES waves per workgroup.
-// RAGGED: N is any number >= 64 and the operands have only their elements' alignment; the last tile then
-// starts at column N - 64 (it overlaps its neighbour, both write the same values to the shared columns).
+__device__ __forceinline__ f4 mfma_fp8_fp4(v8i a, v8i b, f4 c) {
+  // A fp8 e4m3 (cbsz 0), B fp4 e2m1 (blgp 4), both block scales 2^0
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 4, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+}
+
+constexpr int kDigQuad = 4 * 4 * 32 + 16;  // digits of one quad [k-word][digit][32 operand bytes], then 16 zero bytes
+constexpr int planes_of_set(int nb, int s) { return nb - 3 * s < 3 ? nb - 3 * s : 3; }
+
 template <int NB, int QUADS, int WAVES, bool BIAS, bool RAGGED>
-__global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
+__global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
+  constexpr int SETS = (NB + 2) / 3;
+  constexpr int SP = (QUADS + 1) / 2;  // staging passes per round (two quads per pass)
   extern __shared__ float lds[];
-  char* xs = reinterpret_cast<char*>(lds);                             // [waves][QUADS][5 rows][4 kb][32 B]
-  float* red = reinterpret_cast<float*>(xs + WAVES * QUADS * kQuadBytes);  // [waves][5 columns][64]
-  float* poison_w = red + WAVES * 5 * 64;                                  // [waves]
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  char* xs = reinterpret_cast<char*>(lds);                                   // [waves][QUADS][kDigQuad]
+  float* red = reinterpret_cast<float*>(xs + WAVES * QUADS * kDigQuad);      // [waves][4 quarters][64]
+  float* poison_w = red + WAVES * 4 * 64;                                    // [waves]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses of a round stay scalar
   const int c = lane & 15, kb = lane >> 4;
   const int tile = blockIdx.x;
   const int nquads = a.K >> 7;
   const size_t n0 = RAGGED ? (size_t)min(tile * 64, a.N - 64) : (size_t)tile * 64;
-  const uint32_t col_off = 4u * c;   // first of the lane's 4 columns (no partial tiles: N % 64 == 0 or RAGGED)
-  const uint32_t acol = 16u * kb;    // first of the 16 columns this lane applies alpha to
-  char* xs_w = xs + wv * (QUADS * kQuadBytes);
+  const uint32_t col_off = 4u * c;  // the lane's four columns: weights, alpha and results
+  char* xs_w = xs + wv * (QUADS * kDigQuad);
   // Staging role of a lane: 32 lanes per quad; lane (sa, sp, sh) owns the four activations
-  // k = 32*sa + 4*(4*sh + j) + sp, j = 0..3, i.e. A elements 8*sp + 4*sh + j of word sa.  The
-  // fp8 operand of lane quarter b holds MFMA K indices 16b .. 16b+15 in bytes 0..15 and
-  // 64+16b .. 64+16b+15 in bytes 16..31, the fp4 operand of quarter sa holds 32sa .. 32sa+31.
+  // k = 32*sa + 4*(4*sh + j) + sp, j = 0..3: elements 8*sp + 4*sh + j of the fp4 operand block of k-word sa
+  // (element e of a block is bit 4*(e & 7) + (e >> 3) of the word).
   const int st = lane >> 5, sa = (lane >> 3) & 3, sp = (lane >> 1) & 3, sh = lane & 1;
-  const int e0 = 8 * sp + 4 * sh;
-  const int s_quarter = 2 * (sa & 1) + (e0 >> 4), s_byte = 16 * (sa >> 1) + (e0 & 15);
-  constexpr int SP = (QUADS + 1) / 2;  // staging passes per round (two quads per pass)
+  const int stage_off = sa * 128 + (2 * sp + sh) * 4;
 
-  v8i ones;  // every slot's bit set: one MFMA with it sums the digits of a quad
+  // what a lane multiplies its combined digits with, per set: alpha of plane 3s + kb, the bias (quarter 3
+  // of set 0) or nothing (then its sums are zero)
+  const _Float16* cbase[SETS];
+  size_t cstride[SETS];  // elements per group
+  float half_sign[SETS];
 #pragma unroll
-  for (int r = 0; r < 8; ++r) ones[r] = r < 4 ? 0x11111111 : 0;
-  // row 4 of every quad is the constant one (fp8 0x01 = 2^-9, the unit of the digits)
-  if (lane < 32) {
-#pragma unroll
-    for (int t = 0; t < QUADS; ++t) *reinterpret_cast<uint32_t*>(xs_w + t * kQuadBytes + 4 * kLutRow + lane * 4) = 0x01010101u;
+  for (int s = 0; s < SETS; ++s) {
+    const int P = planes_of_set(NB, s);
+    const bool is_bias = BIAS && s == 0 && kb == 3;
+    const bool has_plane = kb < P;
+    cbase[s] = (is_bias ? a.qbias : a.alpha + (size_t)(3 * s + min(kb, P - 1)) * a.N) + n0 + col_off;
+    cstride[s] = is_bias ? (size_t)a.N : (size_t)NB * a.N;
+    half_sign[s] = is_bias ? 0.5f : (has_plane ? -0.5f : 0.f);
   }
 
-  float tot[4][4];
+  // byte offsets of the lane's weight rows inside a quad's 4*NB rows: block j = 4m + kb of set s is k-word
+  // j / P, plane 3s + j % P (a quad's rows stay below 4 GB: the host checks N)
+  uint32_t wbyte[NB];
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
+  for (int s = 0; s < SETS; ++s) {
+    const int P = planes_of_set(NB, s);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) tot[q][i] = 0.f;
+    for (int m = 0; m < 3; ++m) {
+      if (m >= P) continue;
+      const int j = 4 * m + kb;
+      wbyte[3 * s + m] = (uint32_t)(((size_t)((j / P) * NB + 3 * s + j % P) * a.N + n0 + col_off) * 4);
+    }
+  }
+
+  float tot[4] = {0.f, 0.f, 0.f, 0.f};
   float poison = 0.f;  // becomes NaN when an activation is NaN or infinite (the digits cannot carry that)
 
-  for (int q0 = wv * QUADS; q0 < nquads; q0 += WAVES * QUADS) {
-    // ---- loads of this round (unconditional, clamped): activations, then packed words -------
-    float xv[SP][4];
+  // One round of a wave: QUADS quads.  The loads of a round are issued one round ahead into the other of
+  // two register sets (the loop is unrolled by two, the sets swap without copies).
+  struct Round {
+    _Float16 xh[SP][4];
     u4v wq[QUADS][NB];
+    h4v cf[QUADS][SETS];
+  };
+  auto load_round = [&](int q0, Round& r) {  // unconditional, clamped
 #pragma unroll
     for (int sp_ = 0; sp_ < SP; ++sp_) {
       const int quad = min(q0 + min(2 * sp_ + st, QUADS - 1), nquads - 1);
       const _Float16* xp = a.x + (size_t)quad * 128 + 32 * sa + 16 * sh + sp;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xv[sp_][j] = (float)xp[4 * j];
+      for (int j = 0; j < 4; ++j) r.xh[sp_][j] = xp[4 * j];
     }
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
       const int quad = min(q0 + t, nquads - 1);
-      const uint32_t* wp = a.bW + ((size_t)(4 * quad + kb) * NB) * a.N + n0 + col_off;
+      const char* qb = reinterpret_cast<const char*>(a.bW + ((size_t)(4 * quad) * NB) * a.N);  // scalar
 #pragma unroll
-      for (int b = 0; b < NB; ++b) wq[t][b] = load_words<RAGGED>(wp + (size_t)b * a.N);
+      for (int i = 0; i < NB; ++i) r.wq[t][i] = load_words<RAGGED>(reinterpret_cast<const uint32_t*>(qb + wbyte[i]));
+      const int g = (quad * 128) / a.G;
+#pragma unroll
+      for (int s = 0; s < SETS; ++s) {
+        const _Float16* cp = cbase[s] + (size_t)g * cstride[s];
+        if (RAGGED) r.cf[t][s] = *reinterpret_cast<const h4v_any*>(cp);
+        else r.cf[t][s] = *reinterpret_cast<const h4v*>(cp);
+      }
     }
-    // alpha and bias of the round's quads: issued here so that they arrive with the words
-    Half16 al[QUADS][NB], bi[QUADS];
+  };
+  // The first round's loads go out before anything else is set up.
+  Round ra, rb;
+  int q0 = wv * QUADS;
+  load_round(q0, ra);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // Digit operand reads.  The fp8 operand of lane quarter kb holds MFMA K indices 16kb .. 16kb+15 in its
+  // first 16 bytes and 64+16kb .. 64+16kb+15 in its last 16: halves h = 0, 1 lie in block 2h + (kb >> 1),
+  // elements 16*(kb & 1) .. +15 of it.  Row c = 4b + d takes digit d there if the block's plane is b.
+  const int half_off = 16 * (kb & 1);
+  int doff[SETS][3][2];
 #pragma unroll
-    for (int t = 0; t < QUADS; ++t) {
-      const int g = (min(q0 + t, nquads - 1) * 128) / a.G;
+  for (int s = 0; s < SETS; ++s) {
+    const int P = planes_of_set(NB, s);
 #pragma unroll
-      for (int b = 0; b < NB; ++b) al[t][b] = load_half16<RAGGED>(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
-      if (BIAS) bi[t] = load_half16<RAGGED>(a.qbias + (size_t)g * a.N + n0 + acol);
-    }
-    // ---- scale to 16-bit fixed point, bias, cut into nibbles, stage (wave-local) ------------
+    for (int m = 0; m < 3; ++m)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int jj = 4 * m + 2 * h + (kb >> 1);
+        const int b = jj % P, kw = jj / P;
+        doff[s][m][h] = (m < P && (c >> 2) == b) ? (kw * 4 + (c & 3)) * 32 + half_off : 512;
+      }
+  }
+  // plain operand (every row r holds digit r & 3 of all four k-words): one MFMA with all-ones weights
+  // gives the digit sums of the quad in every lane
+  const int poff0 = ((kb >> 1) * 4 + (c & 3)) * 32 + half_off, poff1 = poff0 + 2 * 128;
+  v8i ones;
+#pragma unroll
+  for (int r = 0; r < 8; ++r) ones[r] = r < 4 ? 0x11111111 : 0;
+  if (lane < 4 * QUADS) *reinterpret_cast<uint32_t*>(xs_w + (lane >> 2) * kDigQuad + 512 + (lane & 3) * 4) = 0u;
+
+  auto compute_round = [&](int q0, const Round& r) {
+    // ---- scale to 16-bit fixed point magnitudes, cut into nibbles, sign into every byte, stage ----
+    float xv[SP][4];
     float amax = 0.f;
 #pragma unroll
     for (int sp_ = 0; sp_ < SP; ++sp_) {
@@ -356,15 +424,14 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
       const bool live = t < QUADS && q0 + t < nquads;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        if (!live) xv[sp_][j] = 0.f;
+        xv[sp_][j] = live ? (float)r.xh[sp_][j] : 0.f;
         poison = fmaf(xv[sp_][j], 0.f, poison);
         amax = fmaxf(amax, fabsf(xv[sp_][j]));
       }
     }
     const float xmax = wave_max(amax);
-    // 2^E * max|x| lies in [2^13, 2^14): v = rint(x * 2^E) + 0x8888 stays inside 16 bits and its
-    // nibbles n_d satisfy v = sum_d 16^d (n_d - 8)
-    int E = 13 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
+    // 2^E * max|x| lies in [2^14, 2^15): u = rint(|x| * 2^E) <= 2^15 stays inside 16 bits
+    int E = 14 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
     E = xmax > 0.f ? max(-120, min(120, E)) : 0;
     const float scaleE = __uint_as_float((uint32_t)(E + 127) << 23);
 #pragma unroll
@@ -372,91 +439,99 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
       uint32_t ev[4], od[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t u = (uint32_t)((int)rintf(xv[sp_][j] * scaleE) + 0x8888);
-        ev[j] = u & 0x0f0fu;         // nibbles 0 (byte 0) and 2 (byte 1)
-        od[j] = (u >> 4) & 0x0f0fu;  // nibbles 1 and 3
+        const uint32_t u = (uint32_t)(int)rintf(fabsf(xv[sp_][j]) * scaleE);
+        const uint32_t sg = (uint32_t)((int)__float_as_uint(xv[sp_][j]) >> 31) & 0x8080u;
+        ev[j] = (u & 0x0f0fu) | sg;         // nibbles 0 (byte 0) and 2 (byte 1)
+        od[j] = ((u >> 4) & 0x0f0fu) | sg;  // nibbles 1 and 3
       }
       // byte transposes: digit d of the four activations in one dword
-      const uint32_t pe = __builtin_amdgcn_perm(ev[1], ev[0], 0x05010400u);  // a0 b0 a2 b2
-      const uint32_t qe = __builtin_amdgcn_perm(ev[3], ev[2], 0x05010400u);  // c0 d0 c2 d2
+      const uint32_t pe = __builtin_amdgcn_perm(ev[1], ev[0], 0x05010400u);
+      const uint32_t qe = __builtin_amdgcn_perm(ev[3], ev[2], 0x05010400u);
       const uint32_t po = __builtin_amdgcn_perm(od[1], od[0], 0x05010400u);
       const uint32_t qo = __builtin_amdgcn_perm(od[3], od[2], 0x05010400u);
       const uint32_t dg[4] = {__builtin_amdgcn_perm(qe, pe, 0x05040100u), __builtin_amdgcn_perm(qo, po, 0x05040100u),
                               __builtin_amdgcn_perm(qe, pe, 0x07060302u), __builtin_amdgcn_perm(qo, po, 0x07060302u)};
       const int t = 2 * sp_ + st;
       if (t < QUADS) {
-        char* dst = xs_w + t * kQuadBytes + s_quarter * 32 + s_byte;
+        char* dst = xs_w + t * kDigQuad + stage_off;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(dst + d * kLutRow) = dg[d];
+        for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(dst + d * 32) = dg[d];
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     // ---- MFMAs ------------------------------------------------------------------------------------
-    float run[4][4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) run[q][i] = 0.f;
+    float run[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
       if (q0 + t >= nquads) break;  // wave-uniform
-      // MFMA columns 5..15 are never read: they re-use the ones row
-      const u4v* bp = reinterpret_cast<const u4v*>(xs_w + t * kQuadBytes + min(c, 4) * kLutRow + kb * 32);
-      const u4v b0 = bp[0], b1 = bp[1];
-      const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
-      // column sum of the quad (digits 0..3: sum of the nibbles; column 4: 128), in units of
-      // 2^-10, identical in all four result rows
-      const f4 dsum = mfma_fp4_fp8(ones, B, f4{0.f, 0.f, 0.f, 0.f});
-      const f4 init = {-0.5f * dsum[0], -0.5f * dsum[1], -0.5f * dsum[2], -0.5f * dsum[3]};
-      if (BIAS) {
+      const char* dq = xs_w + t * kDigQuad;
+      auto operand = [&](int o0, int o1) {
+        const u4v lo = *reinterpret_cast<const u4v*>(dq + o0), hi = *reinterpret_cast<const u4v*>(dq + o1);
+        const v8i A = {(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+        return A;
+      };
+      // digit sums of the quad (register i: digit i), in units of 2^-10, identical in all lanes
+      const f4 dsum = mfma_fp8_fp4(operand(poff0, poff1), ones, f4{0.f, 0.f, 0.f, 0.f});
+      const float xsum = fmaf(fmaf(fmaf(dsum[3], 16.f, dsum[2]), 16.f, dsum[1]), 16.f, dsum[0]);  // sum of the quad's x
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+      for (int s = 0; s < SETS; ++s) {
+        const int P = planes_of_set(NB, s);
+        const float h0 = half_sign[s] * xsum;  // sum s*x = 2 sum bit*x - sum x; +sum x / 2 for the bias quarter
+        f4 acc[4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) run[q][i] = fmaf(bi[t].get(4 * i + q), 0.5f * dsum[i], run[q][i]);
-      }
+        for (int q = 0; q < 4; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        const uint32_t words[4] = {wq[t][b].x, wq[t][b].y, wq[t][b].z, wq[t][b].w};
+        for (int m = 0; m < 3; ++m) {
+          if (m >= P) continue;
+          const v8i A = operand(doff[s][m][0], doff[s][m][1]);
+          const u4v wv4 = r.wq[t][3 * s + m];
+          const uint32_t words[4] = {wv4.x, wv4.y, wv4.z, wv4.w};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) acc[q] = mfma_fp8_fp4(A, unpack_bits_fp4(words[q]), acc[q]);
+        }
+        // registers 0..3 are the digits of the lane's plane for weight column 4c + q
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          // one MFMA = this column's sum over the quad of bit*nibble, minus half the column sum
-          const f4 acc = mfma_fp4_fp8(unpack_bits_fp4(words[q]), B, init);
-          // rows 4*kb + i of the tile's 16-column block q: column 16*kb + 4*i + q
-#pragma unroll
-          for (int i = 0; i < 4; ++i) run[q][i] = fmaf(al[t][b].get(4 * i + q), acc[i], run[q][i]);
+          const float h = fmaf(fmaf(fmaf(acc[q][3], 16.f, acc[q][2]), 16.f, acc[q][1]), 16.f, acc[q][0] + h0);
+          run[q] = fmaf((float)r.cf[t][s][q], h, run[q]);
         }
       }
     }
     const float descale = __uint_as_float((uint32_t)(127 - E) << 23);
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) tot[q][i] = fmaf(run[q][i], descale, tot[q][i]);
+    for (int q = 0; q < 4; ++q) tot[q] = fmaf(run[q], descale, tot[q]);
+    // the digits of this round are consumed before the next round overwrites them
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
+  };
+  {
+    constexpr int STRIDE = WAVES * QUADS;
+    while (q0 < nquads) {
+      if (q0 + STRIDE < nquads) load_round(q0 + STRIDE, rb);
+      compute_round(q0, ra);
+      q0 += STRIDE;
+      if (q0 >= nquads) break;
+      if (q0 + STRIDE < nquads) load_round(q0 + STRIDE, ra);
+      compute_round(q0, rb);
+      q0 += STRIDE;
+    }
   }
-  // ---- combine columns and waves ------------------------------------------------------------------
+  // ---- combine lane quarters (planes, bias) and waves --------------------------------------------------
   {
     const float wp = wave_sum(poison);
     if (lane == 0) poison_w[wv] = wp;
   }
-  if (c < 5) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) red[(wv * 5 + c) * 64 + 16 * kb + 4 * i + q] = tot[q][i];
-  }
+  *reinterpret_cast<f4*>(red + (wv * 4 + kb) * 64 + 4 * c) = f4{tot[0], tot[1], tot[2], tot[3]};
   __syncthreads();
   const int n = (int)n0 + tid;
   if (tid < 64 && n < a.N) {
     float v = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      const float* rw = red + (w * 5) * 64 + tid;
-      // digits 3..0, then the bias of 8 per nibble times the (centred) bit count of column 4
-      v += (((rw[192] * 16.f + rw[128]) * 16.f + rw[64]) * 16.f + rw[0]) - 34952.f * rw[256];
+      const float* rw = red + (w * 4) * 64 + tid;
+      v += (rw[0] + rw[64]) + (rw[128] + rw[192]);
       v += poison_w[w];
     }
     // operand units 2^-10, and the sums hold half of sum s*x
@@ -465,12 +540,20 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_kernel(LutArgs a) {
 }
 
 // ---- group sizes 64 and 32 --------------------------------------------------------------------------
-// A 128-element quad then spans GS = 2 or 4 alpha / bias groups, so one sum per quad is not enough.  The
+// Here the weights are the first operand (lane quarter kb streams k-word 4*quad + kb of one plane, one MFMA
+// sums a quad of one bit plane for 16 columns) and the digits the second: the activations are biased by
+// 0x8888 before they are cut into nibbles, MFMA column d carries nibble d, and a column of ones counts the
+// set bits, which takes the bias out at the very end.
+// A 128-element quad spans GS = 2 or 4 alpha / bias groups, so one sum per quad is not enough.  The
 // B operand gets a row per (group, digit): row 4g + d holds digit d at the K positions of group g and zeros
 // elsewhere (GS * 4 <= 16 MFMA columns), and a second operand holds a row of ones per group for the bit
 // counts; both are zeroed once, their constant parts written once, and only the digit bytes are rewritten
 // per round.  Every MFMA column then carries one group's sum, is scaled by that group's alpha (lane column
 // c takes the alpha of group c / 4), and the groups are added when the digits are combined at the end.
+// One B operand row is 4 lane quarters x 32 B, rows 128 B apart.  Rows 0, 2, 4 (and 1, 3) then share LDS banks
+// and the bank-conflict counter shows it; rows 144 B apart (an odd multiple of 16 B, no two rows on the same
+// banks) were built and measured slower, so the operand reads are not what bounds the kernel.
+constexpr int kLutRow = 128;
 constexpr int kGroupedQuadBytes = 20 * kLutRow;  // sixteen digit rows and up to four rows of ones
 constexpr int kGroupedRedBytes = 20 * 64 * 4;  // a wave's final sums: twenty columns of 64 outputs
 
@@ -704,15 +787,15 @@ int launch_bcq_grouped_nb(const LutArgs& a, bool ragged, hipStream_t stream) {
   }
 }
 
-// Eight waves per workgroup (two per SIMD, up to 256 VGPRs each): sixteen-wave variants
-// spill and measured slower.
+// Eight waves per workgroup (two per SIMD, up to 256 VGPRs each); QUADS is bounded by the two register
+// sets of a round's loads.
 template <int NB, int QUADS>
-int launch_bcq_mfma(const LutArgs& a, bool ragged, hipStream_t stream) {
+int launch_bcq_planes(const LutArgs& a, bool ragged, hipStream_t stream) {
   constexpr int WAVES = 8;
-  const size_t smem = (size_t)WAVES * QUADS * kQuadBytes + (size_t)WAVES * 5 * 64 * 4 + (size_t)WAVES * 4;
   const dim3 grid((a.N + 63) / 64), block(WAVES * 64);
+  const size_t smem = (size_t)WAVES * QUADS * kDigQuad + (size_t)WAVES * 4 * 64 * 4 + (size_t)WAVES * 4;
 #define HQ_LUT_GO(BIAS, RAG) \
-  hipLaunchKernelGGL((bcq_mfma_kernel<NB, QUADS, WAVES, BIAS, RAG>), grid, block, smem, stream, a)
+  hipLaunchKernelGGL((bcq_planes_kernel<NB, QUADS, WAVES, BIAS, RAG>), grid, block, smem, stream, a)
   if (a.qbias) { if (ragged) HQ_LUT_GO(true, true); else HQ_LUT_GO(true, false); }
   else { if (ragged) HQ_LUT_GO(false, true); else HQ_LUT_GO(false, false); }
 #undef HQ_LUT_GO
@@ -722,7 +805,7 @@ int launch_bcq_mfma(const LutArgs& a, bool ragged, hipStream_t stream) {
 // Which kernel a call takes (HQ_LUT_PLAN_* in hq.h).
 int lut_plan(const void* bW, const void* alpha, const void* q_bias, int K, int N, int group_size) {
   if (hq_tune(HQ_TUNE_LUT_PATH, 1) != 1) return HQ_LUT_PLAN_TABLE;
-  if (K % 128 != 0 || N < 64) return HQ_LUT_PLAN_TABLE;
+  if (K % 128 != 0 || N < 64 || N >= (1 << 25)) return HQ_LUT_PLAN_TABLE;  // 32-bit byte offsets inside 32 rows
   const bool aligned = N % 64 == 0 && !((uintptr_t)bW & 15) && !((uintptr_t)alpha & 15) && !((uintptr_t)q_bias & 15);
   int plan;
   if (group_size == 64 || group_size == 32) plan = HQ_LUT_PLAN_MFMA_GROUPED;
@@ -756,14 +839,14 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
     if ((plan & ~HQ_LUT_PLAN_RAGGED) == HQ_LUT_PLAN_MFMA_GROUPED)
       return group_size == 64 ? launch_bcq_grouped_nb<2>(a, ragged, stream) : launch_bcq_grouped_nb<4>(a, ragged, stream);
     switch (nbits) {  // quads per wave per round, bounded by the register budget
-      case 1: return launch_bcq_mfma<1, 2>(a, ragged, stream);
-      case 2: return launch_bcq_mfma<2, 2>(a, ragged, stream);
-      case 3: return launch_bcq_mfma<3, 2>(a, ragged, stream);
-      case 4: return launch_bcq_mfma<4, 2>(a, ragged, stream);
-      case 5: return launch_bcq_mfma<5, 2>(a, ragged, stream);
-      case 6: return launch_bcq_mfma<6, 2>(a, ragged, stream);
-      case 7: return launch_bcq_mfma<7, 1>(a, ragged, stream);
-      default: return launch_bcq_mfma<8, 1>(a, ragged, stream);
+      case 1: return launch_bcq_planes<1, 4>(a, ragged, stream);
+      case 2: return launch_bcq_planes<2, 4>(a, ragged, stream);
+      case 3: return launch_bcq_planes<3, 4>(a, ragged, stream);
+      case 4: return launch_bcq_planes<4, 2>(a, ragged, stream);
+      case 5: return launch_bcq_planes<5, 2>(a, ragged, stream);
+      case 6: return launch_bcq_planes<6, 2>(a, ragged, stream);
+      case 7: return launch_bcq_planes<7, 1>(a, ragged, stream);
+      default: return launch_bcq_planes<8, 1>(a, ragged, stream);
     }
   }
   const bool pair = (N % 2 == 0) && !((uintptr_t)bW & 7);
