@@ -426,7 +426,7 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
                       float* y, int K, int N, int M, unsigned flags, hipStream_t stream, const HqQ3Scratch* fixed);
 
 int hq_q3_rows_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                      int K, int N, int M, unsigned flags, hipStream_t stream);
+                      int K, int N, unsigned flags, hipStream_t stream);
 
 namespace {
 // Zeroes n words with a kernel (a memset node inside a captured graph is not an option for callers
@@ -440,7 +440,7 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(unsigned* p, int n) {
 namespace {
 int q3_plan(const HqDevice* dev, int N, int batch_M) {
   if (batch_M == 1) return HQ_Q3_PLAN_MATVEC;
-  if (batch_M <= 3 && 2 * ((N + 63) / 64) >= dev->cus && hq_tune(HQ_TUNE_Q3_SMALL_BATCH, 1) != 0)
+  if (batch_M == 2 && 2 * ((N + 63) / 64) >= dev->cus && hq_tune(HQ_TUNE_Q3_SMALL_BATCH, 1) != 0)
     return HQ_Q3_PLAN_ROWS;
   return HQ_Q3_PLAN_GEMM;
 }
@@ -475,11 +475,10 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   if (rc != HQ_OK) return rc;
   if (batch_M > 1) {
     if (x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
-    // Batches of 2 and 3 ride on the matvec's digit kernel (one pass over the weights, no workspace)
-    // when the column tiles alone give at least every other CU a workgroup; everything else takes the
-    // batched GEMM.
+    // A batch of 2 rides on the matvec's digit kernel (one pass over the weights, no workspace) when the
+    // column tiles alone give at least every other CU a workgroup; everything else takes the batched GEMM.
     if (q3_plan(dev, N, batch_M) == HQ_Q3_PLAN_ROWS)
-      return hq_q3_rows_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream);
+      return hq_q3_rows_launch(x, qweight, scales, zeros, y, K, N, flags, stream);
     return hq_q3_gemm_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream, fixed);
   }
 

@@ -1,15 +1,18 @@
-// GPTQ 3-bit matvec for two or three activation rows at once (batches of 2 and 3) for gfx950.
+// GPTQ 3-bit matvec for two activation rows at once (batch 2) for gfx950.
 //
 // The batch-1 kernel (q3.hip) leaves seven of the sixteen matrix-core columns unused: its B operand
-// carries the eight 4-bit digits of ONE fixed-point activation vector plus a column of ones.  fp16
-// activations need far fewer digits, so here the sixteen columns carry FIVE digits (20-bit fixed point
-// relative to the wave's largest magnitude of that row) of up to THREE rows, plus the ones column: the
-// packed weights are read once for the whole batch at the matvec's nine VALU instructions per 32 weights
-// instead of the batched GEMM's twenty plus its pre-pass.  Everything else follows q3.hip: a workgroup
-// owns a 64-column tile and all of K, a wave's 16-lane quarter streams one k-group per step as three
-// 128-bit loads, every wave stages its own digits in LDS behind a wave-local fence, all products and
-// partial sums inside the matrix core are small integers (exact), and the waves meet once at the end.
-// No counterpart in the reference (its kernels are batch 1: src/quant3MatMul-hip/kernels.h:12-217).
+// carries the eight 4-bit digits of ONE fixed-point activation vector plus a column of ones.  Here the
+// sixteen columns carry SEVEN digits of each of TWO rows: |x| in 28-bit fixed point relative to the wave's
+// largest magnitude of that row, cut into nibbles, the sign in the fp8 sign bit of every digit byte (so no
+// bias has to be taken out and no column of ones is needed).  The packed weights are read once for both
+// rows at the matvec's nine VALU instructions per 32 weights, instead of the batched GEMM's twenty plus
+// its pre-pass.  Everything else follows q3.hip: a workgroup owns a 64-column tile and all of K, a wave's
+// 16-lane quarter streams one k-group per step as three 128-bit loads, every wave stages its own digits
+// in LDS behind a wave-local fence, all products and partial sums inside the matrix core are small
+// integers (exact), and the waves meet once at the end.  (Three rows of five digits fit as well and were
+// built: 25.1 us against the GEMM's 26 at K=8192, N=28672, with 20-bit activations - not worth a second
+// accuracy class.)  No counterpart in the reference (its kernels are batch 1:
+// src/quant3MatMul-hip/kernels.h:12-217).
 #include "hq_internal.h"
 
 namespace {
@@ -52,8 +55,6 @@ __device__ __forceinline__ float wave_sum(float v) {
   v += dpp_f<0x140>(v);
   return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
 }
-// Row-wise broadcast of lane 15 of each 16-lane row (DPP row_newbcast:15): the ones column.
-__device__ __forceinline__ float row_bcast15(float v) { return dpp_f<0x15F>(v); }
 
 constexpr uint32_t low3_mask(int word) {
   uint32_t m = 0;
@@ -74,9 +75,9 @@ __device__ __forceinline__ void transpose4(uint32_t a, uint32_t b, uint32_t c, u
   o[3] = __builtin_amdgcn_perm(p3, p1, 0x07060302u);
 }
 
-constexpr int kDigits = 5;          // 4-bit digits per activation: 20-bit fixed point
+constexpr int kDigits = 7;          // 4-bit digits per activation: 28-bit fixed point
 constexpr int kRowBytes = 144;      // one B operand row (4 lane quarters x 32 B) plus 16 B: rows start 4 banks apart
-constexpr int kStepBytes = 2560;    // sixteen B operand rows of one step, padded
+constexpr int kStepBytes = 2560;    // fourteen digit rows and a row of zeros per step, padded
 constexpr int kRedStride = 68;      // floats per digit column of a wave's final sums
 __device__ __forceinline__ constexpr int step_off(int s) {
   return s * kStepBytes + (s & 1) * 32 + ((s >> 1) & 1) * 128;
@@ -89,7 +90,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
   char* dig = reinterpret_cast<char*>(smem);
   float* part = reinterpret_cast<float*>(dig + WAVES * STEPS * kStepBytes);
   float* wsum = part + WAVES * ROWS * 64;
-  static_assert(STEPS * kStepBytes >= 16 * kRedStride * 4, "a wave's digit area must hold its final sums");
+  static_assert(STEPS * kStepBytes >= 14 * kRedStride * 4, "a wave's digit area must hold its final sums");
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int c = lane & 15, kb = lane >> 4;
@@ -136,14 +137,14 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
   };
 
   char* dig_w = dig + wv * (STEPS * kStepBytes);
-  // Row 15 of every step is the constant one (fp8 0x01 = 2^-9, the unit of the digits); MFMA column c reads
-  // row c while it carries a digit (c < 5 ROWS) and the ones row otherwise.
+  // Row 14 of every step stays zero: MFMA column c reads row c while it carries a digit (c < 7 ROWS) and the
+  // zero row otherwise.
+  static_assert(kDigits * ROWS <= 14, "the digit rows and the zero row must fit the sixteen operand rows");
   if (lane < 32) {
 #pragma unroll
-    for (int s = 0; s < STEPS; ++s)
-      *reinterpret_cast<uint32_t*>(dig_w + step_off(s) + 15 * kRowBytes + lane * 4) = 0x01010101u;
+    for (int s = 0; s < STEPS; ++s) *reinterpret_cast<uint32_t*>(dig_w + step_off(s) + 14 * kRowBytes + lane * 4) = 0u;
   }
-  const int rowsel = c < kDigits * ROWS ? c : 15;
+  const int rowsel = c < kDigits * ROWS ? c : 14;
   const int my_row = min(c / kDigits, ROWS - 1);  // the activation row whose digit this lane's MFMA column carries
 
   float run[4][4];
@@ -184,9 +185,9 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
       }
       const float xmax = wave_max(amax);
       asum_total[m] += wave_sum(asum);
-      // 2^E * max|x| lies in [2^17, 2^18): v = rint(x * 2^E) + 0x88888 stays inside 20 bits and its
-      // nibbles n_d satisfy v = sum_d 16^d (n_d - 8)
-      int E = 17 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
+      // 2^E * max|x| lies in [2^27, 2^28): u = rint(|x| * 2^E) stays inside 28 bits (an fp16 maximum times
+      // 2^E is a multiple of 2^17), u = sum_d 16^d n_d
+      int E = 27 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
       E = xmax > 0.f ? max(-120, min(120, E)) : 0;
       const float scaleE = pow2f(E);
       if (my_row == m) descale_lane = pow2f(-E);
@@ -195,9 +196,10 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
         uint32_t ev[8], od[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const uint32_t t = (uint32_t)((int)rintf(xr[p][j] * scaleE) + 0x88888);
-          ev[j] = t & 0x000f0f0fu;         // nibbles 0 2 4
-          od[j] = (t >> 4) & 0x00000f0fu;  // nibbles 1 3
+          const uint32_t u = (uint32_t)(int)rintf(fabsf(xr[p][j]) * scaleE);
+          const uint32_t sg = (uint32_t)((int)__float_as_uint(xr[p][j]) >> 31) & 0x80808080u;  // fp8 sign bits
+          ev[j] = (u & 0x0f0f0f0fu) | sg;         // nibbles 0 2 4 6
+          od[j] = ((u >> 4) & 0x0f0f0f0fu) | sg;  // nibbles 1 3 5 (the fourth byte is a signed zero)
         }
         // even / odd elements of the k-group go to neighbouring lane quarters of the fp8 operand (see q3.hip)
         uint32_t de[2][4], dd[2][4];
@@ -210,11 +212,10 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
           char* dst = dig_w + step_off(s) + (kDigits * m) * kRowBytes + (xkb & 1) * 64 + (xkb >> 1) * 16 + xq * 4;
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
-            *reinterpret_cast<uint32_t*>(dst + 0 * kRowBytes + h * 32) = de[h][0];
-            *reinterpret_cast<uint32_t*>(dst + 1 * kRowBytes + h * 32) = dd[h][0];
-            *reinterpret_cast<uint32_t*>(dst + 2 * kRowBytes + h * 32) = de[h][1];
-            *reinterpret_cast<uint32_t*>(dst + 3 * kRowBytes + h * 32) = dd[h][1];
-            *reinterpret_cast<uint32_t*>(dst + 4 * kRowBytes + h * 32) = de[h][2];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<uint32_t*>(dst + (2 * i) * kRowBytes + h * 32) = de[h][i];
+#pragma unroll
+            for (int i = 0; i < 3; ++i) *reinterpret_cast<uint32_t*>(dst + (2 * i + 1) * kRowBytes + h * 32) = dd[h][i];
           }
         }
       }
@@ -243,15 +244,11 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
         acc[q] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, acc[q], 2, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
       }
     }
-    // column 15 holds 2^-12 * sum q: take the bias 8 out of every digit while all is an exact integer,
-    // then leave the fixed-point scale of the column's activation row
+    // leave the fixed-point scale of the column's activation row
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float unbiased = fmaf(row_bcast15(acc[q][i]), -8.f, acc[q][i]);
-        run[q][i] = fmaf(unbiased, descale_lane, run[q][i]);
-      }
+      for (int i = 0; i < 4; ++i) run[q][i] = fmaf(acc[q][i], descale_lane, run[q][i]);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
     if (r + 1 < rounds) {
@@ -322,12 +319,12 @@ int launch_rows(const RowsArgs& a, hipStream_t stream) {
 
 }  // namespace
 
-// Batches of 2 and 3 fp16 activation rows; the caller has validated the arguments.
+// Two fp16 activation rows; the caller has validated the arguments.
 int hq_q3_rows_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                      int K, int N, int M, unsigned flags, hipStream_t stream) {
+                      int K, int N, unsigned flags, hipStream_t stream) {
   RowsArgs a;
   a.x = reinterpret_cast<const _Float16*>(x);
   a.w = reinterpret_cast<const uint32_t*>(qweight);
   a.scales = scales; a.zeros = zeros; a.y = y; a.K = K; a.N = N; a.flags = flags & HQ_FLAG_ACCUMULATE;
-  return M == 2 ? launch_rows<2>(a, stream) : launch_rows<3>(a, stream);
+  return launch_rows<2>(a, stream);
 }

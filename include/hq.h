@@ -131,11 +131,11 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  * batch_M == 1 replaces vecquant3matmul / vecquant3matmul_faster
  * (src/quant3MatMul-hip/kernels.h:171-217) — pass HQ_FLAG_ACCUMULATE for their
  * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 (no counterpart in the
- * reference): batches of 2 and 3 with at least one 64-column tile per two compute
- * units run on the matvec's kernel with the rows side by side in the matrix-core
- * operand (20-bit fixed point relative to the largest magnitude among each 512
- * consecutive activations of a row, so exact for fp16 entries within 2^7 of it and
- * to 2^-18 of it otherwise); all other batches run the MFMA GEMM path.
+ * reference): a batch of 2 with at least one 64-column tile per two compute units
+ * runs on the matvec's kernel with the two rows side by side in the matrix-core
+ * operand (28-bit fixed point relative to the largest magnitude among each 512
+ * consecutive activations of a row: exact for fp16 entries within 2^17 of it);
+ * all other batches run the MFMA GEMM path.
  */
 int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float* scales,
                  const float* zeros, float* y, int K, int N, int batch_M, unsigned flags,
@@ -146,7 +146,7 @@ int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float
  * tunables (for tests and tuning; negative = error code).
  */
 #define HQ_Q3_PLAN_MATVEC 0 /* batch_M == 1 */
-#define HQ_Q3_PLAN_ROWS 1   /* batch_M 2 or 3 on the matvec's digit kernel */
+#define HQ_Q3_PLAN_ROWS 1   /* batch_M == 2 on the matvec's digit kernel */
 #define HQ_Q3_PLAN_GEMM 2   /* batched MFMA GEMM */
 int hq_q3_matvec_plan(int K, int N, int batch_M);
 

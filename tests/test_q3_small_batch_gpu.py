@@ -1,5 +1,5 @@
-"""Batches 2 ... 15 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): batches of 2 and 3 on
-wide matrices run on the matvec's digit kernel with the rows side by side in the matrix-core operand,
+"""Batches 2 ... 15 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): a batch of 2 on a wide
+matrix runs on the matvec's digit kernel with the two rows side by side in the matrix-core operand,
 all others on the batched GEMM.  Every batch size is checked against the CPU oracle through the C ABI,
 and the kernel that ran is asserted through hq_q3_matvec_plan.  The reference has no batched kernel:
 the oracle is the matvec formula applied row by row (parity unpinned by the reference)."""
@@ -43,20 +43,19 @@ def _check(y, exact):
 @pytest.mark.parametrize("K,N", [(512, 16388), (4128, 8192), (1024, 132)])
 def test_every_batch_vs_oracle(hq, oracle, M, K, N):
     if K == 4128 and M > 4:
-        pytest.skip("the long-K shape is there for the kernel of batches 2 and 3")
+        pytest.skip("the long-K shape is there for the two-row kernel and its neighbours")
     codes, scales, zeros, A = oa.make_q3_problem(1000 + 16 * M + (K % 7), K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
-    want_plan = PLAN_ROWS if (M <= 3 and N > 8000) else PLAN_GEMM
+    want_plan = PLAN_ROWS if (M == 2 and N > 8000) else PLAN_GEMM
     assert _plan(K, N, M) == want_plan
     y = _run(hq, A, mat, scales, zeros)
     _check(y, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
 
 
-@pytest.mark.parametrize("M", [2, 3])
-def test_rows_kernel_against_the_gemm_and_the_matvec(hq, oracle, tunable, M):
-    """The same call with the small-batch kernel switched off takes the GEMM; each row also equals the
+def test_rows_kernel_against_the_gemm_and_the_matvec(hq, oracle, tunable):
+    """The same call with the two-row kernel switched off takes the GEMM; each row also equals the
     batch-1 matvec on that row.  Three kernels, one result (to the accuracy each of them states)."""
-    K, N = 2048, 16640
+    M, K, N = 2, 2048, 16640
     codes, scales, zeros, A = oa.make_q3_problem(500 + M, K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
     assert _plan(K, N, M) == PLAN_ROWS
@@ -72,7 +71,7 @@ def test_rows_kernel_against_the_gemm_and_the_matvec(hq, oracle, tunable, M):
 
 @pytest.mark.parametrize("scale_exp", [-16, -8, 0, 4])
 def test_rows_kernel_dynamic_range(hq, oracle, scale_exp):
-    """Rows of very different magnitude side by side in one matrix-core operand, an all-zero row, a row
+    """Two rows of very different magnitude side by side in one matrix-core operand, an all-zero row, a row
     with one large outlier, magnitudes spread over 2^8 inside a row, fp16 subnormals: every row is held
     to the bound the N(0,1) cases meet, measured against that row's own RMS."""
     K, N = 2048, 8256
@@ -88,7 +87,7 @@ def test_rows_kernel_dynamic_range(hq, oracle, scale_exp):
         np.exp2(rng.integers(-8, 1, K)).astype(np.float32)
     A[7, 512:] = 0.0                                       # whole rounds of a wave are zero
     A = A.astype(np.float16)
-    for rows in ([0, 1, 2], [3, 4, 5], [6, 7], [4, 8]):
+    for rows in ([0, 1], [2, 4], [3, 5], [6, 7], [4, 8]):
         sub = np.ascontiguousarray(A[rows])
         assert _plan(K, N, len(rows)) == PLAN_ROWS
         y = _run(hq, sub, mat, scales, zeros)
@@ -114,8 +113,8 @@ def test_rows_kernel_non_finite_activations(hq, oracle):
 
 
 def test_config4_shape_batches_2_and_3(hq, oracle):
-    """K=8192, N=28672 (the GEMM configuration's weights) at batches 2 and 3: sampled columns against the
-    oracle, all columns against the batch-1 matvec."""
+    """K=8192, N=28672 (the GEMM configuration's weights) at batch 2 (two-row kernel) and 3 (GEMM): sampled
+    columns against the oracle, all columns against the batch-1 matvec."""
     import torch
     K, N = 8192, 28672
     rng = np.random.default_rng(45)
@@ -127,7 +126,7 @@ def test_config4_shape_batches_2_and_3(hq, oracle):
     sub = np.ascontiguousarray(mat[:, cols])
     for M in (2, 3):
         A = rng.standard_normal((M, K)).astype(np.float16)
-        assert _plan(K, N, M) == PLAN_ROWS
+        assert _plan(K, N, M) == (PLAN_ROWS if M == 2 else PLAN_GEMM)
         y = hq.q3_gemm(_t(A), dm, ds, dz)
         torch.cuda.synchronize()
         y = y.cpu().numpy()
@@ -137,12 +136,11 @@ def test_config4_shape_batches_2_and_3(hq, oracle):
             assert rel_err(y[m], yv) <= 5e-3
 
 
-@pytest.mark.parametrize("M", [2, 3])
-def test_rows_kernel_accumulates(hq, oracle, M):
+def test_rows_kernel_accumulates(hq, oracle):
     """HQ_FLAG_ACCUMULATE adds to what y holds, as for batch 1."""
     import torch
     from hecbench_amd import _lib
-    K, N = 256, 8196
+    M, K, N = 2, 256, 8196
     codes, scales, zeros, A = oa.make_q3_problem(300 + M, K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
     rng = np.random.default_rng(5)
