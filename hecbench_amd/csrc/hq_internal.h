@@ -66,3 +66,20 @@ enum HqTunable {
   HQ_TUNE_NF4_PIPE, HQ_TUNE_AQLM_ROWS, HQ_TUNE_Q8_WGS, HQ_TUNE_Q8_FAST, HQ_TUNE_ACTQ_GROUPS, HQ_TUNE_SPLITK_FENCES, HQ_TUNE_COUNT
 };
 int hq_tune(HqTunable id, int dflt);
+
+// Streaming stores: write-through (sc1) and nontemporal (nt), i.e. the data is on its way to memory at once
+// and is not kept in the L2.  For a 33.5 MB write stream on MI355X: 5.80 us against 6.46 us with nt alone
+// and 7.04 us with plain stores.  The compiler cannot see that the assembly is a store, so the wait states it
+// would put between a store of more than 64 bits and the next write to the data registers are part of the
+// assembly.
+typedef uint32_t hq_u2v __attribute__((ext_vector_type(2)));
+typedef uint32_t hq_u4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void hq_store_stream(hq_u4v* p, hq_u4v v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void hq_store_stream(hq_u2v* p, hq_u2v v) {
+  asm volatile("global_store_dwordx2 %0, %1, off sc1 nt" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void hq_store_stream(uint32_t* p, uint32_t v) {
+  asm volatile("global_store_dword %0, %1, off sc1 nt" ::"v"(p), "v"(v) : "memory");
+}

@@ -39,9 +39,7 @@ __device__ __forceinline__ float mul_rounded_f32(float a, float b) {
 // Streaming 128-bit store, write-through and non-temporal ("sc1 nt"): the line goes straight to memory
 // and is not kept in the L2.  Measured on MI355X for a 33.5 MB write stream: 5.80 us against 6.46 us
 // with nt alone and 7.04 us with plain stores; with the 9.4 MB of reads next to it 7.23 against 7.32 us.
-__device__ __forceinline__ void store_stream(u4v* p, u4v v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" ::"v"(p), "v"(v) : "memory");
-}
+__device__ __forceinline__ void store_stream(u4v* p, u4v v) { hq_store_stream(reinterpret_cast<hq_u4v*>(p), v); }
 
 // The fp32 product as an instruction of its own (one rounding), so that the conversion to fp16 that follows
 // is a second rounding: written as inline assembly, the compiler can neither fuse the two nor needs a copy.
