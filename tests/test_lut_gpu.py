@@ -28,6 +28,8 @@ def _run(hq, bW, alpha, qbias, x, group):
     (8192, 64, 7, 256, False, 10), (384, 128, 6, 384, False, 11),
     # several rounds per wave (the next round's loads in flight), the last one partly filled
     (12416, 128, 3, 128, False, 28), (16384, 64, 2, 256, True, 29), (5248, 192, 4, 128, False, 30),
+    # fewer quads than waves
+    (128, 64, 3, 128, False, 31), (256, 64, 1, 256, False, 32), (640, 128, 8, 128, True, 33),
     # group sizes 64 and 32: the grouped matrix-core kernel (N % 64 == 0, K % 128 == 0), every plane count
     (4096, 16384, 3, 64, False, 12), (4096, 4096, 3, 32, False, 13), (1024, 256, 1, 32, False, 14),
     (2048, 128, 2, 64, True, 15), (1152, 192, 4, 32, False, 16), (640, 64, 5, 64, False, 17),

@@ -155,3 +155,13 @@ def test_rows_kernel_accumulates(hq, oracle):
     got = dy.cpu().numpy() - y0
     for m in range(M):
         assert rel_err(got[m], exact[m], FLOOR_F16) <= 1e-3   # y0 ~ 1 costs a few fp32 ulps of it
+
+
+@pytest.mark.parametrize("K", [32, 96, 160])
+def test_rows_kernel_short_k(hq, oracle, K):
+    """Fewer k-groups than a workgroup's waves cover: idle waves, partly filled steps."""
+    N = 8200
+    codes, scales, zeros, A = oa.make_q3_problem(700 + K, K, N, x_dtype=np.float16, batch=2)
+    mat = oracle.q3_pack(codes)
+    assert _plan(K, N, 2) == PLAN_ROWS
+    _check(_run(hq, A, mat, scales, zeros), oracle.q3_gemm(A, mat, scales, zeros, mode=0))
