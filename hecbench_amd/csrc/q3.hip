@@ -486,8 +486,7 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   const int ntiles = (N + 63) / 64;
   // Launch shape: a workgroup of WAVES waves covers WAVES*4*STEPS k-groups per round and
   // walks its K range in rounds (the next round's loads are in flight during the current
-  // one).  K is split across workgroups only as far as needed to give every CU a
-  // workgroup: the split costs a device-scope round trip per workgroup.
+  // one), or K is split across workgroups whose partial sums the last one to arrive adds up.
   int waves = hq_tune(HQ_TUNE_Q3_WAVES, 8);
   int steps = hq_tune(HQ_TUNE_Q3_STEPS, 0);
   if (waves != 4 && waves != 8 && waves != 16) waves = 8;
@@ -499,7 +498,18 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   const int gpr = waves * 4 * steps;  // k-groups one workgroup covers per round
   const int max_split = (G + gpr - 1) / gpr;
   int nsplit = hq_tune(HQ_TUNE_Q3_KSPLIT, 0);
-  if (nsplit <= 0) nsplit = dev->cus / ntiles;  // only when there are fewer tiles than half the CUs
+  if (nsplit <= 0) {
+    // Up to eight rounds of K: one workgroup per round.  Single-round workgroups need half the registers,
+    // so two share a CU and one's reduction tail runs under the other's loads, and 2-8 times as many
+    // workgroups spread evenly over the CUs whatever the tile count (at K=8192: N=22016, 344 tiles, 20.4 ->
+    // 15.1 us; N=28672, 448 tiles, 21.4 -> 18.6 us; K=28672, N=8192 21.7 -> 19.6 us).  Longer K: only as
+    // many splits as it takes to give every CU a workgroup - each split adds a partial-sum row per tile
+    // and a device-scope round trip (K=49152, N=12288: 43 us unsplit, 51-58 us split).
+    nsplit = max_split <= 8 ? max_split : dev->cus / ntiles;
+    if (fixed && nsplit > 1 &&
+        ((size_t)ntiles * nsplit * 64 > fixed->partial_floats || (size_t)ntiles > fixed->ncounters))
+      nsplit = dev->cus / ntiles;  // the fixed scratch is too small for the full split
+  }
   if (nsplit > max_split) nsplit = max_split;
   if (nsplit < 1) nsplit = 1;
   int gpw = (G + nsplit - 1) / nsplit;

@@ -143,6 +143,25 @@ def test_launch_shapes_match(hq, oracle, tunable):
                 tunable("HQ_SPLITK_FENCES", 0)
 
 
+@pytest.mark.parametrize("K,N", [(8192, 22016), (16384, 16644), (28672, 1028), (5120, 13824)])
+def test_default_k_split_on_long_k(hq, oracle, tunable, K, N):
+    """Up to eight rounds of K run as one workgroup per round whatever the tile count (more column tiles than
+    compute units included): sampled columns against the oracle, every column against the unsplit launch."""
+    rng = np.random.default_rng(K + N)
+    mat = rng.integers(-2 ** 31, 2 ** 31, size=(3 * K // 32, N), dtype=np.int64).astype(np.int32)
+    scales = rng.uniform(0.005, 0.02, size=N).astype(np.float32)
+    zeros = (scales * rng.integers(3, 5, size=N)).astype(np.float32)
+    x = rng.standard_normal(K).astype(np.float32)
+    y = _run(hq, x, mat, scales, zeros)
+    y_again = _run(hq, x, mat, scales, zeros)          # the arrival counters reset themselves
+    assert np.array_equal(y, y_again)
+    cols = np.unique(np.concatenate([np.arange(0, 68), np.arange(N - 68, N), rng.integers(0, N, 64)]))
+    ref = oracle.q3_matvec_f64(x, np.ascontiguousarray(mat[:, cols]), scales[cols], zeros[cols])
+    assert rel_err(y[cols], ref) <= 1e-4
+    tunable("HQ_Q3_KSPLIT", 1)
+    assert rel_err(y, _run(hq, x, mat, scales, zeros)) <= 1e-4
+
+
 def test_rejects_bad_arguments(hq):
     import torch
     dev = torch.device("cuda:0")
