@@ -118,11 +118,16 @@ extern "C" int hq_reserve_workspace(void* stream, int max_K, int max_N) {
   int rc = hq_current_device(&d);
   if (rc != HQ_OK) return rc;
   // batched GEMM: re-ordered activations of 64 rows (128 bytes per input feature, K padded to 1024) plus
-  // the row sums and scales; split-K matvecs: at most one partial row of 64 floats per compute unit
+  // the row sums and scales; split-K matvecs: a partial row of 64 floats per column tile and split - up to
+  // eight splits (one per 4096 elements of K) whatever the tile count, beyond that only as many as give every
+  // compute unit a workgroup (the LUT table kernel: two per compute unit, 128 floats each)
   const size_t kpad = ((size_t)max_K + 1023) / 1024 * 1024;
   const size_t gemm_floats = kpad * 32 + 128;
   const size_t tiles = ((size_t)max_N + 63) / 64;
-  const size_t split_floats = (tiles > (size_t)d->cus ? tiles : (size_t)d->cus) * 64 * 2;
+  const size_t rounds = ((size_t)max_K + 4095) / 4096;
+  const size_t full_split = tiles * (rounds <= 8 ? rounds : 1);
+  const size_t per_cu = tiles + 2 * (size_t)d->cus;
+  const size_t split_floats = (full_split > per_cu ? full_split : per_cu) * 64 * 2;
   HqWorkspace ws;
   return hq_get_workspace((hipStream_t)stream, gemm_floats > split_floats ? gemm_floats : split_floats,
                           tiles > 1 ? tiles : 1, &ws);

@@ -1,0 +1,65 @@
+"""Calls recorded into a HIP graph: after hq_reserve_workspace the entry points that use a workspace (split-K
+matvec, batched GEMM) allocate nothing during capture, and hq_q3_matvec_noalloc never does.  Every replay is
+checked against the eager result, with eager work and synchronisations between the replays."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from tests import oracle_api as oa
+
+pytestmark = pytest.mark.gpu
+
+
+def _t(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+
+
+def test_replays_match_eager(hq, oracle):
+    import torch
+    from hecbench_amd import _lib
+    lib = _lib.load()
+    K, N = 8192, 8256                       # two rounds of K: split over two workgroups per tile (workspace)
+    codes, scales, zeros, x = oa.make_q3_problem(901, K, N)
+    mat = oracle.q3_pack(codes)
+    Kg, Ng, M = 1024, 516, 16               # batched GEMM: pre-pass and main kernel meet in the workspace
+    codes_g, scales_g, zeros_g, A = oa.make_q3_problem(902, Kg, Ng, x_dtype=np.float16, batch=M)
+    mat_g = oracle.q3_pack(codes_g)
+    dx, dm, ds, dz = _t(x), _t(mat), _t(scales), _t(zeros)
+    dA, dmg, dsg, dzg = _t(A), _t(mat_g), _t(scales_g), _t(zeros_g)
+    y = torch.zeros(N, device="cuda:0")
+    y_na = torch.zeros(N, device="cuda:0")
+    yg = torch.zeros(M, Ng, device="cuda:0")
+    stream = torch.cuda.Stream()
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def noalloc(s):
+        rc = lib.hq_q3_matvec_noalloc(vp(dx), 0, vp(dm), vp(ds), vp(dz), vp(y_na), K, N, 1, 0,
+                                      ctypes.c_void_p(s.cuda_stream))
+        assert rc == 0, rc
+
+    with torch.cuda.stream(stream):
+        assert lib.hq_reserve_workspace(ctypes.c_void_p(stream.cuda_stream), K, N) == 0
+        hq.q3_matvec(dx, dm, ds, dz, out=y)
+        hq.q3_gemm(dA, dmg, dsg, dzg, out=yg)
+        noalloc(stream)
+    stream.synchronize()
+    want, want_g, want_na = y.clone(), yg.clone(), y_na.clone()
+    assert torch.equal(want, want_na)
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        hq.q3_matvec(dx, dm, ds, dz, out=y)
+        hq.q3_gemm(dA, dmg, dsg, dzg, out=yg)
+        noalloc(torch.cuda.current_stream())
+    for rep in range(4):
+        y.fill_(float(rep)); yg.fill_(-1.0); y_na.fill_(7.0)       # eager work between the replays
+        other = hq.q3_matvec(dx, dm, ds, dz)                       # an eager call on another stream's workspace
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), rep
+        assert torch.equal(yg, want_g), rep
+        assert torch.equal(y_na, want_na), rep
+        assert torch.equal(other, want), rep
