@@ -302,7 +302,6 @@ constexpr int planes_of_set(int nb, int s) { return nb - 3 * s < 3 ? nb - 3 * s 
 template <int NB, int QUADS, int WAVES, bool BIAS, bool RAGGED>
 __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
   constexpr int SETS = (NB + 2) / 3;
-  constexpr int SP = (QUADS + 1) / 2;  // staging passes per round (two quads per pass)
   extern __shared__ float lds[];
   char* xs = reinterpret_cast<char*>(lds);                                   // [waves][QUADS][kDigQuad]
   float* red = reinterpret_cast<float*>(xs + WAVES * QUADS * kDigQuad);      // [waves][4 quarters][64]
@@ -315,11 +314,12 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
   const size_t n0 = RAGGED ? (size_t)min(tile * 64, a.N - 64) : (size_t)tile * 64;
   const uint32_t col_off = 4u * c;  // the lane's four columns: weights, alpha and results
   char* xs_w = xs + wv * (QUADS * kDigQuad);
-  // Staging role of a lane: 32 lanes per quad; lane (sa, sp, sh) owns the four activations
-  // k = 32*sa + 4*(4*sh + j) + sp, j = 0..3: elements 8*sp + 4*sh + j of the fp4 operand block of k-word sa
-  // (element e of a block is bit 4*(e & 7) + (e >> 3) of the word).
-  const int st = lane >> 5, sa = (lane >> 3) & 3, sp = (lane >> 1) & 3, sh = lane & 1;
-  const int stage_off = sa * 128 + (2 * sp + sh) * 4;
+  // Staging role of a lane: 16 lanes per quad; lane (st, sm) owns the eight consecutive activations
+  // 8*sm .. 8*sm+7 of quad st (one 128-bit load).  Element e of the fp4 operand block of a k-word is bit
+  // 4*(e & 7) + (e >> 3) of the word, so activation 8*(sm & 3) + i of k-word sm >> 2 is element
+  // 8*(i & 3) + 2*(sm & 3) + (i >> 2): activations i and i + 4 are neighbours in a digit row.
+  const int st = lane >> 4, sm = lane & 15;
+  const int stage_off = (sm >> 2) * 128 + 2 * (sm & 3);
 
   // what a lane multiplies its combined digits with, per set: alpha of plane 3s + kb, the bias (quarter 3
   // of set 0) or nothing (then its sums are zero)
@@ -356,17 +356,14 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
   // One round of a wave: QUADS quads.  The loads of a round are issued one round ahead into the other of
   // two register sets (the loop is unrolled by two, the sets swap without copies).
   struct Round {
-    _Float16 xh[SP][4];
+    u4v xh;  // eight fp16 activations
     u4v wq[QUADS][NB];
     h4v cf[QUADS][SETS];
   };
   auto load_round = [&](int q0, Round& r) {  // unconditional, clamped
-#pragma unroll
-    for (int sp_ = 0; sp_ < SP; ++sp_) {
-      const int quad = min(q0 + min(2 * sp_ + st, QUADS - 1), nquads - 1);
-      const _Float16* xp = a.x + (size_t)quad * 128 + 32 * sa + 16 * sh + sp;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) r.xh[sp_][j] = xp[4 * j];
+    {
+      const int quad = min(q0 + min(st, QUADS - 1), nquads - 1);
+      r.xh = *reinterpret_cast<const u4v*>(a.x + (size_t)quad * 128 + 8 * sm);
     }
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
@@ -416,17 +413,16 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
 
   auto compute_round = [&](int q0, const Round& r) {
     // ---- scale to 16-bit fixed point magnitudes, cut into nibbles, sign into every byte, stage ----
-    float xv[SP][4];
+    float xv[8];
     float amax = 0.f;
+    const bool live = st < QUADS && q0 + st < nquads;
+    {
+      const h8 h = __builtin_bit_cast(h8, r.xh);
 #pragma unroll
-    for (int sp_ = 0; sp_ < SP; ++sp_) {
-      const int t = 2 * sp_ + st;
-      const bool live = t < QUADS && q0 + t < nquads;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        xv[sp_][j] = live ? (float)r.xh[sp_][j] : 0.f;
-        poison = fmaf(xv[sp_][j], 0.f, poison);
-        amax = fmaxf(amax, fabsf(xv[sp_][j]));
+      for (int j = 0; j < 8; ++j) {
+        xv[j] = live ? (float)h[j] : 0.f;
+        poison = fmaf(xv[j], 0.f, poison);
+        amax = fmaxf(amax, fabsf(xv[j]));
       }
     }
     const float xmax = wave_max(amax);
@@ -434,28 +430,27 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
     int E = 14 - ((int)((__float_as_uint(xmax) >> 23) & 255u) - 127);
     E = xmax > 0.f ? max(-120, min(120, E)) : 0;
     const float scaleE = __uint_as_float((uint32_t)(E + 127) << 23);
+    {
+      uint32_t ev[8], od[8];
 #pragma unroll
-    for (int sp_ = 0; sp_ < SP; ++sp_) {
-      uint32_t ev[4], od[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t u = (uint32_t)(int)rintf(fabsf(xv[sp_][j]) * scaleE);
-        const uint32_t sg = (uint32_t)((int)__float_as_uint(xv[sp_][j]) >> 31) & 0x8080u;
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t u = (uint32_t)(int)rintf(fabsf(xv[j]) * scaleE);
+        const uint32_t sg = (uint32_t)((int)__float_as_uint(xv[j]) >> 31) & 0x8080u;
         ev[j] = (u & 0x0f0fu) | sg;         // nibbles 0 (byte 0) and 2 (byte 1)
         od[j] = ((u >> 4) & 0x0f0fu) | sg;  // nibbles 1 and 3
       }
-      // byte transposes: digit d of the four activations in one dword
-      const uint32_t pe = __builtin_amdgcn_perm(ev[1], ev[0], 0x05010400u);
-      const uint32_t qe = __builtin_amdgcn_perm(ev[3], ev[2], 0x05010400u);
-      const uint32_t po = __builtin_amdgcn_perm(od[1], od[0], 0x05010400u);
-      const uint32_t qo = __builtin_amdgcn_perm(od[3], od[2], 0x05010400u);
-      const uint32_t dg[4] = {__builtin_amdgcn_perm(qe, pe, 0x05040100u), __builtin_amdgcn_perm(qo, po, 0x05040100u),
-                              __builtin_amdgcn_perm(qe, pe, 0x07060302u), __builtin_amdgcn_perm(qo, po, 0x07060302u)};
-      const int t = 2 * sp_ + st;
-      if (t < QUADS) {
-        char* dst = xs_w + t * kDigQuad + stage_off;
+      if (st < QUADS) {
+        char* dst = xs_w + st * kDigQuad + stage_off;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(dst + d * 32) = dg[d];
+        for (int i = 0; i < 4; ++i) {
+          // digits of activations i and i + 4 side by side: bytes (d0, d0', d2, d2') and (d1, d1', d3, d3')
+          const uint32_t pe = __builtin_amdgcn_perm(ev[i + 4], ev[i], 0x05010400u);
+          const uint32_t po = __builtin_amdgcn_perm(od[i + 4], od[i], 0x05010400u);
+          *reinterpret_cast<uint16_t*>(dst + 0 * 32 + 8 * i) = (uint16_t)pe;
+          *reinterpret_cast<uint16_t*>(dst + 1 * 32 + 8 * i) = (uint16_t)po;
+          *reinterpret_cast<uint16_t*>(dst + 2 * 32 + 8 * i) = (uint16_t)(pe >> 16);
+          *reinterpret_cast<uint16_t*>(dst + 3 * 32 + 8 * i) = (uint16_t)(po >> 16);
+        }
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
