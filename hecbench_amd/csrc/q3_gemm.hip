@@ -54,7 +54,12 @@ __global__ __launch_bounds__(256) void q3_gemm_prep(const _Float16* __restrict__
                                                    int M, int K, int Mpad, int Gpad) {
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int G = K >> 5;
-  const int m = blockIdx.x;
+  // Eight consecutive rows share the 128-byte lines of Ap; workgroups b, b + 8, b + 16, ... run on the same
+  // XCD, so the rows of a line go to workgroups of one XCD and its L2 writes whole lines back instead of
+  // eight XCDs writing an eighth of every line each.
+  // (64 workgroups whatever Mpad; those beyond Mpad have nothing to do).
+  const int m = (blockIdx.x & 7) * 8 + (blockIdx.x >> 3);
+  if (m >= Mpad) return;
   __shared__ float s_sum[4], s_max[4];
   float sum = 0.f, amax = 0.f;
   if (m < M) {
@@ -309,7 +314,7 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
     const int MB = Mb > 32 ? 2 : 1;
     const int Mpad = 32 * MB;
     const _Float16* A = reinterpret_cast<const _Float16*>(x) + (size_t)m0 * K;
-    hipLaunchKernelGGL(q3_gemm_prep, dim3(Mpad), dim3(256), 0, stream, A, Ap, rowsum, rowinv, Mb, K, Mpad, Gpad);
+    hipLaunchKernelGGL(q3_gemm_prep, dim3(64), dim3(256), 0, stream, A, Ap, rowsum, rowinv, Mb, K, Mpad, Gpad);
     rc = hq_launch_status();
     if (rc != HQ_OK) return rc;
     GemmArgs a;
