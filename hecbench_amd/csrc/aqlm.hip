@@ -48,7 +48,12 @@ __device__ __forceinline__ float dot8(u4v e, u4v xv, float acc) {
 template <int ROWS>
 __global__ __launch_bounds__(256) void aqlm_matvec_kernel(AqlmArgs a) {
   const int lane = threadIdx.x & 63;
-  const int wave = (blockIdx.x * 256 + threadIdx.x) >> 6;
+  // Workgroups b, b + 8, b + 16, ... run on the same XCD; inside every 64 of them the row blocks are dealt
+  // out so that the eight workgroups whose results share a 128-byte line of y are on one XCD (its L2 then
+  // writes the line back whole instead of eight XCDs writing 16 bytes of it each).
+  const int b = blockIdx.x;
+  const int blk = b < (int)(gridDim.x & ~63u) ? ((b & ~63) | ((b & 7) << 3) | ((b >> 3) & 7)) : b;
+  const int wave = (blk * 256 + threadIdx.x) >> 6;
   const int row0 = wave * ROWS;
   if (row0 >= a.M) return;  // wave-uniform
   const int units_per_row = a.K >> 6;         // 16-byte code units (8 codes) per row; K % 64 == 0
