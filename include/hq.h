@@ -173,7 +173,8 @@ int hq_q3_matvec_noalloc(const void* x, int x_dtype, const int32_t* qweight, con
  *   s = +1 if bit (k%32) of bW[k/32][b][n] is set, else -1
  * Layouts (src/lut-gemm-hip/nQWeight_fp16.h:24-26): bW uint32[K/32][nbits][N],
  * alpha fp16[K/G][nbits][N], q_bias fp16[K/G][N] or NULL, x fp16[K], y fp16[N].
- * K % 32 == 0, G % 32 == 0, K % G == 0, 1 <= nbits <= 8; any N.
+ * K % 32 == 0, G % 32 == 0, K % G == 0, 1 <= nbits <= 8; any N.  x 16-byte aligned, bW 4-byte,
+ * alpha, q_bias and y 2-byte (16-byte aligned operands and N % 64 == 0 take the aligned loads).
  * Sums are kept in fp32 and rounded to fp16 once.  Replaces
  * matmul(output, input, nqW, m), src/lut-gemm-hip/kernels.cu:27-31.
  */
