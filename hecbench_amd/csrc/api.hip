@@ -122,7 +122,10 @@ extern "C" int hq_reserve_workspace(void* stream, int max_K, int max_N) {
   // eight splits (one per 4096 elements of K) whatever the tile count, beyond that only as many as give every
   // compute unit a workgroup (the LUT table kernel: two per compute unit, 128 floats each)
   const size_t kpad = ((size_t)max_K + 1023) / 1024 * 1024;
-  const size_t gemm_floats = kpad * 32 + 128;
+  // (plus, when the 128-column tiles do not fill the device, the raw sums of its K split: at most 256
+  // blocks of 64 x 128)
+  const size_t tiles128 = ((size_t)max_N + 127) / 128;
+  const size_t gemm_floats = kpad * 32 + 128 + (2 * tiles128 <= (size_t)d->cus ? (size_t)256 * 64 * 128 : 0);
   const size_t tiles = ((size_t)max_N + 63) / 64;
   const size_t rounds = ((size_t)max_K + 4095) / 4096;
   const size_t full_split = tiles * (rounds <= 8 ? rounds : 1);

@@ -51,6 +51,8 @@ struct HqQ3Scratch {
   float* rows;             // 128 floats: row sums and row scales of the batched GEMM
   unsigned* counters;      // split-K arrival counters (cleared by the call that uses them)
   size_t ncounters;
+  float* sums;             // raw sums of the batched GEMM's K split
+  size_t sums_floats;
 };
 int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const float* scales, const float* zeros,
                       float* y, int K, int N, int batch_M, unsigned flags, hipStream_t stream,

@@ -40,6 +40,7 @@ constexpr int kDeep = 3;        // steps of operands in flight ahead of the one 
 constexpr int kBufs = kDeep + 1;
 constexpr int kChunk = kStepGroups * kBufs;  // the pre-pass pads K to a multiple of this many k-groups
 constexpr int kTileN = 128;     // output columns per workgroup
+constexpr int kMaxSplitGroups = 256;  // workgroups of a K-split launch (tiles times splits)
 
 
 // ---- pre-pass: activations -> operand-slot order, scaled by P[m] * 2^-pos; row sums ------------
@@ -148,7 +149,9 @@ struct GemmArgs {
   const float* scales;
   const float* zeros;
   float* out;           // [M][N]
+  float* partial;       // K split: [tile][split][Mpad][128] raw sums of a workgroup
   int M, K, N, Gpad;
+  int nsplit, spp;      // workgroups per column tile, steps per workgroup (a multiple of kBufs)
   unsigned flags;
 };
 
@@ -166,7 +169,10 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int nl = lane & 31, kb = lane >> 5;
   const int G = a.K >> 5;
-  const int nsteps = a.Gpad / kStepGroups;  // a multiple of kBufs: Gpad is a multiple of 32 k-groups
+  // K split: workgroup (tile, split) takes steps t_begin .. t_begin + nsteps - 1 (both multiples of kBufs:
+  // Gpad is a multiple of 32 k-groups) and leaves its raw sums to hq_q3_gemm_reduce
+  const int t_begin = blockIdx.y * a.spp;
+  const int nsteps = min(a.spp, a.Gpad / kStepGroups - t_begin);
   const int col0 = blockIdx.x * kTileN;
   const int col = min(col0 + 4 * nl, a.N - 4);
   const size_t row_stride = (size_t)a.N;
@@ -195,7 +201,8 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
       for (int i = 0; i < 16; ++i) acc[mb][q][i] = 0.f;
 
   const u4v* ap_lane = a.Ap + (size_t)((2 * wv + kb) * 4) * Mpad + nl;
-  auto load_step = [&](int t, u4v (&A)[4][MB], uint32_t (&wr)[3][4]) {
+  auto load_step = [&](int tl, u4v (&A)[4][MB], uint32_t (&wr)[3][4]) {
+    const int t = t_begin + tl;
     const int g = min(t * kStepGroups + 2 * wv + kb, G - 1);  // padded groups: any valid weights, zero activations
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
@@ -261,7 +268,10 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
 #pragma unroll
       for (int w = 1; w < kWaves; ++w)
         v += *reinterpret_cast<const f4v*>(red + (size_t)w * REGION + r * kTileN + 4 * nl);
-      if (m < a.M && n_out < a.N) {
+      if (a.nsplit > 1) {
+        f4v* dst = reinterpret_cast<f4v*>(a.partial + (((size_t)blockIdx.x * a.nsplit + blockIdx.y) * Mpad + m) * kTileN) + nl;
+        __builtin_nontemporal_store(v, dst);
+      } else if (m < a.M && n_out < a.N) {
         f4v o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = sc[e] * (v[e] * ri[mb][j]) - zr[e] * rs[mb][j];
@@ -273,13 +283,40 @@ __global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
   }
 }
 
+// K split: sums the workgroups' raw sums of a tile in split order and applies scale, zero and the row's power
+// of two.  A thread owns four adjacent columns of one row.
+__global__ __launch_bounds__(256) void q3_gemm_reduce(GemmArgs a, int Mpad) {
+  const int tile = blockIdx.x;
+  const int nl = threadIdx.x & 31;
+  const int n_out = tile * kTileN + 4 * nl;
+  if (n_out >= a.N) return;
+  const f4v sc = *reinterpret_cast<const f4v*>(a.scales + n_out);
+  const f4v zr = *reinterpret_cast<const f4v*>(a.zeros + n_out);
+  for (int m = blockIdx.y * 8 + (threadIdx.x >> 5); m < a.M; m += gridDim.y * 8) {
+    const float* p = a.partial + (((size_t)tile * a.nsplit) * Mpad + m) * kTileN + 4 * nl;
+    f4v v = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < a.nsplit; ++s) v += __builtin_nontemporal_load(reinterpret_cast<const f4v*>(p + (size_t)s * Mpad * kTileN));
+    const float ri = a.rowinv[m] * 16777216.f, rs = a.rowsum[m];
+    f4v o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = sc[e] * (v[e] * ri) - zr[e] * rs;
+    f4v* dst = reinterpret_cast<f4v*>(a.out + (size_t)m * a.N + n_out);
+    if (a.flags & HQ_FLAG_ACCUMULATE) { const f4v old = *dst; o += old; }
+    *dst = o;
+  }
+}
+
 template <int MB>
 int launch_gemm(const GemmArgs& a, hipStream_t stream) {
   const size_t smem = (size_t)kWaves * 32 * kTileN * 4;
   static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_gemm_kernel<MB>),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (attr != hipSuccess) return (int)attr;
-  hipLaunchKernelGGL((q3_gemm_kernel<MB>), dim3((a.N + kTileN - 1) / kTileN), dim3(kWaves * 64), smem, stream, a);
+  const int ntiles = (a.N + kTileN - 1) / kTileN;
+  hipLaunchKernelGGL((q3_gemm_kernel<MB>), dim3(ntiles, a.nsplit), dim3(kWaves * 64), smem, stream, a);
+  int rc = hq_launch_status();
+  if (rc != HQ_OK || a.nsplit == 1) return rc;
+  hipLaunchKernelGGL(q3_gemm_reduce, dim3(ntiles, (a.M + 7) / 8 < 8 ? (a.M + 7) / 8 : 8), dim3(256), 0, stream, a, 32 * MB);
   return hq_launch_status();
 }
 
@@ -292,22 +329,39 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
   const int G = K / 32;
   const int Gpad = (G + kChunk - 1) / kChunk * kChunk;
   const size_t ap_halves = (size_t)Gpad * 4 * 64 * 8;
+  // K split: column tiles alone leave most CUs idle when N is small (N = 4096: 32 tiles), so K is cut into as
+  // many ranges as give every CU a workgroup (at most kMaxSplitGroups of them, which is what the fixed
+  // scratch of the entry point that allocates nothing holds), each range a multiple of kBufs steps; the
+  // workgroups leave raw sums in the workspace and a second kernel adds them in split order (deterministic).
+  const HqDevice* dev = nullptr;
+  int rc = hq_current_device(&dev);
+  if (rc != HQ_OK) return rc;
+  const int ntiles = (N + kTileN - 1) / kTileN;
+  const int nsteps = Gpad / kStepGroups;
+  int nsplit = (dev->cus < kMaxSplitGroups ? dev->cus : kMaxSplitGroups) / ntiles;
+  if (nsplit > nsteps / kBufs) nsplit = nsteps / kBufs;
+  if (nsplit < 1) nsplit = 1;
+  int spp = (nsteps + nsplit - 1) / nsplit;
+  spp = (spp + kBufs - 1) / kBufs * kBufs;
+  nsplit = (nsteps + spp - 1) / spp;
+  const size_t partial_floats = nsplit > 1 ? (size_t)ntiles * nsplit * 64 * kTileN : 0;
   _Float16* Ap;
-  float *rowsum, *rowinv;
+  float *rowsum, *rowinv, *partial = nullptr;
   if (fixed) {
-    if (ap_halves / 2 > fixed->partial_floats) return HQ_ERR_TOO_LARGE;
+    if (ap_halves / 2 > fixed->partial_floats || partial_floats > fixed->sums_floats) return HQ_ERR_TOO_LARGE;
     Ap = reinterpret_cast<_Float16*>(fixed->partial);
     rowsum = fixed->rows;
     rowinv = fixed->rows + 64;
+    partial = fixed->sums;
   } else {
     HqWorkspace ws;
-    int rc = hq_get_workspace(stream, ap_halves / 2 + 128, 1, &ws);
+    rc = hq_get_workspace(stream, ap_halves / 2 + 128 + partial_floats, 1, &ws);
     if (rc != HQ_OK) return rc;
     Ap = reinterpret_cast<_Float16*>(ws.partial);
     rowsum = ws.partial + ap_halves / 2;
     rowinv = rowsum + 64;
+    partial = rowsum + 128;
   }
-  int rc = HQ_OK;
   // up to 64 rows per pass over the weights
   for (int m0 = 0; m0 < M; m0 += 64) {
     const int Mb = M - m0 < 64 ? M - m0 : 64;
@@ -326,6 +380,7 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
     a.zeros = zeros;
     a.out = y + (size_t)m0 * N;
     a.M = Mb; a.K = K; a.N = N; a.Gpad = Gpad; a.flags = flags;
+    a.partial = partial; a.nsplit = nsplit; a.spp = spp;
     rc = MB == 2 ? launch_gemm<2>(a, stream) : launch_gemm<1>(a, stream);
     if (rc != HQ_OK) return rc;
   }
@@ -334,13 +389,14 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
 
 // ---- the entry point that allocates nothing ----------------------------------------------------
 // Its scratch (split-K partial sums and arrival counters of the matvec, re-ordered activations, row
-// sums and row scales of the batched GEMM) lives in a fixed device array instead of the stream's
+// sums, row scales and K-split sums of the batched GEMM) lives in a fixed device array instead of the stream's
 // workspace.  Every GPU holds its own copy of the array at its own address, resolved once per device.
 namespace {
 constexpr size_t kScratchPartialBytes = (size_t)2 << 20;  // 2 MiB: K <= 16384 batched, 8192 partial rows of 64 floats
 constexpr size_t kScratchRowBytes = 1024;                 // 128 floats used
 constexpr size_t kScratchCounterBytes = 64 * 1024 - kScratchRowBytes;
-constexpr size_t kScratchBytes = kScratchPartialBytes + kScratchRowBytes + kScratchCounterBytes;
+constexpr size_t kScratchSumBytes = (size_t)kMaxSplitGroups * 64 * kTileN * sizeof(float);  // 8 MiB: the GEMM's K split
+constexpr size_t kScratchBytes = kScratchPartialBytes + kScratchRowBytes + kScratchCounterBytes + kScratchSumBytes;
 }  // namespace
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
@@ -383,5 +439,7 @@ extern "C" int hq_q3_matvec_noalloc(const void* x, int x_dtype, const int32_t* q
   s.rows = reinterpret_cast<float*>(b + kScratchPartialBytes);
   s.counters = reinterpret_cast<unsigned*>(b + kScratchPartialBytes + kScratchRowBytes);
   s.ncounters = kScratchCounterBytes / sizeof(unsigned);
+  s.sums = reinterpret_cast<float*>(b + kScratchPartialBytes + kScratchRowBytes + kScratchCounterBytes);
+  s.sums_floats = kScratchSumBytes / sizeof(float);
   return hq_q3_matvec_impl(x, x_dtype, qweight, scales, zeros, y, K, N, batch_M, flags, (hipStream_t)stream, &s);
 }

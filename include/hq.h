@@ -154,7 +154,7 @@ int hq_q3_matvec_plan(int K, int N, int batch_M);
  * hq_q3_matvec for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): same arguments, same kernels and bit-identical results, but the
  * scratch the kernels need (split-K partial sums and arrival counters of the matvec, the batched
- * path's re-ordered activations, row sums and row scales) is a fixed 2 MiB + 64 KiB array in device
+ * path's re-ordered activations, row sums, row scales and K-split sums) is a fixed 10 MiB + 64 KiB array in device
  * memory that each GPU holds from library load to process end, instead of the stream's workspace.
  * The call runs no hipMalloc, hipFree or allocating library routine.  Limits: batch_M > 1 needs
  * K <= 16384; a split-K matvec needs tiles * splits <= 8192 and N <= 1032192 (never exceeded while

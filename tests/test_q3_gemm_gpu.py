@@ -35,6 +35,20 @@ def test_small_shapes_vs_oracle(hq, oracle, M, K, N, seed):
     assert rel_err(y, exact, FLOOR_F16) <= 1e-4
 
 
+@pytest.mark.parametrize("M,K,N,seed", [(16, 4096, 512, 11), (64, 8192, 260, 12), (40, 14336, 1024, 13), (3, 2048, 128, 14),
+                                        (100, 4096, 4096, 15)])
+def test_small_n_splits_k(hq, oracle, M, K, N, seed):
+    """Few column tiles: K is cut into ranges (one workgroup each) whose raw sums a second kernel adds up."""
+    codes, scales, zeros, A = oa.make_q3_problem(seed, K, N, x_dtype=np.float16, batch=M)
+    mat = oracle.q3_pack(codes)
+    y = _run(hq, A, mat, scales, zeros)
+    assert np.array_equal(y, _run(hq, A, mat, scales, zeros))      # the sums are added in a fixed order
+    cols = np.unique(np.concatenate([np.arange(0, min(N, 130)), np.arange(max(0, N - 130), N)]))
+    exact = oracle.q3_gemm(A, np.ascontiguousarray(mat[:, cols]), scales[cols], zeros[cols], mode=0)
+    assert rel_err(y[:, cols], exact) <= 5e-3
+    assert rel_err(y[:, cols], exact, FLOOR_F16) <= 1e-4
+
+
 @pytest.mark.parametrize("scale_exp", [-16, -12, -8, 0, 4])
 def test_dynamic_range(hq, oracle, scale_exp):
     """Accuracy must not depend on the magnitude of the activations: whole problem scaled by a power of
