@@ -118,9 +118,10 @@ extern "C" int hq_reserve_workspace(void* stream, int max_K, int max_N) {
   int rc = hq_current_device(&d);
   if (rc != HQ_OK) return rc;
   // batched GEMM: re-ordered activations of 64 rows (128 bytes per input feature, K padded to 1024) plus
-  // the row sums and scales; split-K matvecs: a partial row of 64 floats per column tile and split - up to
-  // eight splits (one per 4096 elements of K) whatever the tile count, beyond that only as many as give every
-  // compute unit a workgroup (the LUT table kernel: two per compute unit, 128 floats each)
+  // the row sums and scales; split-K matvecs: a partial row of 64 floats per column tile and split (two rows
+  // for a batch of 2) - up to eight splits (one per 4096 elements of K) whatever the tile count, beyond that
+  // only as many as give every compute unit a workgroup (the LUT table kernel: two per compute unit, 128
+  // floats each)
   const size_t kpad = ((size_t)max_K + 1023) / 1024 * 1024;
   // (plus, when the 128-column tiles do not fill the device, the raw sums of its K split: at most 256
   // blocks of 64 x 128)

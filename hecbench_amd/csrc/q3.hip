@@ -426,7 +426,9 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
                       float* y, int K, int N, int M, unsigned flags, hipStream_t stream, const HqQ3Scratch* fixed);
 
 int hq_q3_rows_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                      int K, int N, unsigned flags, hipStream_t stream);
+                      int K, int N, int gpw, int nsplit, float* partial, unsigned* counters, unsigned flags,
+                      hipStream_t stream);
+int hq_q3_rows_groups_per_round(void);
 
 namespace {
 // Zeroes n words with a kernel (a memset node inside a captured graph is not an option for callers
@@ -439,10 +441,60 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(unsigned* p, int n) {
 
 namespace {
 int q3_plan(const HqDevice* dev, int N, int batch_M) {
+  (void)dev; (void)N;
   if (batch_M == 1) return HQ_Q3_PLAN_MATVEC;
-  if (batch_M == 2 && 2 * ((N + 63) / 64) >= dev->cus && hq_tune(HQ_TUNE_Q3_SMALL_BATCH, 1) != 0)
-    return HQ_Q3_PLAN_ROWS;
+  if (batch_M == 2 && hq_tune(HQ_TUNE_Q3_SMALL_BATCH, 1) != 0) return HQ_Q3_PLAN_ROWS;
   return HQ_Q3_PLAN_GEMM;
+}
+
+// How the digit kernels (batch 1 and batch 2) divide K: a workgroup covers gpr k-groups per round and walks
+// its K range in rounds (the next round's loads are in flight during the current one), or K is split across
+// workgroups whose partial sums (rows_out rows of 64 floats per workgroup) the last one to arrive adds up.
+struct Q3Split {
+  int gpw;     // k-groups per workgroup, whole rounds
+  int nsplit;  // workgroups per column tile
+  float* partial;
+  unsigned* counters;
+};
+int q3_split_k(const HqDevice* dev, int G, int gpr, int ntiles, int rows_out, const HqQ3Scratch* fixed,
+               hipStream_t stream, Q3Split* out) {
+  const int max_split = (G + gpr - 1) / gpr;
+  const size_t tile_floats = (size_t)ntiles * rows_out * 64;
+  int nsplit = hq_tune(HQ_TUNE_Q3_KSPLIT, 0);
+  if (nsplit <= 0) {
+    // Up to eight rounds of K: one workgroup per round.  Single-round workgroups need half the registers,
+    // so two share a CU and one's reduction tail runs under the other's loads, and 2-8 times as many
+    // workgroups spread evenly over the CUs whatever the tile count (batch 1 at K=8192: N=22016, 344 tiles,
+    // 20.4 -> 15.1 us; N=28672, 448 tiles, 21.4 -> 18.6 us; K=28672, N=8192 21.7 -> 19.6 us).  Longer K: only
+    // as many splits as it takes to give every CU a workgroup - each split adds a partial-sum row per tile
+    // and a device-scope round trip (K=49152, N=12288: 43 us unsplit, 51-58 us split).
+    nsplit = max_split <= 8 ? max_split : dev->cus / ntiles;
+    if (fixed && nsplit > 1 && (tile_floats * nsplit > fixed->partial_floats || (size_t)ntiles > fixed->ncounters))
+      nsplit = dev->cus / ntiles;  // the fixed scratch is too small for the full split
+  }
+  if (nsplit > max_split) nsplit = max_split;
+  if (nsplit < 1) nsplit = 1;
+  int gpw = (G + nsplit - 1) / nsplit;
+  gpw = (gpw + gpr - 1) / gpr * gpr;  // whole rounds
+  nsplit = (G + gpw - 1) / gpw;
+  out->gpw = gpw; out->nsplit = nsplit; out->partial = nullptr; out->counters = nullptr;
+  if (nsplit > 1 && fixed) {
+    // fixed scratch shared by every call on this device: the counters start from zero by a fill kernel
+    // on the same stream (they also reset themselves, but an earlier call may have been cut short)
+    if (tile_floats * nsplit > fixed->partial_floats || (size_t)ntiles > fixed->ncounters) return HQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((ntiles + 255) / 256), dim3(256), 0, stream, fixed->counters, ntiles);
+    const int rc = hq_launch_status();
+    if (rc != HQ_OK) return rc;
+    out->partial = fixed->partial;
+    out->counters = fixed->counters;
+  } else if (nsplit > 1) {
+    HqWorkspace ws;
+    const int rc = hq_get_workspace(stream, tile_floats * nsplit, (size_t)ntiles, &ws);
+    if (rc != HQ_OK) return rc;
+    out->partial = ws.partial;
+    out->counters = ws.counters;
+  }
+  return HQ_OK;
 }
 }  // namespace
 
@@ -475,10 +527,15 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   if (rc != HQ_OK) return rc;
   if (batch_M > 1) {
     if (x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
-    // A batch of 2 rides on the matvec's digit kernel (one pass over the weights, no workspace) when the
-    // column tiles alone give at least every other CU a workgroup; everything else takes the batched GEMM.
-    if (q3_plan(dev, N, batch_M) == HQ_Q3_PLAN_ROWS)
-      return hq_q3_rows_launch(x, qweight, scales, zeros, y, K, N, flags, stream);
+    // A batch of 2 rides on the matvec's digit kernel (one pass over the weights, one launch); everything
+    // else takes the batched GEMM.
+    if (q3_plan(dev, N, batch_M) == HQ_Q3_PLAN_ROWS) {
+      Q3Split sp;
+      rc = q3_split_k(dev, K / 32, hq_q3_rows_groups_per_round(), (N + 63) / 64, 2, fixed, stream, &sp);
+      if (rc != HQ_OK) return rc;
+      return hq_q3_rows_launch(x, qweight, scales, zeros, y, K, N, sp.gpw, sp.nsplit, sp.partial, sp.counters, flags,
+                               stream);
+    }
     return hq_q3_gemm_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream, fixed);
   }
 
@@ -496,47 +553,14 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
     while (steps > 1 && waves * 4 * (steps / 2) >= G) steps /= 2;  // short K: fewer steps
   }
   const int gpr = waves * 4 * steps;  // k-groups one workgroup covers per round
-  const int max_split = (G + gpr - 1) / gpr;
-  int nsplit = hq_tune(HQ_TUNE_Q3_KSPLIT, 0);
-  if (nsplit <= 0) {
-    // Up to eight rounds of K: one workgroup per round.  Single-round workgroups need half the registers,
-    // so two share a CU and one's reduction tail runs under the other's loads, and 2-8 times as many
-    // workgroups spread evenly over the CUs whatever the tile count (at K=8192: N=22016, 344 tiles, 20.4 ->
-    // 15.1 us; N=28672, 448 tiles, 21.4 -> 18.6 us; K=28672, N=8192 21.7 -> 19.6 us).  Longer K: only as
-    // many splits as it takes to give every CU a workgroup - each split adds a partial-sum row per tile
-    // and a device-scope round trip (K=49152, N=12288: 43 us unsplit, 51-58 us split).
-    nsplit = max_split <= 8 ? max_split : dev->cus / ntiles;
-    if (fixed && nsplit > 1 &&
-        ((size_t)ntiles * nsplit * 64 > fixed->partial_floats || (size_t)ntiles > fixed->ncounters))
-      nsplit = dev->cus / ntiles;  // the fixed scratch is too small for the full split
-  }
-  if (nsplit > max_split) nsplit = max_split;
-  if (nsplit < 1) nsplit = 1;
-  int gpw = (G + nsplit - 1) / nsplit;
-  gpw = (gpw + gpr - 1) / gpr * gpr;  // whole rounds
-  nsplit = (G + gpw - 1) / gpw;
+  Q3Split sp;
+  rc = q3_split_k(dev, G, gpr, ntiles, 1, fixed, stream, &sp);
+  if (rc != HQ_OK) return rc;
 
   Q3Args a;
   a.x = x; a.w = reinterpret_cast<const uint32_t*>(qweight); a.scales = scales; a.zeros = zeros;
-  a.y = y; a.partial = nullptr; a.counters = nullptr; a.K = K; a.N = N; a.gpw = gpw;
-  a.nsplit = nsplit; a.x_f16 = (x_dtype == HQ_DTYPE_F16); a.flags = flags;
-  if (nsplit > 1 && fixed) {
-    // fixed scratch shared by every call on this device: the counters start from zero by a fill kernel
-    // on the same stream (they also reset themselves, but an earlier call may have been cut short)
-    if ((size_t)ntiles * nsplit * 64 > fixed->partial_floats || (size_t)ntiles > fixed->ncounters)
-      return HQ_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((ntiles + 255) / 256), dim3(256), 0, stream, fixed->counters, ntiles);
-    rc = hq_launch_status();
-    if (rc != HQ_OK) return rc;
-    a.partial = fixed->partial;
-    a.counters = fixed->counters;
-  } else if (nsplit > 1) {
-    HqWorkspace ws;
-    rc = hq_get_workspace(stream, (size_t)ntiles * nsplit * 64, (size_t)ntiles, &ws);
-    if (rc != HQ_OK) return rc;
-    a.partial = ws.partial;
-    a.counters = ws.counters;
-  }
+  a.y = y; a.partial = sp.partial; a.counters = sp.counters; a.K = K; a.N = N; a.gpw = sp.gpw;
+  a.nsplit = sp.nsplit; a.x_f16 = (x_dtype == HQ_DTYPE_F16); a.flags = flags;
 #define HQ_Q3_CASE(W, S) \
   if (waves == W && steps == S) return launch_matvec<W, S>(a, ntiles, stream);
   HQ_Q3_CASE(16, 1)

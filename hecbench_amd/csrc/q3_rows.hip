@@ -28,7 +28,11 @@ struct RowsArgs {
   const float* scales;
   const float* zeros;
   float* y;           // [rows][N]
+  float* partial;     // [tile][split][rows][64] when K is split
+  unsigned* counters; // [tile] arrival counters, zero between calls
   int K, N;
+  int gpw;            // k-groups per workgroup
+  int nsplit;         // workgroups per column tile
   unsigned flags;
 };
 
@@ -77,25 +81,32 @@ __device__ __forceinline__ void transpose4(uint32_t a, uint32_t b, uint32_t c, u
 
 constexpr int kDigits = 7;          // 4-bit digits per activation: 28-bit fixed point
 constexpr int kRowBytes = 144;      // one B operand row (4 lane quarters x 32 B) plus 16 B: rows start 4 banks apart
-constexpr int kStepBytes = 2560;    // fourteen digit rows and a row of zeros per step, padded
+constexpr int kStepBytes = 2176;    // fourteen digit rows per step plus room for the step's skew
+constexpr int kZeroBytes = 128;     // a wave's row of zeros (4 lane quarters x 32 B) behind its steps
 constexpr int kRedStride = 68;      // floats per digit column of a wave's final sums
 __device__ __forceinline__ constexpr int step_off(int s) {
   return s * kStepBytes + (s & 1) * 32 + ((s >> 1) & 1) * 128;
 }
 
-template <int WAVES, int STEPS, int ROWS>
+// MULTI: the workgroup walks its K range in rounds, the next round's loads in flight during the current
+// one.  Otherwise its range is one round, it needs half the registers and less than half the LDS of a CU,
+// and two workgroups share a CU.
+template <int WAVES, int STEPS, int ROWS, bool MULTI>
 __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
-  // LDS: dig[WAVES][STEPS * kStepBytes] (a wave's final sums re-use its area) | part[WAVES][ROWS][64] | wsum[WAVES][ROWS]
+  // LDS: dig[WAVES][STEPS * kStepBytes + kZeroBytes] (a wave's final sums re-use its area) | part[WAVES][ROWS][64] |
+  // wsum[WAVES][ROWS]
   extern __shared__ uint4 smem[];
+  constexpr int kWaveBytes = STEPS * kStepBytes + kZeroBytes;
   char* dig = reinterpret_cast<char*>(smem);
-  float* part = reinterpret_cast<float*>(dig + WAVES * STEPS * kStepBytes);
+  float* part = reinterpret_cast<float*>(dig + WAVES * kWaveBytes);
   float* wsum = part + WAVES * ROWS * 64;
   static_assert(STEPS * kStepBytes >= 14 * kRedStride * 4, "a wave's digit area must hold its final sums");
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int c = lane & 15, kb = lane >> 4;
-  const int tile = blockIdx.x;
-  const int G = a.K >> 5;
+  const int tile = blockIdx.x, split = blockIdx.y;
+  const int g_begin = split * a.gpw;
+  const int G = min(a.gpw, (a.K >> 5) - g_begin);  // k-groups of this workgroup
   const int ncol = tile * 64 + (tid & 63);
 
   float sc_n = 0.f, zr_n = 0.f, y_old = 0.f;
@@ -103,7 +114,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
     const int nc = min(ncol, a.N - 1);
     sc_n = a.scales[nc];
     zr_n = a.zeros[nc];
-    y_old = (a.flags & HQ_FLAG_ACCUMULATE) ? a.y[(size_t)(tid >> 6) * a.N + nc] : 0.f;
+    y_old = ((a.flags & HQ_FLAG_ACCUMULATE) && a.nsplit == 1) ? a.y[(size_t)(tid >> 6) * a.N + nc] : 0.f;
   }
   // staging role: lane converts the eight consecutive activations 8*xq .. 8*xq+7 of k-group xkb of step 4*pass + xs
   const int xs = lane >> 4, xkb = (lane >> 2) & 3, xq = lane & 3;
@@ -111,9 +122,10 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
   const int tile_cols = min(64, a.N - tile * 64);  // multiple of 4
   const uint32_t col_off = (uint32_t)min(4 * c, tile_cols - 4) * 4u;
   const uint32_t row_bytes = (uint32_t)a.N * 4u;
-  const char* wbase = reinterpret_cast<const char*>(a.w) + (size_t)tile * 64 * 4;
+  const char* wbase = reinterpret_cast<const char*>(a.w) + (size_t)g_begin * 3 * row_bytes + (size_t)tile * 64 * 4;
+  const _Float16* xbase = a.x + (size_t)g_begin * 32;
   constexpr int GPR = WAVES * 4 * STEPS;  // k-groups per round
-  const int rounds = (G + GPR - 1) / GPR;
+  const int rounds = MULTI ? (G + GPR - 1) / GPR : 1;  // !MULTI: the host sized gpw <= GPR
 
   auto load_round = [&](int r, u4v (&xraw)[ROWS][XP], uint32_t (&wreg)[STEPS][3][4]) {
 #pragma unroll
@@ -122,7 +134,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
       for (int p = 0; p < XP; ++p) {
         const int s = min(4 * p + xs, STEPS - 1);
         const uint32_t g = (uint32_t)min((r * STEPS + s) * (WAVES * 4) + wv * 4 + xkb, G - 1);
-        xraw[m][p] = *reinterpret_cast<const u4v*>(a.x + (size_t)m * a.K + g * 32u + (uint32_t)xq * 8u);
+        xraw[m][p] = *reinterpret_cast<const u4v*>(xbase + (size_t)m * a.K + g * 32u + (uint32_t)xq * 8u);
       }
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
@@ -136,15 +148,13 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
     }
   };
 
-  char* dig_w = dig + wv * (STEPS * kStepBytes);
-  // Row 14 of every step stays zero: MFMA column c reads row c while it carries a digit (c < 7 ROWS) and the
-  // zero row otherwise.
-  static_assert(kDigits * ROWS <= 14, "the digit rows and the zero row must fit the sixteen operand rows");
-  if (lane < 32) {
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) *reinterpret_cast<uint32_t*>(dig_w + step_off(s) + 14 * kRowBytes + lane * 4) = 0u;
-  }
-  const int rowsel = c < kDigits * ROWS ? c : 14;
+  char* dig_w = dig + wv * kWaveBytes;
+  // MFMA column c reads digit row c of the step while it carries a digit (c < 7 ROWS) and the wave's row of
+  // zeros otherwise.
+  static_assert(kDigits * ROWS <= 14, "a step holds fourteen digit rows");
+  if (lane < kZeroBytes / 4) *reinterpret_cast<uint32_t*>(dig_w + STEPS * kStepBytes + lane * 4) = 0u;
+  const bool digit_col = c < kDigits * ROWS;
+  const int b_off = digit_col ? c * kRowBytes + kb * 32 : STEPS * kStepBytes + kb * 32;
   const int my_row = min(c / kDigits, ROWS - 1);  // the activation row whose digit this lane's MFMA column carries
 
   float run[4][4];
@@ -163,7 +173,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
   for (int r = 0; r < rounds; ++r) {
     u4v xraw_next[ROWS][XP];
     uint32_t wreg_next[STEPS][3][4];
-    if (r + 1 < rounds) load_round(r + 1, xraw_next, wreg_next);  // in flight during this round
+    if (MULTI && r + 1 < rounds) load_round(r + 1, xraw_next, wreg_next);  // in flight during this round
 
     // ---- stage this wave's digits, one activation row after the other ----------------------------
     float descale_lane = 0.f;
@@ -231,7 +241,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       if ((r * STEPS + s) * (WAVES * 4) + wv * 4 >= G) continue;  // wave-uniform
-      const u4v* bp = reinterpret_cast<const u4v*>(dig_w + step_off(s) + rowsel * kRowBytes + kb * 32);
+      const u4v* bp = reinterpret_cast<const u4v*>(dig_w + (digit_col ? step_off(s) + b_off : b_off));
       const u4v b0 = bp[0], b1 = bp[1];
       const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
 #pragma unroll
@@ -251,7 +261,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
       for (int i = 0; i < 4; ++i) run[q][i] = fmaf(acc[q][i], descale_lane, run[q][i]);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
-    if (r + 1 < rounds) {
+    if (MULTI && r + 1 < rounds) {
 #pragma unroll
       for (int m = 0; m < ROWS; ++m)
 #pragma unroll
@@ -301,30 +311,71 @@ __global__ __launch_bounds__(WAVES * 64) void q3_rows_kernel(RowsArgs a) {
     }
     float val = sc_n * (qx * 4096.f) - zr_n * xsum;  // 2^12: fp6 unit 2^-3 times fp8 unit 2^-9
     val = fmaf(xsum, 0.f, val);  // a NaN or infinity among the activations makes the result NaN
-    __hip_atomic_store(&a.y[(size_t)m * a.N + ncol], y_old + val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (a.nsplit == 1)
+      __hip_atomic_store(&a.y[(size_t)m * a.N + ncol], y_old + val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+      __hip_atomic_store(&a.partial[(((size_t)tile * a.nsplit + split) * ROWS + m) * 64 + col], val, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (a.nsplit > 1) {
+    // Arrival counting as in q3.hip: write-through partial sums, every wave waits for their acknowledgement,
+    // a barrier, one device-scope fetch-add per workgroup, and the last workgroup to arrive adds the partial
+    // sums in split order with loads that bypass the non-coherent cache levels.
+    __shared__ unsigned s_last;
+    const bool strict = (a.flags & HQ_FLAG_STRICT_FENCES) != 0;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) {
+      const unsigned old = strict ? __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT)
+                                  : __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (old == (unsigned)(a.nsplit - 1));
+    }
+    __syncthreads();
+    if (s_last && strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (s_last) {
+      if (tid < 64 * ROWS && ncol < a.N) {
+        const int m = tid >> 6, col = tid & 63;
+        float sum = 0.f;
+        for (int s = 0; s < a.nsplit; ++s)
+          sum += __hip_atomic_load(&a.partial[(((size_t)tile * a.nsplit + s) * ROWS + m) * 64 + col], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        float* yp = &a.y[(size_t)m * a.N + ncol];
+        *yp = (a.flags & HQ_FLAG_ACCUMULATE) ? *yp + sum : sum;
+      }
+      if (tid == 0)  // ready for the next call
+        __hip_atomic_store(&a.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
 }
 
-template <int ROWS>
-int launch_rows(const RowsArgs& a, hipStream_t stream) {
+template <int ROWS, bool MULTI>
+int launch_rows_t(const RowsArgs& a, hipStream_t stream) {
   constexpr int WAVES = 8, STEPS = 4;
-  const size_t smem = (size_t)WAVES * STEPS * kStepBytes + (size_t)WAVES * ROWS * 64 * 4 + (size_t)WAVES * ROWS * 4 + 16;
+  const size_t smem = (size_t)WAVES * (STEPS * kStepBytes + kZeroBytes) + (size_t)WAVES * ROWS * 64 * 4 +
+                      (size_t)WAVES * ROWS * 4 + 16;
   static const hipError_t attr =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_rows_kernel<WAVES, STEPS, ROWS>),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_rows_kernel<WAVES, STEPS, ROWS, MULTI>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
   if (attr != hipSuccess) return (int)attr;
-  hipLaunchKernelGGL((q3_rows_kernel<WAVES, STEPS, ROWS>), dim3((a.N + 63) / 64), dim3(WAVES * 64), smem, stream, a);
+  hipLaunchKernelGGL((q3_rows_kernel<WAVES, STEPS, ROWS, MULTI>), dim3((a.N + 63) / 64, a.nsplit), dim3(WAVES * 64), smem,
+                     stream, a);
   return hq_launch_status();
 }
 
 }  // namespace
 
-// Two fp16 activation rows; the caller has validated the arguments.
+// k-groups one workgroup of the two-row kernel covers per round
+int hq_q3_rows_groups_per_round(void) { return 8 * 4 * 4; }
+
+// Two fp16 activation rows; the caller has validated the arguments, sized gpw to whole rounds and, for
+// nsplit > 1, provided nsplit * 128 floats of partial sums and one zeroed counter per column tile.
 int hq_q3_rows_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                      int K, int N, unsigned flags, hipStream_t stream) {
+                      int K, int N, int gpw, int nsplit, float* partial, unsigned* counters, unsigned flags,
+                      hipStream_t stream) {
   RowsArgs a;
   a.x = reinterpret_cast<const _Float16*>(x);
   a.w = reinterpret_cast<const uint32_t*>(qweight);
-  a.scales = scales; a.zeros = zeros; a.y = y; a.K = K; a.N = N; a.flags = flags & HQ_FLAG_ACCUMULATE;
-  return launch_rows<2>(a, stream);
+  a.scales = scales; a.zeros = zeros; a.y = y; a.partial = partial; a.counters = counters; a.K = K; a.N = N;
+  a.gpw = gpw; a.nsplit = nsplit; a.flags = flags & (HQ_FLAG_ACCUMULATE | HQ_FLAG_STRICT_FENCES);
+  return gpw > hq_q3_rows_groups_per_round() ? launch_rows_t<2, true>(a, stream) : launch_rows_t<2, false>(a, stream);
 }

@@ -131,8 +131,8 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  * batch_M == 1 replaces vecquant3matmul / vecquant3matmul_faster
  * (src/quant3MatMul-hip/kernels.h:171-217) — pass HQ_FLAG_ACCUMULATE for their
  * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 (no counterpart in the
- * reference): a batch of 2 with at least one 64-column tile per two compute units
- * runs on the matvec's kernel with the two rows side by side in the matrix-core
+ * reference): a batch of 2 runs on the matvec's kernel (at about the cost of
+ * batch 1) with the two rows side by side in the matrix-core
  * operand (28-bit fixed point relative to the largest magnitude among each 512
  * consecutive activations of a row: exact for fp16 entries within 2^17 of it);
  * all other batches run the MFMA GEMM path.
@@ -153,12 +153,13 @@ int hq_q3_matvec_plan(int K, int N, int batch_M);
 /*
  * hq_q3_matvec for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): same arguments, same kernels and bit-identical results, but the
- * scratch the kernels need (split-K partial sums and arrival counters of the matvec, the batched
+ * scratch the kernels need (split-K partial sums and arrival counters of batches 1 and 2, the batched
  * path's re-ordered activations, row sums, row scales and K-split sums) is a fixed 10 MiB + 64 KiB array in device
  * memory that each GPU holds from library load to process end, instead of the stream's workspace.
- * The call runs no hipMalloc, hipFree or allocating library routine.  Limits: batch_M > 1 needs
- * K <= 16384; a split-K matvec needs tiles * splits <= 8192 and N <= 1032192 (never exceeded while
- * the device has at most 8192 compute units); beyond them HQ_ERR_TOO_LARGE.  All calls on one GPU
+ * The call runs no hipMalloc, hipFree or allocating library routine.  Limits: batch_M > 2 needs
+ * K <= 16384; a split-K matvec needs tiles * splits * batch_M <= 8192 (the one-per-round split falls
+ * back to one workgroup per compute unit where it would not fit) and N <= 1032192; beyond them
+ * HQ_ERR_TOO_LARGE.  All calls on one GPU
  * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race;
  * issue them on one stream or order them with events.  Call hq_init() once per device beforehand,
  * outside any capture (it resolves the array's address).  No counterpart in the reference.

@@ -1,6 +1,6 @@
-"""Batches 2 ... 15 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): a batch of 2 on a wide
-matrix runs on the matvec's digit kernel with the two rows side by side in the matrix-core operand,
-all others on the batched GEMM.  Every batch size is checked against the CPU oracle through the C ABI,
+"""Batches 2 ... 15 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): a batch of 2 runs on the
+matvec's digit kernel with the two rows side by side in the matrix-core operand (K split across workgroups
+as for batch 1), all others on the batched GEMM.  Every batch size is checked against the CPU oracle through the C ABI,
 and the kernel that ran is asserted through hq_q3_matvec_plan.  The reference has no batched kernel:
 the oracle is the matvec formula applied row by row (parity unpinned by the reference)."""
 import numpy as np
@@ -37,8 +37,8 @@ def _check(y, exact):
         assert rel_err(y[m], exact[m], FLOOR_F16) <= 1e-4, m
 
 
-# wide: at least one 64-column tile per two compute units (N = 257 tiles, the last one 4 columns wide);
-# narrow: too few tiles, every batch takes the GEMM; K = 4128 is not a multiple of a workgroup's round
+# wide (N = 257 tiles, the last one 4 columns wide) and narrow (3 tiles, the last one 4 columns wide);
+# K = 4128 is not a multiple of a workgroup's round, so the two-row kernel splits it in two;
 # the long-K shape is there for the two-row kernel and its neighbours only
 _EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)] for M in range(2, 16)
                 if K != 4128 or M <= 4]
@@ -48,7 +48,7 @@ _EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)
 def test_every_batch_vs_oracle(hq, oracle, M, K, N):
     codes, scales, zeros, A = oa.make_q3_problem(1000 + 16 * M + (K % 7), K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
-    want_plan = PLAN_ROWS if (M == 2 and N > 8000) else PLAN_GEMM
+    want_plan = PLAN_ROWS if M == 2 else PLAN_GEMM
     assert _plan(K, N, M) == want_plan
     y = _run(hq, A, mat, scales, zeros)
     _check(y, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
@@ -167,3 +167,49 @@ def test_rows_kernel_short_k(hq, oracle, K):
     mat = oracle.q3_pack(codes)
     assert _plan(K, N, 2) == PLAN_ROWS
     _check(_run(hq, A, mat, scales, zeros), oracle.q3_gemm(A, mat, scales, zeros, mode=0))
+
+
+# (K, N, forced split or 0): K rounds of 4096 -> one workgroup per round up to eight (three for K = 11008,
+# the last one partly filled), beyond that as many workgroups per tile as the compute units allow, each
+# walking several rounds (K = 36864, 64 tiles); a forced single workgroup walks all of K in rounds
+_SPLIT_SHAPES = [(11008, 4096, 0), (36864, 4096, 0), (40960, 1028, 0), (11008, 4096, 1), (8192, 260, 2)]
+
+
+@pytest.mark.parametrize("K,N,force", _SPLIT_SHAPES)
+def test_rows_kernel_splits_k(hq, oracle, tunable, K, N, force):
+    """Partial sums of both rows per workgroup, added by the last one to arrive: same result as the
+    oracle, the same bits on a second call (the counters reset themselves), and as the batch-1 matvec."""
+    codes, scales, zeros, A = oa.make_q3_problem(900 + K % 97 + N % 13, K, N, x_dtype=np.float16, batch=2)
+    mat = oracle.q3_pack(codes)
+    if force:
+        tunable("HQ_Q3_KSPLIT", force)
+    assert _plan(K, N, 2) == PLAN_ROWS
+    y = _run(hq, A, mat, scales, zeros)
+    _check(y, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
+    assert np.array_equal(_run(hq, A, mat, scales, zeros), y)
+    for m in range(2):
+        yv = hq.q3_matvec(_t(A[m]), _t(mat), _t(scales), _t(zeros)).cpu().numpy()
+        assert rel_err(y[m], yv) <= 5e-3
+
+
+def test_rows_kernel_split_k_accumulates_and_strict_fences(hq, oracle, tunable):
+    import torch
+    from hecbench_amd import _lib
+    M, K, N = 2, 12288, 2052
+    codes, scales, zeros, A = oa.make_q3_problem(333, K, N, x_dtype=np.float16, batch=M)
+    mat = oracle.q3_pack(codes)
+    y0 = np.random.default_rng(6).standard_normal((M, N)).astype(np.float32)
+    dA, dm, ds, dz = _t(A), _t(mat), _t(scales), _t(zeros)
+    exact = oracle.q3_gemm(A, mat, scales, zeros, mode=0)
+    plain = _run(hq, A, mat, scales, zeros)
+    for strict in (0, 1):
+        tunable("HQ_SPLITK_FENCES", strict)
+        dy = _t(y0)
+        rc = _lib.load().hq_q3_matvec(dA.data_ptr(), 1, dm.data_ptr(), ds.data_ptr(), dz.data_ptr(), dy.data_ptr(),
+                                      K, N, M, 1, None)
+        assert rc == 0
+        torch.cuda.synchronize()
+        got = dy.cpu().numpy()
+        assert np.array_equal(got, y0 + plain)   # one fp32 addition to the finished sum
+        for m in range(M):
+            assert rel_err(got[m] - y0[m], exact[m], FLOOR_F16) <= 1e-3

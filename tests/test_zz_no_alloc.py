@@ -43,7 +43,7 @@ def test_noalloc_matches_workspace_path(hq, oracle):
     big = _problem(oracle, 301, 8192, 2048, 40)
     small = _problem(oracle, 302, 2048, 512, 7)
     for p in (big, small):                      # two calls in a row, the second with a smaller input
-        for batch in (1, p["M"]):
+        for batch in (1, 2, p["M"]):            # the matvec, the two-row kernel (both split K), the GEMM
             want = _call(lib.hq_q3_matvec, p, batch)
             got = _call(lib.hq_q3_matvec_noalloc, p, batch)
             assert np.array_equal(got, want), (p["K"], p["N"], batch)
@@ -51,7 +51,7 @@ def test_noalloc_matches_workspace_path(hq, oracle):
             if batch == 1:
                 assert rel_err(got[0], oracle.q3_matvec_f64(x, mat, scales, zeros)) <= 1e-4
             else:
-                assert rel_err(got, oracle.q3_gemm(A, mat, scales, zeros, mode=0)) <= 5e-3
+                assert rel_err(got, oracle.q3_gemm(A[:batch], mat, scales, zeros, mode=0)) <= 5e-3
     # and again in the other order: the array keeps the last call's contents
     for p in (small, big, small):
         assert np.array_equal(_call(lib.hq_q3_matvec_noalloc, p, 1), _call(lib.hq_q3_matvec, p, 1))
@@ -62,7 +62,7 @@ def test_noalloc_rejects_beyond_its_limits(hq):
     from hecbench_amd import _lib
     lib = _lib.load()
     dev = torch.device("cuda:0")
-    K, N, M = 32768, 64, 2                      # the batched path's activations would need 4 MiB
+    K, N, M = 32768, 64, 3                      # the batched path's activations would need 4 MiB
     A = torch.zeros((M, K), dtype=torch.float16, device=dev)
     w = torch.zeros((3 * K // 32, N), dtype=torch.int32, device=dev)
     s = torch.zeros(N, device=dev)
