@@ -131,7 +131,10 @@ extern "C" int hq_reserve_workspace(void* stream, int max_K, int max_N) {
   const size_t rounds = ((size_t)max_K + 4095) / 4096;
   const size_t full_split = tiles * (rounds <= 8 ? rounds : 1);
   const size_t per_cu = tiles + 2 * (size_t)d->cus;
-  const size_t split_floats = (full_split > per_cu ? full_split : per_cu) * 64 * 2;
+  size_t split_floats = (full_split > per_cu ? full_split : per_cu) * 64 * 2;
+  // batches 3 ... 8 on the matvec-like kernel: one partial row per tile, round of K and activation row, at most 8192
+  const size_t block_rows = rounds <= 8 ? (tiles * rounds * 8 < 8192 ? tiles * rounds * 8 : 8192) : 0;
+  if (block_rows * 64 > split_floats) split_floats = block_rows * 64;
   HqWorkspace ws;
   return hq_get_workspace((hipStream_t)stream, gemm_floats > split_floats ? gemm_floats : split_floats,
                           tiles > 1 ? tiles : 1, &ws);

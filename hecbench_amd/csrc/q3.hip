@@ -429,6 +429,10 @@ int hq_q3_rows_launch(const void* x, const int32_t* qweight, const float* scales
                       int K, int N, int gpw, int nsplit, float* partial, unsigned* counters, unsigned flags,
                       hipStream_t stream);
 int hq_q3_rows_groups_per_round(void);
+int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
+                       int K, int N, int M, int nsplit, float* partial, unsigned* counters, unsigned flags,
+                       hipStream_t stream);
+int hq_q3_block_groups_per_round(void);
 
 namespace {
 // Zeroes n words with a kernel (a memset node inside a captured graph is not an option for callers
@@ -440,10 +444,26 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(unsigned* p, int n) {
 }  // namespace
 
 namespace {
-int q3_plan(const HqDevice* dev, int N, int batch_M) {
-  (void)dev; (void)N;
+// Largest batch the matvec-like kernels take by default, and the most partial-sum rows (tiles x splits x batch)
+// the kernel for 3 ... 8 rows may need: what the fixed scratch of the entry point that allocates nothing holds,
+// applied to every caller so that both entry points run the same kernel on the same shape.
+constexpr int kDigitBatchDefault = 8;
+constexpr size_t kBlockPartialRows = 8192;
+
+int q3_plan(const HqDevice* dev, int K, int N, int batch_M) {
   if (batch_M == 1) return HQ_Q3_PLAN_MATVEC;
-  if (batch_M == 2 && hq_tune(HQ_TUNE_Q3_SMALL_BATCH, 1) != 0) return HQ_Q3_PLAN_ROWS;
+  const int limit = hq_tune(HQ_TUNE_Q3_SMALL_BATCH, kDigitBatchDefault);  // 0: every batch takes the GEMM
+  if (batch_M == 2 && limit >= 2) return HQ_Q3_PLAN_ROWS;
+  // 3 ... 8 rows: one single-round workgroup per 4096 elements of K, up to eight.  Five to eight rows take
+  // two passes per workgroup, which pays while the launch is a matter of latency (at most two workgroups
+  // per compute unit: 9.4-14.6 us against the GEMM's 13-19 us at 4096 x 4096 ... 14336 x 4096) and not
+  // when it is a matter of throughput (K=8192, N=28672, 896 workgroups: 27.8-33.1 us against 25.4 us).
+  const int gpr = hq_q3_block_groups_per_round();
+  const size_t rounds = (size_t)(K / 32 + gpr - 1) / gpr;
+  const size_t groups = (size_t)((N + 63) / 64) * rounds;
+  if (batch_M <= limit && batch_M <= 8 && rounds <= 8 && groups * batch_M <= kBlockPartialRows &&
+      (batch_M <= 4 || groups <= 2 * (size_t)dev->cus))
+    return HQ_Q3_PLAN_BLOCK;
   return HQ_Q3_PLAN_GEMM;
 }
 
@@ -456,11 +476,11 @@ struct Q3Split {
   float* partial;
   unsigned* counters;
 };
-int q3_split_k(const HqDevice* dev, int G, int gpr, int ntiles, int rows_out, const HqQ3Scratch* fixed,
-               hipStream_t stream, Q3Split* out) {
+int q3_split_k(const HqDevice* dev, int G, int gpr, int ntiles, int rows_out, bool single_round,
+               const HqQ3Scratch* fixed, hipStream_t stream, Q3Split* out) {
   const int max_split = (G + gpr - 1) / gpr;
   const size_t tile_floats = (size_t)ntiles * rows_out * 64;
-  int nsplit = hq_tune(HQ_TUNE_Q3_KSPLIT, 0);
+  int nsplit = single_round ? max_split : hq_tune(HQ_TUNE_Q3_KSPLIT, 0);
   if (nsplit <= 0) {
     // Up to eight rounds of K: one workgroup per round.  Single-round workgroups need half the registers,
     // so two share a CU and one's reduction tail runs under the other's loads, and 2-8 times as many
@@ -502,7 +522,7 @@ extern "C" int hq_q3_matvec_plan(int K, int N, int batch_M) {
   if (K <= 0 || N <= 0 || batch_M <= 0 || (K & 31) || (N & 3)) return HQ_ERR_BAD_SHAPE;
   const HqDevice* dev = nullptr;
   const int rc = hq_current_device(&dev);
-  return rc != HQ_OK ? rc : q3_plan(dev, N, batch_M);
+  return rc != HQ_OK ? rc : q3_plan(dev, K, N, batch_M);
 }
 
 extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float* scales,
@@ -527,14 +547,22 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   if (rc != HQ_OK) return rc;
   if (batch_M > 1) {
     if (x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
-    // A batch of 2 rides on the matvec's digit kernel (one pass over the weights, one launch); everything
+    // Small batches ride on the matvec's digit kernels (one pass over the weights, one launch); everything
     // else takes the batched GEMM.
-    if (q3_plan(dev, N, batch_M) == HQ_Q3_PLAN_ROWS) {
+    const int plan = q3_plan(dev, K, N, batch_M);
+    if (plan == HQ_Q3_PLAN_ROWS) {
       Q3Split sp;
-      rc = q3_split_k(dev, K / 32, hq_q3_rows_groups_per_round(), (N + 63) / 64, 2, fixed, stream, &sp);
+      rc = q3_split_k(dev, K / 32, hq_q3_rows_groups_per_round(), (N + 63) / 64, 2, false, fixed, stream, &sp);
       if (rc != HQ_OK) return rc;
       return hq_q3_rows_launch(x, qweight, scales, zeros, y, K, N, sp.gpw, sp.nsplit, sp.partial, sp.counters, flags,
                                stream);
+    }
+    if (plan == HQ_Q3_PLAN_BLOCK) {
+      Q3Split sp;
+      rc = q3_split_k(dev, K / 32, hq_q3_block_groups_per_round(), (N + 63) / 64, batch_M, true, fixed, stream, &sp);
+      if (rc != HQ_OK) return rc;
+      return hq_q3_block_launch(x, qweight, scales, zeros, y, K, N, batch_M, sp.nsplit, sp.partial, sp.counters, flags,
+                                stream);
     }
     return hq_q3_gemm_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream, fixed);
   }
@@ -554,7 +582,7 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   }
   const int gpr = waves * 4 * steps;  // k-groups one workgroup covers per round
   Q3Split sp;
-  rc = q3_split_k(dev, G, gpr, ntiles, 1, fixed, stream, &sp);
+  rc = q3_split_k(dev, G, gpr, ntiles, 1, false, fixed, stream, &sp);
   if (rc != HQ_OK) return rc;
 
   Q3Args a;

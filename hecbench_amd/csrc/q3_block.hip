@@ -1,0 +1,358 @@
+// GPTQ 3-bit product for small batches (3 ... 8 activation rows) on the matvec's matrix-core kernel, gfx950.
+//
+// q3.hip (batch 1) and q3_rows.hip (batch 2) carry the activations as fixed point relative to the largest
+// magnitude a wave sees in a round, eight or seven 4-bit digits per activation, so one matrix-core pass over
+// the weights serves one or two rows.  Here every k-group (32 consecutive activations of a row) has its own
+// power of two, applied by the matrix core itself: the fp8 operand of v_mfma_scale_f32_16x16x128_f8f6f4 takes
+// one E8M0 scale per 32 elements of K and column.  And a digit is not a nibble but a small fp8 (e4m3) number:
+// with v = the activation times the power of two that puts the k-group's largest magnitude into [1/8, 1/4),
+//   b1 = fp8(v), b2 = fp8(16 (v - b1)), b3 = fp8(16 (16 (v - b1) - b2)), b4 likewise,
+// every term takes the next four significant bits of what is left, but never below the fp8 format's
+// subnormal step 2^-9: in units of that step the terms are integers up to 127 with four significant bits.
+// Products with the 3-bit codes and their sums over the 128 elements of an MFMA stay below 2^17 in those
+// units, so the matrix core adds them exactly, as it does the nibbles of q3.hip.  Four terms reach 19 bits
+// below the k-group's largest magnitude (an fp16 activation within 2^8 of it enters exactly, one 2^12 below
+// it keeps seven bits); the 16^-t of term t rides on the same E8M0 scale, so a row's result is the plain sum
+// of its four columns and the sixteen operand columns carry FOUR rows.  (Three terms that follow the
+// activation's own exponent all the way - exact fp16 in fifteen columns for five rows - were built as well:
+// the matrix core does not add products that far apart exactly, 5e-5 of the output RMS was lost.)
+// Five to eight rows take two passes over the weights held in registers: terms of four rows staged in LDS,
+// sixteen MFMAs per wave, the pass's sums folded into four registers, next four rows.  (Three and four
+// passes no longer fit the 128 registers that let two workgroups share a compute unit, and from nine rows on
+// the activations a workgroup reads outweigh its weights: 13.0-21.8 us against the batched GEMM's 13.3-18.0
+// us on 4096 x 4096 ... 8192 x 8192.)
+// Everything else follows q3.hip: a workgroup owns a 64-column tile and one round of K (8 waves x 4 steps x
+// 4 k-groups = 4096 elements), a wave's 16-lane quarter streams one k-group per step as three 128-bit loads,
+// every wave stages its own operand behind a wave-local fence, the waves meet once at the end, and K beyond
+// one round is split across workgroups whose partial sums the last one to arrive adds up in split order.
+// The weights are read once for all rows at nine VALU instructions per 32 weights and pass, in one launch,
+// where the batched GEMM (q3_gemm.hip) needs a pre-pass, twenty per 32 weights, and a third launch when it
+// splits K.  No counterpart in the reference (its kernels are batch 1: src/quant3MatMul-hip/kernels.h:12-217).
+#include "hq_internal.h"
+
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+
+struct BlockArgs {
+  const _Float16* x;  // [M][K]
+  const uint32_t* w;
+  const float* scales;
+  const float* zeros;
+  float* y;           // [M][N]
+  float* partial;     // [tile][split][M][64] when K is split
+  unsigned* counters; // [tile] arrival counters, zero between calls
+  int K, N, M;
+  int nsplit;         // workgroups per column tile, one round of K each
+  unsigned flags;
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_f(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+__device__ __forceinline__ float quad_max(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));  // quad_perm [1,0,3,2]
+  return fmaxf(v, dpp_f<0x4E>(v));  // quad_perm [2,3,0,1]
+}
+__device__ __forceinline__ float quad_sum(float v) {
+  v += dpp_f<0xB1>(v);
+  return v + dpp_f<0x4E>(v);
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v = quad_sum(v);
+  v += dpp_f<0x141>(v);  // row_half_mirror
+  v += dpp_f<0x140>(v);  // row_mirror
+  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
+}
+
+constexpr uint32_t low3_mask(int word) {
+  uint32_t m = 0;
+  for (int b = 0; b < 32; ++b)
+    if ((32 * word + b) % 6 < 3) m |= 1u << b;
+  return m;
+}
+
+typedef float f2 __attribute__((ext_vector_type(2)));
+// Four floats to four fp8 (e4m3, round to nearest even) bytes of one register, and what the bytes are worth.
+__device__ __forceinline__ uint32_t to_fp8x4(const float (&v)[4]) {
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w, true);
+  return (uint32_t)w;
+}
+__device__ __forceinline__ void from_fp8x4(uint32_t w, float (&v)[4]) {
+  const f2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+  v[0] = lo.x; v[1] = lo.y; v[2] = hi.x; v[3] = hi.y;
+}
+
+constexpr int kWaves = 8, kSteps = 4;
+constexpr int kGroupsPerRound = kWaves * 4 * kSteps;  // k-groups of one workgroup
+constexpr int kRowBytes = 144;                // one B operand row (4 lane quarters x 32 B) plus 16 B: rows start 4 banks apart
+constexpr int kTerms = 4;                     // fp8 terms per activation
+constexpr int kPassRows = 4;                  // rows of activations per pass: sixteen operand columns
+constexpr int kStepBytes = 16 * kRowBytes;    // sixteen operand rows
+constexpr int kScaleOff = kSteps * kStepBytes + 160;  // behind the last step and its skew
+constexpr int kWaveBytes = (kScaleOff + 64 + 127) / 128 * 128;  // + scales[4 rows][4 quarters][4 steps], one byte each
+constexpr int kMaxRows = 2 * kPassRows;
+constexpr int kWsumStride = 8;
+// the four steps are written by the four lane quarters of one instruction: 32-byte slots 0, 1, 4, 5 of a 256-byte bank period
+__device__ __forceinline__ constexpr int step_off(int s) {
+  return s * kStepBytes + (s & 1) * 32 + ((s >> 1) & 1) * 128;
+}
+
+// PASSES = ceil(M / 4).  A pass leaves four registers per lane (its sixteen sums spread over the four lanes
+// of a row's columns); a wave's final sums re-use its operand area.  Two workgroups share a compute unit
+// (at most 128 registers, 76 KB of LDS): one's staging and reduction run under the other's loads.
+template <int PASSES>
+__global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void q3_block_kernel(BlockArgs a) {
+  // LDS: dig[kWaves][kWaveBytes] | wsum[kWaves][kWsumStride]
+  extern __shared__ uint4 smem[];
+  char* dig = reinterpret_cast<char*>(smem);
+  float* wsum = reinterpret_cast<float*>(dig + kWaves * kWaveBytes);
+  static_assert(kSteps * kStepBytes >= kMaxRows * 64 * 4, "a wave's digit area must hold its final sums");
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 15, kb = lane >> 4;
+  const int tile = blockIdx.x, split = blockIdx.y;
+  const int g_begin = split * kGroupsPerRound;
+  const int G = min(kGroupsPerRound, (a.K >> 5) - g_begin);  // k-groups of this workgroup
+  const int M = a.M;
+
+  // staging role: lane converts the eight consecutive activations 8*xq .. 8*xq+7 of k-group xkb of step xs
+  const int xs = lane >> 4, xkb = (lane >> 2) & 3, xq = lane & 3;
+  const int tile_cols = min(64, a.N - tile * 64);  // multiple of 4
+  const uint32_t col_off = (uint32_t)min(4 * c, tile_cols - 4) * 4u;
+  const uint32_t row_bytes = (uint32_t)a.N * 4u;
+  const char* wbase = reinterpret_cast<const char*>(a.w) + (size_t)g_begin * 3 * row_bytes + (size_t)tile * 64 * 4;
+  const _Float16* xbase = a.x + (size_t)g_begin * 32;
+
+  // ---- all loads of the workgroup's round: weights first (HBM), then the activation rows (L2) ----------
+  uint32_t wreg[kSteps][3][4];
+#pragma unroll
+  for (int s = 0; s < kSteps; ++s) {
+    const uint32_t g = (uint32_t)min(s * (kWaves * 4) + wv * 4 + kb, G - 1);
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      const size_t off = (size_t)(g * 3u + (uint32_t)j) * row_bytes + col_off;
+      const u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wbase + off));
+      wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
+    }
+  }
+  const int xg = xs * (kWaves * 4) + wv * 4 + xkb;  // the k-group this lane stages
+  const bool live = xg < G;
+  u4v xraw[PASSES][kPassRows];
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p)
+#pragma unroll
+    for (int m = 0; m < kPassRows; ++m) {
+      const int mg = min(kPassRows * p + m, M - 1);  // rows beyond the batch repeat the last one and are not used
+      xraw[p][m] = *reinterpret_cast<const u4v*>(xbase + (size_t)mg * a.K + (uint32_t)min(xg, G - 1) * 32u + (uint32_t)xq * 8u);
+    }
+
+  char* dig_w = dig + wv * kWaveBytes;
+  unsigned char* sc_tab = reinterpret_cast<unsigned char*>(dig_w + kScaleOff);
+  float* red_w = reinterpret_cast<float*>(dig_w);
+  // MFMA column c carries term c % 4 of row c / 4 of the pass
+  const int crow = c >> 2, cterm = c & 3;
+  f4 keep[PASSES];
+  constexpr uint32_t M0 = low3_mask(0), M1 = low3_mask(1), M2 = low3_mask(2);
+
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    // ---- stage the fp8 terms and scales of rows 4p .. 4p+3 -------------------------------------------
+#pragma unroll
+    for (int m = 0; m < kPassRows; ++m) {
+      if (kPassRows * p + m >= M) continue;  // uniform; the operand columns of a missing row feed result columns nobody reads
+      const h8 h = __builtin_bit_cast(h8, xraw[p][m]);
+      float xr[8];
+      float amax = 0.f, asum = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        xr[j] = live ? (float)h[j] : 0.f;
+        amax = fmaxf(amax, fabsf(xr[j]));
+        asum += xr[j];
+      }
+      const float gmax = quad_max(amax);  // the k-group's largest magnitude (its four lanes)
+      const float total = wave_sum(asum);
+      if (lane == 0) wsum[wv * kWsumStride + kPassRows * p + m] = total;
+      // 2^E * max|x| lies in [2^-3, 2^-2): 64 ... 127 subnormal steps of the fp8 format.  fp16 magnitudes: E in -18 ... 21.
+      int E = -3 - ((int)((__float_as_uint(gmax) >> 23) & 255u) - 127);
+      E = gmax > 0.f ? max(-18, min(21, E)) : 0;
+      const float scaleE = __uint_as_float((uint32_t)(E + 127) << 23);
+      // even / odd elements of the k-group go to neighbouring lane quarters of the fp8 operand (see q3.hip)
+      float ve[4], vo[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        ve[j] = xr[2 * j] * scaleE;
+        vo[j] = xr[2 * j + 1] * scaleE;
+      }
+      char* dst = dig_w + step_off(xs) + (kTerms * m) * kRowBytes + (xkb & 1) * 64 + (xkb >> 1) * 16 + xq * 4;
+#pragma unroll
+      for (int t = 0; t < kTerms; ++t) {
+        const uint32_t be = to_fp8x4(ve), bo = to_fp8x4(vo);
+        *reinterpret_cast<uint32_t*>(dst + t * kRowBytes) = be;
+        *reinterpret_cast<uint32_t*>(dst + t * kRowBytes + 32) = bo;
+        if (t + 1 < kTerms) {  // what the term left out (at most half its last place), sixteen times: exact in fp32
+          float fe[4], fo[4];
+          from_fp8x4(be, fe);
+          from_fp8x4(bo, fo);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            ve[j] = (ve[j] - fe[j]) * 16.f;
+            vo[j] = (vo[j] - fo[j]) * 16.f;
+          }
+        }
+      }
+      // E8M0 scale of term 0: 2^-E for the k-group's power of two, 2^3 for the unit of the fp6 operand (code / 8)
+      if (xq == 0) sc_tab[(m * 4 + xkb) * 4 + xs] = (unsigned char)(127 + 3 - E);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+
+    // ---- mask + MFMA -----------------------------------------------------------------------
+    // The matrix-core operand of the weights (six registers per sixteen MFMAs) is rebuilt in every pass: kept
+    // across passes it would double the registers the weights take.  The empty statement hides from the compiler
+    // that the weights are the same as in the last pass.
+    if (p > 0) {
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s)
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(wreg[s][j][q]));
+    }
+    // the scales of the column's row for this lane quarter's k-group in the four steps, times 16^-term
+    const uint32_t sc4 = *reinterpret_cast<const uint32_t*>(sc_tab + (crow * 4 + kb) * 4) - (uint32_t)cterm * 0x04040404u;
+    f4 acc[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+      if (s * (kWaves * 4) + wv * 4 >= G) continue;  // wave-uniform
+      const u4v* bp = reinterpret_cast<const u4v*>(dig_w + step_off(s) + c * kRowBytes + kb * 32);
+      const u4v b0 = bp[0], b1 = bp[1];
+      const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
+      const int scale_b = (int)(sc4 >> (8 * s));  // byte 0: this step's scale
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t w0 = wreg[s][0][q], w1 = wreg[s][1][q], w2 = wreg[s][2][q];
+        const v8i A = {(int)(w0 & M0), (int)(w1 & M1), (int)(w2 & M2),
+                       (int)(__builtin_amdgcn_alignbit(w1, w0, 3) & M0),
+                       (int)(__builtin_amdgcn_alignbit(w2, w1, 3) & M1), (int)((w2 >> 3) & M2), 0, 0};
+        // A: fp6 e2m3 (cbsz 2), unit scale; B: fp8 e4m3 (blgp 0), scale per lane = per column and k-group
+        acc[q] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(A, B, acc[q], 2, 0, 0, 0x7f7f7f7f, 0, scale_b);
+      }
+    }
+    // D[row = 4*kb + i][col = c]: row is the weight column 4*row + q of the tile; a row of activations is the
+    // sum of its four columns (four neighbouring lanes).  Lane c keeps the sums of i = c & 3.
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float v0 = quad_sum(acc[q][0]), v1 = quad_sum(acc[q][1]), v2 = quad_sum(acc[q][2]), v3 = quad_sum(acc[q][3]);
+      float v = (c & 2) ? ((c & 1) ? v3 : v2) : ((c & 1) ? v1 : v0);
+      asm volatile("" : "+v"(v));  // selected here, not where it is stored (four candidates alive until then)
+      keep[p][q] = v;
+    }
+    // the next pass rewrites, and the sums below overwrite, the operand and scales this pass's lanes have just read
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+  }
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p)
+    *reinterpret_cast<f4*>(red_w + (kPassRows * p + crow) * 64 + 4 * (4 * kb + cterm)) = keep[p];
+  __syncthreads();
+
+  // ---- combine the waves, scale and zero --------------------------------------------------------------
+  const int col = tid & 63;
+  const int ncol = tile * 64 + col;
+  const int nc = min(ncol, a.N - 1);
+  const float sc_n = a.scales[nc], zr_n = a.zeros[nc];
+  for (int m = tid >> 6; m < M; m += kWaves) {
+    float qx = 0.f, xsum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float* rw = reinterpret_cast<const float*>(dig + w * kWaveBytes);
+      qx += rw[m * 64 + col];
+      xsum += wsum[w * kWsumStride + m];
+    }
+    float val = sc_n * qx - zr_n * xsum;
+    val = fmaf(xsum, 0.f, val);  // a NaN or infinity among the activations makes the result NaN
+    if (ncol < a.N) {
+      if (a.nsplit == 1) {
+        float* yp = &a.y[(size_t)m * a.N + ncol];
+        const float y_old = (a.flags & HQ_FLAG_ACCUMULATE) ? *yp : 0.f;
+        __hip_atomic_store(yp, y_old + val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        __hip_atomic_store(&a.partial[(((size_t)tile * a.nsplit + split) * M + m) * 64 + col], val, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  if (a.nsplit > 1) {
+    // Arrival counting as in q3.hip: write-through partial sums, every wave waits for their acknowledgement,
+    // a barrier, one device-scope fetch-add per workgroup, and the last workgroup to arrive adds the partial
+    // sums in split order with loads that bypass the non-coherent cache levels.
+    __shared__ unsigned s_last;
+    const bool strict = (a.flags & HQ_FLAG_STRICT_FENCES) != 0;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) {
+      const unsigned old = strict ? __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT)
+                                  : __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = (old == (unsigned)(a.nsplit - 1));
+    }
+    __syncthreads();
+    if (s_last && strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (s_last) {
+      if (ncol < a.N) {
+        for (int m = tid >> 6; m < M; m += kWaves) {
+          float sum = 0.f;
+          for (int s = 0; s < a.nsplit; ++s)
+            sum += __hip_atomic_load(&a.partial[(((size_t)tile * a.nsplit + s) * M + m) * 64 + col], __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+          float* yp = &a.y[(size_t)m * a.N + ncol];
+          *yp = (a.flags & HQ_FLAG_ACCUMULATE) ? *yp + sum : sum;
+        }
+      }
+      if (tid == 0)  // ready for the next call
+        __hip_atomic_store(&a.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+template <int PASSES>
+int launch_block_t(const BlockArgs& a, hipStream_t stream) {
+  const size_t smem = (size_t)kWaves * kWaveBytes + (size_t)kWaves * kWsumStride * 4 + 16;
+  static const hipError_t attr =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_block_kernel<PASSES>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+  if (attr != hipSuccess) return (int)attr;
+  hipLaunchKernelGGL((q3_block_kernel<PASSES>), dim3((a.N + 63) / 64, a.nsplit), dim3(kWaves * 64), smem, stream, a);
+  return hq_launch_status();
+}
+
+}  // namespace
+
+// k-groups one workgroup covers (its one round)
+int hq_q3_block_groups_per_round(void) { return kGroupsPerRound; }
+
+// 3 ... 8 fp16 activation rows; the caller has validated the arguments, set nsplit = ceil(K / 4096) and, for
+// nsplit > 1, provided nsplit * M * 64 floats of partial sums and one zeroed counter per column tile.
+int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
+                       int K, int N, int M, int nsplit, float* partial, unsigned* counters, unsigned flags,
+                       hipStream_t stream) {
+  if (M < 1 || M > kMaxRows || nsplit != (K / 32 + kGroupsPerRound - 1) / kGroupsPerRound) return HQ_ERR_BAD_SHAPE;
+  BlockArgs a;
+  a.x = reinterpret_cast<const _Float16*>(x);
+  a.w = reinterpret_cast<const uint32_t*>(qweight);
+  a.scales = scales; a.zeros = zeros; a.y = y; a.partial = partial; a.counters = counters; a.K = K; a.N = N; a.M = M;
+  a.nsplit = nsplit; a.flags = flags & (HQ_FLAG_ACCUMULATE | HQ_FLAG_STRICT_FENCES);
+  return M <= kPassRows ? launch_block_t<1>(a, stream) : launch_block_t<2>(a, stream);
+}

@@ -124,18 +124,23 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  *   y        : fp32 [batch_M][N]
  *   K % 32 == 0, N % 4 == 0, batch_M >= 1; qweight and x 16-byte aligned.
  * Products are accumulated in fp32 for both dtypes (the reference's fp16
- * variant accumulates 16 terms in fp16).  batch_M > 1 pre-scales every activation
- * row by a power of two, so accuracy does not depend on the magnitude of the
- * activations: entries within 2^21 of their row's largest magnitude enter the
- * matrix cores exactly, smaller ones lose low bits (those 2^32 below it vanish).
+ * variant accumulates 16 terms in fp16).
  * batch_M == 1 replaces vecquant3matmul / vecquant3matmul_faster
  * (src/quant3MatMul-hip/kernels.h:171-217) — pass HQ_FLAG_ACCUMULATE for their
- * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 (no counterpart in the
- * reference): a batch of 2 runs on the matvec's kernel (at about the cost of
- * batch 1) with the two rows side by side in the matrix-core
- * operand (28-bit fixed point relative to the largest magnitude among each 512
- * consecutive activations of a row: exact for fp16 entries within 2^17 of it);
- * all other batches run the MFMA GEMM path.
+ * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 and has no counterpart in
+ * the reference; which kernel serves it (hq_q3_matvec_plan tells):
+ *   - batch 2: the matvec's kernel, at about the cost of batch 1, the two rows side
+ *     by side in the matrix-core operand (28-bit fixed point relative to the largest
+ *     magnitude among each 512 consecutive activations of a row: exact for fp16
+ *     entries within 2^17 of it);
+ *   - batches 3 ... 8 with K <= 32768 (5 ... 8 only while the launch has at most two
+ *     workgroups per compute unit): the matvec's kernel, four rows side by side;
+ *     every activation enters with an error of at most 2^-19 of the largest magnitude
+ *     among its 32 neighbours (exactly, if within 2^8 of it);
+ *   - everything else: the MFMA GEMM path, which pre-scales every activation row by a
+ *     power of two, so accuracy does not depend on the magnitude of the activations:
+ *     entries within 2^21 of their row's largest magnitude enter the matrix cores
+ *     exactly, smaller ones lose low bits (those 2^32 below it vanish).
  */
 int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float* scales,
                  const float* zeros, float* y, int K, int N, int batch_M, unsigned flags,
@@ -148,6 +153,7 @@ int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float
 #define HQ_Q3_PLAN_MATVEC 0 /* batch_M == 1 */
 #define HQ_Q3_PLAN_ROWS 1   /* batch_M == 2 on the matvec's digit kernel */
 #define HQ_Q3_PLAN_GEMM 2   /* batched MFMA GEMM */
+#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 3 ... 8, K <= 32768: the matvec's kernel, four rows per pass */
 int hq_q3_matvec_plan(int K, int N, int batch_M);
 
 /*

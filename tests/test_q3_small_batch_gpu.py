@@ -1,6 +1,7 @@
-"""Batches 2 ... 15 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): a batch of 2 runs on the
+"""Batches 2 ... 16 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): a batch of 2 runs on the
 matvec's digit kernel with the two rows side by side in the matrix-core operand (K split across workgroups
-as for batch 1), all others on the batched GEMM.  Every batch size is checked against the CPU oracle through the C ABI,
+as for batch 1), batches 3 ... 8 on the same kernel with every activation as four small fp8 terms under one
+scale per 32 activations (four rows per pass over the weights), all others on the batched GEMM.  Every batch size is checked against the CPU oracle through the C ABI,
 and the kernel that ran is asserted through hq_q3_matvec_plan.  The reference has no batched kernel:
 the oracle is the matvec formula applied row by row (parity unpinned by the reference)."""
 import numpy as np
@@ -11,7 +12,7 @@ from tests.tol import FLOOR_F16, rel_err
 
 pytestmark = pytest.mark.gpu
 
-PLAN_MATVEC, PLAN_ROWS, PLAN_GEMM = 0, 1, 2
+PLAN_MATVEC, PLAN_ROWS, PLAN_GEMM, PLAN_BLOCK = 0, 1, 2, 3
 
 
 def _t(a):
@@ -48,7 +49,7 @@ _EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)
 def test_every_batch_vs_oracle(hq, oracle, M, K, N):
     codes, scales, zeros, A = oa.make_q3_problem(1000 + 16 * M + (K % 7), K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
-    want_plan = PLAN_ROWS if M == 2 else PLAN_GEMM
+    want_plan = PLAN_ROWS if M == 2 else (PLAN_BLOCK if M <= 8 else PLAN_GEMM)
     assert _plan(K, N, M) == want_plan
     y = _run(hq, A, mat, scales, zeros)
     _check(y, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
@@ -114,9 +115,9 @@ def test_rows_kernel_non_finite_activations(hq, oracle):
     assert np.all(np.isnan(y[1]))
 
 
-def test_config4_shape_batches_2_and_3(hq, oracle):
-    """K=8192, N=28672 (the GEMM configuration's weights) at batch 2 (two-row kernel) and 3 (GEMM): sampled
-    columns against the oracle, all columns against the batch-1 matvec."""
+def test_config4_shape_batches_2_3_and_11(hq, oracle):
+    """K=8192, N=28672 (the GEMM configuration's weights) at batch 2 (two-row kernel), 3 (four rows per pass)
+    and 11 (GEMM): sampled columns against the oracle, all columns against the batch-1 matvec."""
     import torch
     K, N = 8192, 28672
     rng = np.random.default_rng(45)
@@ -126,9 +127,9 @@ def test_config4_shape_batches_2_and_3(hq, oracle):
     dm, ds, dz = _t(mat), _t(scales), _t(zeros)
     cols = np.unique(np.concatenate([np.arange(0, 132), np.arange(N - 132, N), rng.integers(0, N, 120)]))
     sub = np.ascontiguousarray(mat[:, cols])
-    for M in (2, 3):
+    for M in (2, 3, 11):
         A = rng.standard_normal((M, K)).astype(np.float16)
-        assert _plan(K, N, M) == (PLAN_ROWS if M == 2 else PLAN_GEMM)
+        assert _plan(K, N, M) == {2: PLAN_ROWS, 3: PLAN_BLOCK, 11: PLAN_GEMM}[M]
         y = hq.q3_gemm(_t(A), dm, ds, dz)
         torch.cuda.synchronize()
         y = y.cpu().numpy()
@@ -213,3 +214,138 @@ def test_rows_kernel_split_k_accumulates_and_strict_fences(hq, oracle, tunable):
         assert np.array_equal(got, y0 + plain)   # one fp32 addition to the finished sum
         for m in range(M):
             assert rel_err(got[m] - y0[m], exact[m], FLOOR_F16) <= 1e-3
+
+
+@pytest.mark.parametrize("M,K,N", [(M, K, N) for (K, N) in [(1024, 196), (4128, 8192)] for M in (2, 3, 4, 5, 8)])
+def test_small_batches_on_the_gemm(hq, oracle, tunable, M, K, N):
+    """HQ_Q3_SMALL_BATCH=0 keeps the digit kernels out: the GEMM serves the small batches as well."""
+    tunable("HQ_Q3_SMALL_BATCH", 0)
+    assert _plan(K, N, M) == PLAN_GEMM
+    codes, scales, zeros, A = oa.make_q3_problem(1300 + M, K, N, x_dtype=np.float16, batch=M)
+    mat = oracle.q3_pack(codes)
+    _check(_run(hq, A, mat, scales, zeros), oracle.q3_gemm(A, mat, scales, zeros, mode=0))
+
+
+# one and two passes of four rows, full and partly filled; K of one round, a K the rounds do not divide
+# (two workgroups per tile) and eight rounds; N with a 4-column last tile
+_BLOCK_CASES = [(M, K, N) for (K, N) in [(4128, 1028), (160, 16388)] for M in (3, 4, 5, 6, 7, 8)] + \
+               [(6, 32768, 260), (8, 16384, 196), (4, 8192, 4096)]
+
+
+@pytest.mark.parametrize("M,K,N", _BLOCK_CASES)
+def test_block_kernel_vs_oracle(hq, oracle, M, K, N):
+    """Four rows per pass, four fp8 terms per activation: against the oracle at the batch-1 kernel's bound
+    (N(0,1) activations enter exactly) and, row by row, the batch-1 matvec; a second call gives the same bits
+    (partial sums and counters are left ready)."""
+    assert _plan(K, N, M) == PLAN_BLOCK
+    codes, scales, zeros, A = oa.make_q3_problem(1500 + 16 * M + K % 11, K, N, x_dtype=np.float16, batch=M)
+    mat = oracle.q3_pack(codes)
+    y = _run(hq, A, mat, scales, zeros)
+    exact = oracle.q3_gemm(A, mat, scales, zeros, mode=0)
+    for m in range(M):
+        assert rel_err(y[m], exact[m]) <= 1e-3, m
+    assert np.array_equal(_run(hq, A, mat, scales, zeros), y)
+    dm, ds, dz = _t(mat), _t(scales), _t(zeros)
+    for m in (0, M - 1):
+        yv = hq.q3_matvec(_t(A[m]), dm, ds, dz).cpu().numpy()
+        assert rel_err(y[m], yv) <= 1e-3
+
+
+def test_block_kernel_plan_limits(hq, tunable):
+    """Beyond eight rounds of K, beyond 8 rows, beyond two workgroups per compute unit for 5 ... 8 rows, or with
+    more partial sums than the fixed scratch of the entry point that allocates nothing holds, the batch takes
+    the GEMM; HQ_Q3_SMALL_BATCH lowers the limit.  (The counts below are for 256 compute units.)"""
+    assert _plan(32768, 256, 8) == PLAN_BLOCK
+    assert _plan(32800, 256, 8) == PLAN_GEMM
+    assert _plan(4096, 4096, 8) == PLAN_BLOCK
+    assert _plan(4096, 4096, 9) == PLAN_GEMM
+    assert _plan(8192, 28672, 4) == PLAN_BLOCK        # 448 tiles x 2 rounds: 896 workgroups, one pass each
+    assert _plan(8192, 28672, 5) == PLAN_GEMM         # two passes each only up to two workgroups per compute unit
+    assert _plan(8192, 16384, 8) == PLAN_BLOCK        # 512 workgroups
+    assert _plan(12288, 65536, 2) == PLAN_ROWS
+    assert _plan(12288, 65536, 3) == PLAN_GEMM        # 1024 tiles x 3 rounds x 3 rows = 9216 partial rows
+    tunable("HQ_Q3_SMALL_BATCH", 16)
+    assert _plan(4096, 4096, 9) == PLAN_GEMM
+    tunable("HQ_Q3_SMALL_BATCH", 4)
+    assert _plan(4096, 4096, 4) == PLAN_BLOCK
+    assert _plan(4096, 4096, 5) == PLAN_GEMM
+    tunable("HQ_Q3_SMALL_BATCH", 1)
+    assert _plan(4096, 4096, 2) == PLAN_GEMM
+
+
+@pytest.mark.parametrize("scale_exp", [-16, -8, 0, 4])
+def test_block_kernel_dynamic_range(hq, oracle, scale_exp):
+    """Rows of very different magnitude side by side in one matrix-core operand, an all-zero row, a row with
+    one large outlier, magnitudes spread over 2^8 inside a row, a large entry in every k-group, fp16
+    subnormals: every row is held to the bound the N(0,1) cases meet, measured against that row's own RMS."""
+    K, N = 2048, 2052
+    rng = np.random.default_rng(211 + scale_exp)
+    codes, scales, zeros, A = oa.make_q3_problem(280 + scale_exp, K, N, x_dtype=np.float16, batch=9)
+    mat = oracle.q3_pack(codes)
+    A = A.astype(np.float32) * np.float32(2.0 ** scale_exp)
+    A[1] *= np.float32(2.0 ** -6)
+    A[2] *= np.float32(2.0 ** 5)
+    A[4] = 0.0
+    A[5, 100] = np.float32(2.0 ** min(15, scale_exp + 12))
+    A[6] = rng.standard_normal(K).astype(np.float32) * np.float32(2.0 ** scale_exp) * \
+        np.exp2(rng.integers(-8, 1, K)).astype(np.float32)
+    A[7, 512:] = 0.0
+    A[8, ::32] *= np.float32(64.0)                         # one large entry in every group of 32
+    A = A.astype(np.float16)
+    exact = oracle.q3_gemm(A, mat, scales, zeros, mode=0)
+    for rows in (list(range(8)), [5, 4, 1, 2], [6, 7, 8], [8, 3, 5, 0, 4, 7]):
+        sub = np.ascontiguousarray(A[rows])
+        assert _plan(K, N, len(rows)) == PLAN_BLOCK
+        y = _run(hq, sub, mat, scales, zeros)
+        for i, m in enumerate(rows):
+            if m == 4:
+                assert np.all(y[i] == 0.0)
+            else:
+                assert rel_err(y[i], exact[m]) <= 5e-3, (scale_exp, m)
+                assert rel_err(y[i], exact[m], FLOOR_F16) <= 1e-4, (scale_exp, m)
+
+
+def test_block_kernel_non_finite_activations(hq, oracle):
+    """An infinity or NaN in one row makes that row NaN and leaves the other rows alone."""
+    K, N = 4608, 1024
+    codes, scales, zeros, A = oa.make_q3_problem(92, K, N, x_dtype=np.float16, batch=6)
+    mat = oracle.q3_pack(codes)
+    A[1, 37] = np.float16(np.inf)
+    A[4, 4500] = np.float16(np.nan)
+    assert _plan(K, N, 6) == PLAN_BLOCK
+    y = _run(hq, A, mat, scales, zeros)
+    exact = oracle.q3_gemm(A, mat, scales, zeros, mode=0)
+    for m in (0, 2, 3, 5):
+        assert rel_err(y[m], exact[m]) <= 5e-3
+    assert np.all(np.isnan(y[1])) and np.all(np.isnan(y[4]))
+
+
+def test_block_kernel_accumulates_and_strict_fences(hq, oracle, tunable):
+    import torch
+    from hecbench_amd import _lib
+    for (M, K, N) in [(5, 12288, 2052), (3, 512, 8196)]:     # K split three ways; one workgroup per tile
+        codes, scales, zeros, A = oa.make_q3_problem(433 + M, K, N, x_dtype=np.float16, batch=M)
+        mat = oracle.q3_pack(codes)
+        y0 = np.random.default_rng(7).standard_normal((M, N)).astype(np.float32)
+        dA, dm, ds, dz = _t(A), _t(mat), _t(scales), _t(zeros)
+        assert _plan(K, N, M) == PLAN_BLOCK
+        plain = _run(hq, A, mat, scales, zeros)
+        _check(plain, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
+        for strict in (0, 1):
+            tunable("HQ_SPLITK_FENCES", strict)
+            dy = _t(y0)
+            rc = _lib.load().hq_q3_matvec(dA.data_ptr(), 1, dm.data_ptr(), ds.data_ptr(), dz.data_ptr(), dy.data_ptr(),
+                                          K, N, M, 1, None)
+            assert rc == 0
+            torch.cuda.synchronize()
+            assert np.array_equal(dy.cpu().numpy(), y0 + plain)   # one fp32 addition to the finished sum
+
+
+@pytest.mark.parametrize("K", [32, 96, 160])
+def test_block_kernel_short_k(hq, oracle, K):
+    """Fewer k-groups than a workgroup's waves cover: idle waves, partly filled steps."""
+    N = 520
+    codes, scales, zeros, A = oa.make_q3_problem(800 + K, K, N, x_dtype=np.float16, batch=7)
+    mat = oracle.q3_pack(codes)
+    assert _plan(K, N, 7) == PLAN_BLOCK
+    _check(_run(hq, A, mat, scales, zeros), oracle.q3_gemm(A, mat, scales, zeros, mode=0))
