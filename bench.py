@@ -212,6 +212,27 @@ def bench_configs(steps, warmup, windows):
                                                        "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                                        "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None}
     del mats, Ag, og
+    # the headline shape at batches 2, 4 and 8 (extension: one pass over the weights for all rows, 34 rotated buffers)
+    Ks, Ns = K, N
+    nb = 34
+    mats = [torch.randint(-2 ** 31, 2 ** 31 - 1, (3 * Ks // 32, Ns), dtype=torch.int32, device=dev, generator=g)
+            for _ in range(nb)]
+    ss = torch.empty(Ns, device=dev).uniform_(0.005, 0.02, generator=g)
+    zs = ss * torch.randint(3, 5, (Ns,), device=dev, generator=g).float()
+    pm = [vp(m) for m in mats]
+    for Ms in (2, 4, 8):
+        As = torch.randn(Ms, Ks, device=dev, generator=g).half()
+        os_ = torch.empty(Ms, Ns, device=dev)
+        pA, pss, pzs, pos = vp(As), vp(ss), vp(zs), vp(os_)
+        plan = lib.hq_q3_matvec_plan(Ks, Ns, Ms)
+        secs = _time_windows(lambda i: check(lib.hq_q3_matvec(pA, 1, pm[i], pss, pzs, pos, Ks, Ns, Ms, 0, stream)),
+                             nb, steps, warmup, windows)
+        entry("1_q3_matvec_4096x11008_batch%d" % Ms,
+              "GPTQ 3-bit K=4096 N=11008, %d fp16 activation rows in one call, 34 rotated weight buffers (575 MB)" % Ms,
+              3 * Ks // 32 * Ns * 4 + 2 * Ns * 4 + Ms * Ks * 2 + Ms * Ns * 4, secs, steps, "q3_batch%d_4096x11008" % Ms,
+              dtype="fp6 x fp8 MFMA, exact integer sums, f32 out",
+              kernel={1: "two rows per pass", 2: "batched GEMM", 3: "four rows per pass"}.get(plan, str(plan)))
+    del mats
     return out
 
 
