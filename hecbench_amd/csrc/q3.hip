@@ -156,9 +156,27 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   constexpr int GPR = WAVES * 4 * STEPS;  // k-groups per round
   const int rounds = MULTI ? (g_count + GPR - 1) / GPR : 1;  // !MULTI: the host sized gpw <= GPR
 
-  // Every global load of a round is issued up front and none sits under a branch
-  // (addresses are clamped instead), so the compiler can count them and the wait for the
-  // activations does not wait for the weights.
+  // No global load sits under a branch (addresses are clamped instead), so the compiler can count
+  // them and the wait for the activations does not wait for the weights.  A workgroup with more than one
+  // round issues a round's loads at once, one round ahead.  A single-round workgroup issues the
+  // activations and the first kEarly steps' weights at entry and the weights of step s + kEarly just before the
+  // arithmetic of step s: a compute unit takes about 64 KB of outstanding loads, a wave stalls at a
+  // load while that queue is full, and a stalled wave stages nothing (K=4096, N=11008: 5.45 -> 5.38 us; one
+  // step early 5.42, three 5.40).
+  constexpr int kEarly = MULTI ? STEPS : (STEPS < 2 ? STEPS : 2);
+  auto load_steps = [&](int r, uint32_t (&wreg)[STEPS][3][4], int s0, int s1) {
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      if (s < s0 || s >= s1) continue;
+      const uint32_t g = (uint32_t)min((r * STEPS + s) * (WAVES * 4) + wv * 4 + kb, g_count - 1);
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const uint32_t off = (g * 3u + (uint32_t)j) * row_bytes + col_off;
+        u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wbase + off));
+        wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
+      }
+    }
+  };
   auto load_round = [&](int r, float (&xr)[XP][8], uint32_t (&wreg)[STEPS][3][4]) {
 #pragma unroll
     for (int p = 0; p < XP; ++p) {
@@ -177,16 +195,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
         for (int j = 0; j < 4; ++j) { xr[p][j] = lo[j]; xr[p][4 + j] = hi[j]; }
       }
     }
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const uint32_t g = (uint32_t)min((r * STEPS + s) * (WAVES * 4) + wv * 4 + kb, g_count - 1);
-#pragma unroll
-      for (int j = 0; j < 3; ++j) {
-        const uint32_t off = (g * 3u + (uint32_t)j) * row_bytes + col_off;
-        u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wbase + off));
-        wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
-      }
-    }
+    load_steps(r, wreg, 0, kEarly);
   };
 
   char* dig_w = dig + wv * (STEPS * kStepBytes);
@@ -207,6 +216,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   float xr[XP][8];
   uint32_t wreg[STEPS][3][4];
   load_round(0, xr, wreg);
+  if (!MULTI) __builtin_amdgcn_sched_barrier(0);
   for (int r = 0; r < rounds; ++r) {
     float xr_next[XP][8];
     uint32_t wreg_next[STEPS][3][4];
@@ -273,6 +283,10 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
     for (int q = 0; q < 4; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
+      if (!MULTI && s + kEarly < STEPS) {
+        load_steps(0, wreg, s + kEarly, s + kEarly + 1);
+        __builtin_amdgcn_sched_barrier(0);  // issued here, not where the compiler would like it
+      }
       if ((r * STEPS + s) * (WAVES * 4) + wv * 4 >= g_count) continue;  // wave-uniform
       // MFMA columns 9..15 are never read: they re-use row 8
       const u4v* bp = reinterpret_cast<const u4v*>(dig_w + step_off(s) + min(c, 8) * kRowBytes + kb * 32);
