@@ -469,14 +469,15 @@ int q3_plan(const HqDevice* dev, int K, int N, int batch_M) {
   const int limit = hq_tune(HQ_TUNE_Q3_SMALL_BATCH, kDigitBatchDefault);  // 0: every batch takes the GEMM
   if (batch_M == 2 && limit >= 2) return HQ_Q3_PLAN_ROWS;
   // 3 ... 8 rows: one single-round workgroup per 4096 elements of K, up to eight.  Five to eight rows take
-  // two passes per workgroup, which pays while the launch is a matter of latency (at most two workgroups
-  // per compute unit: 9.4-14.6 us against the GEMM's 13-19 us at 4096 x 4096 ... 14336 x 4096) and not
-  // when it is a matter of throughput (K=8192, N=28672, 896 workgroups: 27.8-33.1 us against 25.4 us).
+  // two passes per workgroup, which beats the GEMM (7.8-12.4 us against 13-19 us at 4096 x 4096 ... 14336 x
+  // 4096, 20.7-24.9 against 24.7 at K=8192, N=22016, 26.5-31.9 against 31.6 at K=28672, N=8192) except where
+  // the GEMM's 128-column tiles fill the device without a K split (K=8192, N=28672: 27.8-31.1 against 25.3 us).
   const int gpr = hq_q3_block_groups_per_round();
   const size_t rounds = (size_t)(K / 32 + gpr - 1) / gpr;
   const size_t groups = (size_t)((N + 63) / 64) * rounds;
+  const size_t tiles128 = (size_t)(N + 127) / 128;
   if (batch_M <= limit && batch_M <= 8 && rounds <= 8 && groups * batch_M <= kBlockPartialRows &&
-      (batch_M <= 4 || groups <= 2 * (size_t)dev->cus))
+      (batch_M <= 4 || 8 * tiles128 < 7 * (size_t)dev->cus))
     return HQ_Q3_PLAN_BLOCK;
   return HQ_Q3_PLAN_GEMM;
 }

@@ -133,8 +133,8 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  *     by side in the matrix-core operand (28-bit fixed point relative to the largest
  *     magnitude among each 512 consecutive activations of a row: exact for fp16
  *     entries within 2^17 of it);
- *   - batches 3 ... 8 with K <= 32768 (5 ... 8 only while the launch has at most two
- *     workgroups per compute unit): the matvec's kernel, four rows side by side;
+ *   - batches 3 ... 8 with K <= 32768 (5 ... 8 unless N / 128 is at least 7/8 of the
+ *     compute units): the matvec's kernel, four rows side by side;
  *     every activation enters with an error of at most 2^-19 of the largest magnitude
  *     among its 32 neighbours (exactly, if within 2^8 of it);
  *   - everything else: the MFMA GEMM path, which pre-scales every activation row by a

@@ -252,16 +252,17 @@ def test_block_kernel_vs_oracle(hq, oracle, M, K, N):
 
 
 def test_block_kernel_plan_limits(hq, tunable):
-    """Beyond eight rounds of K, beyond 8 rows, beyond two workgroups per compute unit for 5 ... 8 rows, or with
-    more partial sums than the fixed scratch of the entry point that allocates nothing holds, the batch takes
-    the GEMM; HQ_Q3_SMALL_BATCH lowers the limit.  (The counts below are for 256 compute units.)"""
+    """Beyond eight rounds of K, beyond 8 rows, for 5 ... 8 rows where the GEMM's 128-column tiles fill the device,
+    or with more partial sums than the fixed scratch of the entry point that allocates nothing holds, the batch
+    takes the GEMM; HQ_Q3_SMALL_BATCH lowers the limit.  (The counts below are for 256 compute units.)"""
     assert _plan(32768, 256, 8) == PLAN_BLOCK
     assert _plan(32800, 256, 8) == PLAN_GEMM
     assert _plan(4096, 4096, 8) == PLAN_BLOCK
     assert _plan(4096, 4096, 9) == PLAN_GEMM
-    assert _plan(8192, 28672, 4) == PLAN_BLOCK        # 448 tiles x 2 rounds: 896 workgroups, one pass each
-    assert _plan(8192, 28672, 5) == PLAN_GEMM         # two passes each only up to two workgroups per compute unit
-    assert _plan(8192, 16384, 8) == PLAN_BLOCK        # 512 workgroups
+    assert _plan(8192, 28672, 4) == PLAN_BLOCK        # one pass per workgroup: always
+    assert _plan(8192, 28672, 5) == PLAN_GEMM         # two passes: not where the GEMM's 224 tiles fill the device
+    assert _plan(8192, 22016, 8) == PLAN_BLOCK        # 172 tiles of 128 columns
+    assert _plan(28672, 8192, 8) == PLAN_BLOCK
     assert _plan(12288, 65536, 2) == PLAN_ROWS
     assert _plan(12288, 65536, 3) == PLAN_GEMM        # 1024 tiles x 3 rounds x 3 rows = 9216 partial rows
     tunable("HQ_Q3_SMALL_BATCH", 16)
