@@ -621,21 +621,23 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a)
 #pragma unroll
       for (int j = 0; j < 4; ++j) xv[sp_][j] = (float)xp[4 * j];
     }
-#pragma unroll
-    for (int t = 0; t < QUADS; ++t) {
+    // The activations and the first quad's loads go out here, every further quad's just before the
+    // arithmetic of the quad ahead of it (see bcq_planes_kernel: a wave stalls at a load while the compute
+    // unit's queue of outstanding loads is full, and with a round's loads issued at once the later waves
+    // get their data, and do their arithmetic, after the stream has ended).
+    Half16 al[QUADS][NB], bi[QUADS];
+    auto load_quad = [&](int t) {
       const int quad = min(q0 + t, nquads - 1);
       const uint32_t* wp = a.bW + ((size_t)(4 * quad + kb) * NB) * a.N + n0 + col_off;
 #pragma unroll
       for (int b = 0; b < NB; ++b) wq[t][b] = load_words<RAGGED>(wp + (size_t)b * a.N);
-    }
-    Half16 al[QUADS][NB], bi[QUADS];
-#pragma unroll
-    for (int t = 0; t < QUADS; ++t) {
-      const int g = min(q0 + t, nquads - 1) * GS + cg;
+      const int g = quad * GS + cg;
 #pragma unroll
       for (int b = 0; b < NB; ++b) al[t][b] = load_half16<RAGGED>(a.alpha + ((size_t)g * NB + b) * a.N + n0 + acol);
       if (BIAS) bi[t] = load_half16<RAGGED>(a.qbias + (size_t)g * a.N + n0 + acol);
-    }
+    };
+    load_quad(0);
+    __builtin_amdgcn_sched_barrier(0);
     float amax = 0.f;
 #pragma unroll
     for (int sp_ = 0; sp_ < SP; ++sp_) {
@@ -685,6 +687,10 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a)
 #pragma unroll
     for (int t = 0; t < QUADS; ++t) {
       if (q0 + t >= nquads) break;  // wave-uniform
+      if (t + 1 < QUADS) {
+        load_quad(t + 1);
+        __builtin_amdgcn_sched_barrier(0);  // issued here, not where the compiler would like it
+      }
       // digit rows: MFMA column c reads row c (rows past 4 GS stay zero and are never used);
       // rows of ones: column c reads its group's
       const u4v* bp = reinterpret_cast<const u4v*>(xs_w + t * kGroupedQuadBytes + c * kLutRow + kb * 32);
