@@ -444,7 +444,7 @@ int hq_q3_rows_launch(const void* x, const int32_t* qweight, const float* scales
                       hipStream_t stream);
 int hq_q3_rows_groups_per_round(void);
 int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                       int K, int N, int M, int nsplit, float* partial, unsigned* counters, unsigned flags,
+                       int K, int N, int M, int nsplit, int rpw, float* partial, unsigned* counters, unsigned flags,
                        hipStream_t stream);
 int hq_q3_block_groups_per_round(void);
 
@@ -464,20 +464,37 @@ namespace {
 constexpr int kDigitBatchDefault = 8;
 constexpr size_t kBlockPartialRows = 8192;
 
+// How the kernel for 3 ... 8 rows cuts K: up to eight rounds of 4096 elements, one workgroup per round (as the
+// batch-1 kernel); beyond that as many workgroups per column tile as give every compute unit two, each taking
+// several rounds one after the other.
+void q3_block_split(const HqDevice* dev, int K, int N, int* nsplit, int* rpw) {
+  const int gpr = hq_q3_block_groups_per_round();
+  const int rounds = (K / 32 + gpr - 1) / gpr;
+  const int ntiles = (N + 63) / 64;
+  int ns = rounds;
+  if (rounds > 8) {
+    ns = 2 * dev->cus / ntiles;
+    if (ns < 1) ns = 1;
+    if (ns > rounds) ns = rounds;
+  }
+  *rpw = (rounds + ns - 1) / ns;
+  *nsplit = (rounds + *rpw - 1) / *rpw;
+}
+
 int q3_plan(const HqDevice* dev, int K, int N, int batch_M) {
   if (batch_M == 1) return HQ_Q3_PLAN_MATVEC;
   const int limit = hq_tune(HQ_TUNE_Q3_SMALL_BATCH, kDigitBatchDefault);  // 0: every batch takes the GEMM
   if (batch_M == 2 && limit >= 2) return HQ_Q3_PLAN_ROWS;
-  // 3 ... 8 rows: one single-round workgroup per 4096 elements of K, up to eight.  Five to eight rows take
+  // 3 ... 8 rows.  Five to eight rows take
   // two passes per workgroup, which beats the GEMM (7.8-12.4 us against 13-19 us at 4096 x 4096 ... 14336 x
   // 4096, 20.7-24.9 against 24.7 at K=8192, N=22016, 26.5-31.9 against 31.6 at K=28672, N=8192) except where
   // the GEMM's 128-column tiles fill the device without a K split (K=8192, N=28672: 27.8-31.1 against 25.3 us).
-  const int gpr = hq_q3_block_groups_per_round();
-  const size_t rounds = (size_t)(K / 32 + gpr - 1) / gpr;
-  const size_t groups = (size_t)((N + 63) / 64) * rounds;
+  int nsplit, rpw;
+  q3_block_split(dev, K, N, &nsplit, &rpw);
+  const size_t groups = (size_t)((N + 63) / 64) * nsplit;
   const size_t tiles128 = (size_t)(N + 127) / 128;
-  if (batch_M <= limit && batch_M <= 8 && rounds <= 8 && groups * batch_M <= kBlockPartialRows &&
-      (batch_M <= 4 || 8 * tiles128 < 7 * (size_t)dev->cus))
+  if (batch_M <= limit && batch_M <= 8 && groups * batch_M <= kBlockPartialRows &&
+      (batch_M <= 4 || (rpw == 1 && 8 * tiles128 < 7 * (size_t)dev->cus)))
     return HQ_Q3_PLAN_BLOCK;
   return HQ_Q3_PLAN_GEMM;
 }
@@ -574,9 +591,12 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
     }
     if (plan == HQ_Q3_PLAN_BLOCK) {
       Q3Split sp;
-      rc = q3_split_k(dev, K / 32, hq_q3_block_groups_per_round(), (N + 63) / 64, batch_M, true, fixed, stream, &sp);
+      int nsplit, rpw;
+      q3_block_split(dev, K, N, &nsplit, &rpw);
+      rc = q3_split_k(dev, K / 32, rpw * hq_q3_block_groups_per_round(), (N + 63) / 64, batch_M, true, fixed, stream, &sp);
       if (rc != HQ_OK) return rc;
-      return hq_q3_block_launch(x, qweight, scales, zeros, y, K, N, batch_M, sp.nsplit, sp.partial, sp.counters, flags,
+      if (sp.nsplit != nsplit) return HQ_ERR_BAD_SHAPE;
+      return hq_q3_block_launch(x, qweight, scales, zeros, y, K, N, batch_M, nsplit, rpw, sp.partial, sp.counters, flags,
                                 stream);
     }
     return hq_q3_gemm_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream, fixed);

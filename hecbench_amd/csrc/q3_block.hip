@@ -46,7 +46,8 @@ struct BlockArgs {
   float* partial;     // [tile][split][M][64] when K is split
   unsigned* counters; // [tile] arrival counters, zero between calls
   int K, N, M;
-  int nsplit;         // workgroups per column tile, one round of K each
+  int nsplit;         // workgroups per column tile
+  int rpw;            // rounds of K per workgroup
   unsigned flags;
 };
 
@@ -109,7 +110,8 @@ __device__ __forceinline__ constexpr int step_off(int s) {
 // PASSES = ceil(M / 4).  A pass leaves four registers per lane (its sixteen sums spread over the four lanes
 // of a row's columns); a wave's final sums re-use its operand area.  Two workgroups share a compute unit
 // (at most 128 registers, 76 KB of LDS): one's staging and reduction run under the other's loads.
-template <int PASSES>
+// MULTI: the workgroup takes several rounds of K (K beyond eight rounds; one pass only).
+template <int PASSES, bool MULTI>
 __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void q3_block_kernel(BlockArgs a) {
   // LDS: dig[kWaves][kWaveBytes] | wsum[kWaves][kWsumStride]
   extern __shared__ uint4 smem[];
@@ -121,8 +123,8 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, kb = lane >> 4;
   const int tile = blockIdx.x, split = blockIdx.y;
-  const int g_begin = split * kGroupsPerRound;
-  const int G = min(kGroupsPerRound, (a.K >> 5) - g_begin);  // k-groups of this workgroup
+  const int g_begin = split * a.rpw * kGroupsPerRound;
+  const int g_count = min(a.rpw * kGroupsPerRound, (a.K >> 5) - g_begin);  // k-groups of this workgroup
   const int M = a.M;
 
   // staging role: lane converts the eight consecutive activations 8*xq .. 8*xq+7 of k-group xkb of step xs
@@ -130,8 +132,27 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   const int tile_cols = min(64, a.N - tile * 64);  // multiple of 4
   const uint32_t col_off = (uint32_t)min(4 * c, tile_cols - 4) * 4u;
   const uint32_t row_bytes = (uint32_t)a.N * 4u;
-  const char* wbase = reinterpret_cast<const char*>(a.w) + (size_t)g_begin * 3 * row_bytes + (size_t)tile * 64 * 4;
-  const _Float16* xbase = a.x + (size_t)g_begin * 32;
+  char* dig_w = dig + wv * kWaveBytes;
+  unsigned char* sc_tab = reinterpret_cast<unsigned char*>(dig_w + kScaleOff);
+  float* red_w = reinterpret_cast<float*>(dig_w);
+  // MFMA column c carries term c % 4 of row c / 4 of the pass
+  const int crow = c >> 2, cterm = c & 3;
+  f4 keep[PASSES];
+  float rowsum[PASSES][kPassRows];  // uniform
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    keep[p] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int m = 0; m < kPassRows; ++m) rowsum[p][m] = 0.f;
+  }
+  constexpr uint32_t M0 = low3_mask(0), M1 = low3_mask(1), M2 = low3_mask(2);
+
+  // A workgroup's rounds run one after the other, nothing of the next round in flight during this one: two
+  // workgroups share the compute unit and one's loads run under the other's arithmetic.
+  for (int g0 = 0; g0 < (MULTI ? g_count : 1); g0 += kGroupsPerRound) {
+  const int G = min(kGroupsPerRound, g_count - g0);  // k-groups of this round
+  const char* wbase = reinterpret_cast<const char*>(a.w) + (size_t)(g_begin + g0) * 3 * row_bytes + (size_t)tile * 64 * 4;
+  const _Float16* xbase = a.x + (size_t)(g_begin + g0) * 32;
 
   // ---- the loads of the workgroup's round: the activation rows first (L2 hits: a compute unit returns its
   // loads in issue order, so the rows are there, and can be staged, while the weights still stream in from HBM)
@@ -166,14 +187,6 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   for (int s = 0; s < kEarly; ++s) load_step(s);
   __builtin_amdgcn_sched_barrier(0);
 
-  char* dig_w = dig + wv * kWaveBytes;
-  unsigned char* sc_tab = reinterpret_cast<unsigned char*>(dig_w + kScaleOff);
-  float* red_w = reinterpret_cast<float*>(dig_w);
-  // MFMA column c carries term c % 4 of row c / 4 of the pass
-  const int crow = c >> 2, cterm = c & 3;
-  f4 keep[PASSES];
-  constexpr uint32_t M0 = low3_mask(0), M1 = low3_mask(1), M2 = low3_mask(2);
-
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     // ---- stage the fp8 terms and scales of rows 4p .. 4p+3 -------------------------------------------
@@ -197,7 +210,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
       }
       const float gmax = quad_max(amax);  // the k-group's largest magnitude (its four lanes)
       const float total = wave_sum(asum);
-      if (lane == 0) wsum[wv * kWsumStride + kPassRows * p + m] = total;
+      rowsum[p][m] += total;
       // 2^E * max|x| lies in [2^-3, 2^-2): 64 ... 127 subnormal steps of the fp8 format.  fp16 magnitudes: E in -18 ... 21.
       int E = -3 - ((int)((__float_as_uint(gmax) >> 23) & 255u) - 127);
       E = gmax > 0.f ? max(-18, min(21, E)) : 0;
@@ -274,15 +287,20 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
       const float v0 = quad_sum(acc[q][0]), v1 = quad_sum(acc[q][1]), v2 = quad_sum(acc[q][2]), v3 = quad_sum(acc[q][3]);
       float v = (c & 2) ? ((c & 1) ? v3 : v2) : ((c & 1) ? v1 : v0);
       asm volatile("" : "+v"(v));  // selected here, not where it is stored (four candidates alive until then)
-      keep[p][q] = v;
+      keep[p][q] += v;
     }
     // the next pass rewrites, and the sums below overwrite, the operand and scales this pass's lanes have just read
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
   }
+  }  // rounds
 #pragma unroll
-  for (int p = 0; p < PASSES; ++p)
+  for (int p = 0; p < PASSES; ++p) {
     *reinterpret_cast<f4*>(red_w + (kPassRows * p + crow) * 64 + 4 * (4 * kb + cterm)) = keep[p];
+#pragma unroll
+    for (int m = 0; m < kPassRows; ++m)
+      if (lane == 0) wsum[wv * kWsumStride + kPassRows * p + m] = rowsum[p][m];
+  }
   __syncthreads();
 
   // ---- combine the waves, scale and zero --------------------------------------------------------------
@@ -343,14 +361,14 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   }
 }
 
-template <int PASSES>
+template <int PASSES, bool MULTI>
 int launch_block_t(const BlockArgs& a, hipStream_t stream) {
   const size_t smem = (size_t)kWaves * kWaveBytes + (size_t)kWaves * kWsumStride * 4 + 16;
   static const hipError_t attr =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_block_kernel<PASSES>),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_block_kernel<PASSES, MULTI>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
   if (attr != hipSuccess) return (int)attr;
-  hipLaunchKernelGGL((q3_block_kernel<PASSES>), dim3((a.N + 63) / 64, a.nsplit), dim3(kWaves * 64), smem, stream, a);
+  hipLaunchKernelGGL((q3_block_kernel<PASSES, MULTI>), dim3((a.N + 63) / 64, a.nsplit), dim3(kWaves * 64), smem, stream, a);
   return hq_launch_status();
 }
 
@@ -359,16 +377,19 @@ int launch_block_t(const BlockArgs& a, hipStream_t stream) {
 // k-groups one workgroup covers (its one round)
 int hq_q3_block_groups_per_round(void) { return kGroupsPerRound; }
 
-// 3 ... 8 fp16 activation rows; the caller has validated the arguments, set nsplit = ceil(K / 4096) and, for
-// nsplit > 1, provided nsplit * M * 64 floats of partial sums and one zeroed counter per column tile.
+// 3 ... 8 fp16 activation rows; the caller has validated the arguments, cut K into nsplit ranges of rpw rounds
+// of 4096 elements and, for nsplit > 1, provided nsplit * M * 64 floats of partial sums per column tile and
+// one zeroed counter per column tile.
 int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                       int K, int N, int M, int nsplit, float* partial, unsigned* counters, unsigned flags,
+                       int K, int N, int M, int nsplit, int rpw, float* partial, unsigned* counters, unsigned flags,
                        hipStream_t stream) {
-  if (M < 1 || M > kMaxRows || nsplit != (K / 32 + kGroupsPerRound - 1) / kGroupsPerRound) return HQ_ERR_BAD_SHAPE;
+  const int rounds = (K / 32 + kGroupsPerRound - 1) / kGroupsPerRound;
+  if (M < 1 || M > kMaxRows || rpw < 1 || nsplit != (rounds + rpw - 1) / rpw) return HQ_ERR_BAD_SHAPE;
   BlockArgs a;
   a.x = reinterpret_cast<const _Float16*>(x);
   a.w = reinterpret_cast<const uint32_t*>(qweight);
   a.scales = scales; a.zeros = zeros; a.y = y; a.partial = partial; a.counters = counters; a.K = K; a.N = N; a.M = M;
-  a.nsplit = nsplit; a.flags = flags & (HQ_FLAG_ACCUMULATE | HQ_FLAG_STRICT_FENCES);
-  return M <= kPassRows ? launch_block_t<1>(a, stream) : launch_block_t<2>(a, stream);
+  a.nsplit = nsplit; a.rpw = rpw; a.flags = flags & (HQ_FLAG_ACCUMULATE | HQ_FLAG_STRICT_FENCES);
+  if (rpw > 1) return M <= kPassRows ? launch_block_t<1, true>(a, stream) : HQ_ERR_BAD_SHAPE;
+  return M <= kPassRows ? launch_block_t<1, false>(a, stream) : launch_block_t<2, false>(a, stream);
 }

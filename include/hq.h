@@ -133,8 +133,9 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  *     by side in the matrix-core operand (28-bit fixed point relative to the largest
  *     magnitude among each 512 consecutive activations of a row: exact for fp16
  *     entries within 2^17 of it);
- *   - batches 3 ... 8 with K <= 32768 (5 ... 8 unless N / 128 is at least 7/8 of the
- *     compute units): the matvec's kernel, four rows side by side;
+ *   - batches 3 ... 4, and 5 ... 8 unless N / 128 is at least 7/8 of the compute units or
+ *     K is so long that a workgroup takes several rounds of 4096: the matvec's kernel,
+ *     four rows side by side;
  *     every activation enters with an error of at most 2^-19 of the largest magnitude
  *     among its 32 neighbours (exactly, if within 2^8 of it);
  *   - everything else: the MFMA GEMM path, which pre-scales every activation row by a
@@ -153,7 +154,7 @@ int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float
 #define HQ_Q3_PLAN_MATVEC 0 /* batch_M == 1 */
 #define HQ_Q3_PLAN_ROWS 1   /* batch_M == 2 on the matvec's digit kernel */
 #define HQ_Q3_PLAN_GEMM 2   /* batched MFMA GEMM */
-#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 3 ... 8, K <= 32768: the matvec's kernel, four rows per pass */
+#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 3 ... 8: the matvec's kernel, four rows per pass */
 int hq_q3_matvec_plan(int K, int N, int batch_M);
 
 /*

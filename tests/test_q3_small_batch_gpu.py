@@ -227,9 +227,10 @@ def test_small_batches_on_the_gemm(hq, oracle, tunable, M, K, N):
 
 
 # one and two passes of four rows, full and partly filled; K of one round, a K the rounds do not divide
-# (two workgroups per tile) and eight rounds; N with a 4-column last tile
+# (two workgroups per tile), eight rounds, and more (workgroups that take several rounds, the last one partly
+# filled); N with a 4-column last tile
 _BLOCK_CASES = [(M, K, N) for (K, N) in [(4128, 1028), (160, 16388)] for M in (3, 4, 5, 6, 7, 8)] + \
-               [(6, 32768, 260), (8, 16384, 196), (4, 8192, 4096)]
+               [(6, 32768, 260), (8, 16384, 196), (4, 8192, 4096), (4, 36864, 1028), (3, 49184, 260)]
 
 
 @pytest.mark.parametrize("M,K,N", _BLOCK_CASES)
@@ -252,11 +253,13 @@ def test_block_kernel_vs_oracle(hq, oracle, M, K, N):
 
 
 def test_block_kernel_plan_limits(hq, tunable):
-    """Beyond eight rounds of K, beyond 8 rows, for 5 ... 8 rows where the GEMM's 128-column tiles fill the device,
+    """Beyond 8 rows, for 5 ... 8 rows beyond eight rounds of K or where the GEMM's 128-column tiles fill the device,
     or with more partial sums than the fixed scratch of the entry point that allocates nothing holds, the batch
     takes the GEMM; HQ_Q3_SMALL_BATCH lowers the limit.  (The counts below are for 256 compute units.)"""
     assert _plan(32768, 256, 8) == PLAN_BLOCK
-    assert _plan(32800, 256, 8) == PLAN_GEMM
+    assert _plan(32800, 256, 8) == PLAN_BLOCK         # nine rounds, four tiles: still one workgroup per round
+    assert _plan(49152, 12288, 8) == PLAN_GEMM        # twelve rounds, 192 tiles: six rounds per workgroup, one pass only
+    assert _plan(49152, 12288, 4) == PLAN_BLOCK
     assert _plan(4096, 4096, 8) == PLAN_BLOCK
     assert _plan(4096, 4096, 9) == PLAN_GEMM
     assert _plan(8192, 28672, 4) == PLAN_BLOCK        # one pass per workgroup: always
