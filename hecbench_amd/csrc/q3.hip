@@ -115,7 +115,10 @@ __device__ __forceinline__ constexpr int step_off(int s) {
   return s * kStepBytes + (s & 1) * 32 + ((s >> 1) & 1) * 128;
 }
 
-template <int WAVES, int STEPS, bool XF16, bool MULTI>
+// ROUNDS: 0 one round per workgroup, 1 several with a round's loads issued at once one round ahead, 2 several
+// with only the first step's loads at the top of a round and step s + 1 of the next round before the
+// arithmetic of step s.
+template <int WAVES, int STEPS, bool XF16, int ROUNDS>
 __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   // LDS: dig[WAVES][STEPS * kStepBytes] | red[WAVES][8][kRedStride] | part[WAVES][64] | xsum[WAVES]
   extern __shared__ uint4 smem[];
@@ -154,6 +157,8 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   const uint32_t row_bytes = (uint32_t)a.N * 4u;
   const char* wbase = reinterpret_cast<const char*>(a.w) + ((size_t)(3 * g_begin) * row_stride + (size_t)tile * 64) * 4;
   constexpr int GPR = WAVES * 4 * STEPS;  // k-groups per round
+  constexpr bool MULTI = ROUNDS != 0;
+  constexpr int kNextEarly = ROUNDS == 2 ? 1 : STEPS;  // steps of the next round loaded at the top of a round
   const int rounds = MULTI ? (g_count + GPR - 1) / GPR : 1;  // !MULTI: the host sized gpw <= GPR
 
   // No global load sits under a branch (addresses are clamped instead), so the compiler can count
@@ -195,7 +200,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
         for (int j = 0; j < 4; ++j) { xr[p][j] = lo[j]; xr[p][4 + j] = hi[j]; }
       }
     }
-    load_steps(r, wreg, 0, kEarly);
+    load_steps(r, wreg, 0, (MULTI && r > 0) ? kNextEarly : kEarly);
   };
 
   char* dig_w = dig + wv * (STEPS * kStepBytes);
@@ -286,6 +291,10 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
       if (!MULTI && s + kEarly < STEPS) {
         load_steps(0, wreg, s + kEarly, s + kEarly + 1);
         __builtin_amdgcn_sched_barrier(0);  // issued here, not where the compiler would like it
+      }
+      if (ROUNDS == 2 && s + kNextEarly < STEPS && r + 1 < rounds) {
+        load_steps(r + 1, wreg_next, s + kNextEarly, s + kNextEarly + 1);
+        __builtin_amdgcn_sched_barrier(0);
       }
       if ((r * STEPS + s) * (WAVES * 4) + wv * 4 >= g_count) continue;  // wave-uniform
       // MFMA columns 9..15 are never read: they re-use row 8
@@ -412,26 +421,33 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
   }
 }
 
-template <int WAVES, int STEPS, bool XF16, bool MULTI>
+template <int WAVES, int STEPS, bool XF16, int ROUNDS>
 int launch_matvec_t(const Q3Args& a, int ntiles, hipStream_t stream) {
   const size_t smem = (size_t)WAVES * STEPS * kStepBytes + (size_t)WAVES * 8 * kRedStride * 4 + (size_t)WAVES * 64 * 4 +
                       (size_t)WAVES * 4 + 16;
   static const hipError_t attr =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_matvec_kernel<WAVES, STEPS, XF16, MULTI>),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_matvec_kernel<WAVES, STEPS, XF16, ROUNDS>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
   if (attr != hipSuccess) return (int)attr;
-  hipLaunchKernelGGL((q3_matvec_kernel<WAVES, STEPS, XF16, MULTI>), dim3(ntiles, a.nsplit), dim3(WAVES * 64), smem,
+  hipLaunchKernelGGL((q3_matvec_kernel<WAVES, STEPS, XF16, ROUNDS>), dim3(ntiles, a.nsplit), dim3(WAVES * 64), smem,
                      stream, a);
   return hq_launch_status();
 }
 template <int WAVES, int STEPS>
-int launch_matvec(const Q3Args& a, int ntiles, hipStream_t stream) {
+int launch_matvec(const Q3Args& a, int ntiles, int cus, hipStream_t stream) {
+  // Several rounds per workgroup: with a workgroup on every compute unit the next round's loads go out a
+  // step at a time (K=36864, N=16384 41.0 -> 37.4 us, K=40960, N=8192 25.9 -> 23.6, K=65536, N=4096 22.6 -> 20.7);
+  // with compute units to spare a whole round at once keeps more in flight (K=49152, N=12288, 192 tiles: 42.2
+  // against 46.9 us).  The default workgroup only: the other shapes are for sweeps.
   const bool multi = a.gpw > WAVES * 4 * STEPS;
+  const bool ahead = WAVES == 8 && STEPS == 4 && ntiles * a.nsplit >= cus;
+  if (WAVES == 8 && STEPS == 4 && multi && ahead)
+    return a.x_f16 ? launch_matvec_t<8, 4, true, 2>(a, ntiles, stream) : launch_matvec_t<8, 4, false, 2>(a, ntiles, stream);
   if (a.x_f16)
-    return multi ? launch_matvec_t<WAVES, STEPS, true, true>(a, ntiles, stream)
-                 : launch_matvec_t<WAVES, STEPS, true, false>(a, ntiles, stream);
-  return multi ? launch_matvec_t<WAVES, STEPS, false, true>(a, ntiles, stream)
-               : launch_matvec_t<WAVES, STEPS, false, false>(a, ntiles, stream);
+    return multi ? launch_matvec_t<WAVES, STEPS, true, 1>(a, ntiles, stream)
+                 : launch_matvec_t<WAVES, STEPS, true, 0>(a, ntiles, stream);
+  return multi ? launch_matvec_t<WAVES, STEPS, false, 1>(a, ntiles, stream)
+               : launch_matvec_t<WAVES, STEPS, false, 0>(a, ntiles, stream);
 }
 
 }  // namespace
@@ -625,7 +641,7 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   a.y = y; a.partial = sp.partial; a.counters = sp.counters; a.K = K; a.N = N; a.gpw = sp.gpw;
   a.nsplit = sp.nsplit; a.x_f16 = (x_dtype == HQ_DTYPE_F16); a.flags = flags;
 #define HQ_Q3_CASE(W, S) \
-  if (waves == W && steps == S) return launch_matvec<W, S>(a, ntiles, stream);
+  if (waves == W && steps == S) return launch_matvec<W, S>(a, ntiles, dev->cus, stream);
   HQ_Q3_CASE(16, 1)
   HQ_Q3_CASE(8, 1) HQ_Q3_CASE(8, 2) HQ_Q3_CASE(8, 4)
   HQ_Q3_CASE(4, 1) HQ_Q3_CASE(4, 2) HQ_Q3_CASE(4, 4) HQ_Q3_CASE(4, 8)

@@ -162,6 +162,26 @@ def test_default_k_split_on_long_k(hq, oracle, tunable, K, N):
     assert rel_err(y, _run(hq, x, mat, scales, zeros)) <= 1e-4
 
 
+@pytest.mark.parametrize("K,N,x_dtype", [(36864, 16384, np.float32), (33792, 16388, np.float16), (36864, 4096, np.float32)])
+def test_more_than_eight_rounds_of_k(hq, oracle, tunable, K, N, x_dtype):
+    """Workgroups that walk several rounds of K: a workgroup on every compute unit (256 and 257 tiles, the last
+    one 4 columns wide: the next round's loads go out a step at a time), a K the rounds do not divide, and
+    64 tiles with K split four ways.  Sampled columns against the oracle, every column against a different
+    split, the same bits on a second call."""
+    rng = np.random.default_rng(K + N)
+    mat = rng.integers(-2 ** 31, 2 ** 31, size=(3 * K // 32, N), dtype=np.int64).astype(np.int32)
+    scales = rng.uniform(0.005, 0.02, size=N).astype(np.float32)
+    zeros = (scales * rng.integers(3, 5, size=N)).astype(np.float32)
+    x = rng.standard_normal(K).astype(x_dtype)
+    y = _run(hq, x, mat, scales, zeros)
+    assert np.array_equal(y, _run(hq, x, mat, scales, zeros))
+    cols = np.unique(np.concatenate([np.arange(0, 68), np.arange(N - 68, N), rng.integers(0, N, 64)]))
+    ref = oracle.q3_matvec_f64(x.astype(np.float32), np.ascontiguousarray(mat[:, cols]), scales[cols], zeros[cols])
+    assert rel_err(y[cols], ref) <= 1e-4
+    tunable("HQ_Q3_KSPLIT", 3)
+    assert rel_err(y, _run(hq, x, mat, scales, zeros)) <= 2e-4   # two results, each within 1e-4 of the exact one
+
+
 def test_rejects_bad_arguments(hq):
     import torch
     dev = torch.device("cuda:0")
