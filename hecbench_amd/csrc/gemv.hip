@@ -177,10 +177,17 @@ int launch_gemv(const void* mat, const void* vec, void* res, int rows, int n, fl
   a.zp = (float)(_Float16)zp;
   // several rows per wave (the vector piece is loaded and prepared once for them) once there are
   // enough rows to fill the chip with such waves
+  // (int4 reads four times as many bytes of the vector per byte of the matrix as fp16: rows per wave pay
+  // there even when they leave only eight waves per compute unit - 8192 x 28672: 33.1 us with one row per
+  // wave, 25.0 with two, 20.6 with four; fp16 at 4096 x 16384: 23.7 us with one row, 28.0 with two)
   constexpr int RMAX = MODE == kI4 ? 4 : 2;
-  if (rows >= dev->cus * 16 * RMAX) {
+  constexpr int kMinWaves = MODE == kI4 ? 8 : 16;  // per compute unit
+  if (rows >= dev->cus * kMinWaves * RMAX) {
     const int waves = (rows + RMAX - 1) / RMAX;
     hipLaunchKernelGGL((gemv_kernel<MODE, RMAX>), dim3((waves + 3) / 4), dim3(256), 0, stream, a);
+  } else if (RMAX > 2 && rows >= dev->cus * kMinWaves * 2) {
+    const int waves = (rows + 1) / 2;
+    hipLaunchKernelGGL((gemv_kernel<MODE, 2>), dim3((waves + 3) / 4), dim3(256), 0, stream, a);
   } else {
     hipLaunchKernelGGL((gemv_kernel<MODE, 1>), dim3((rows + 3) / 4), dim3(256), 0, stream, a);
   }
