@@ -9,6 +9,9 @@
 //   b1 = fp8(v), b2 = fp8(16 (v - b1)), b3 = fp8(16 (16 (v - b1) - b2)), b4 likewise,
 // every term takes the next four significant bits of what is left, but never below the fp8 format's
 // subnormal step 2^-9: in units of that step the terms are integers up to 127 with four significant bits.
+// (All of it in packed fp16, two activations per instruction: v_cvt_scalef32_pk_fp8_f16 divides by the scale
+// 2^-E / 16^t while it converts, v_cvt_scalef32_pk_f16_fp8 multiplies by it on the way back, and what is left of
+// an fp16 number after its rounded leading part is an fp16 number again, exactly.)
 // Products with the 3-bit codes and their sums over the 128 elements of an MFMA stay below 2^17 in those
 // units, so the matrix core adds them exactly, as it does the nibbles of q3.hip.  Four terms reach 19 bits
 // below the k-group's largest magnitude (an fp16 activation within 2^8 of it enters exactly, one 2^12 below
@@ -32,10 +35,12 @@
 
 namespace {
 
-typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+typedef short s2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ h2v as_h2(uint32_t v) { return __builtin_bit_cast(h2v, v); }
 
 struct BlockArgs {
   const _Float16* x;  // [M][K]
@@ -80,18 +85,6 @@ constexpr uint32_t low3_mask(int word) {
   return m;
 }
 
-typedef float f2 __attribute__((ext_vector_type(2)));
-// Four floats to four fp8 (e4m3, round to nearest even) bytes of one register, and what the bytes are worth.
-__device__ __forceinline__ uint32_t to_fp8x4(const float (&v)[4]) {
-  int w = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
-  w = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w, true);
-  return (uint32_t)w;
-}
-__device__ __forceinline__ void from_fp8x4(uint32_t w, float (&v)[4]) {
-  const f2 lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
-  v[0] = lo.x; v[1] = lo.y; v[2] = hi.x; v[3] = hi.y;
-}
-
 constexpr int kWaves = 8, kSteps = 4;
 constexpr int kGroupsPerRound = kWaves * 4 * kSteps;  // k-groups of one workgroup
 constexpr int kRowBytes = 144;                // one B operand row (4 lane quarters x 32 B) plus 16 B: rows start 4 banks apart
@@ -111,12 +104,16 @@ __device__ __forceinline__ constexpr int step_off(int s) {
 // of a row's columns); a wave's final sums re-use its operand area.  Two workgroups share a compute unit
 // (at most 128 registers, 76 KB of LDS): one's staging and reduction run under the other's loads.
 // MULTI: the workgroup takes several rounds of K (K beyond eight rounds; one pass only).
+// (Staging both passes' operands, in areas of their own, before the first MFMA - possible where a launch has
+// at most one workgroup per compute unit - changes nothing: a pass costs its ~450 VALU instructions per wave
+// wherever they stand.)
 template <int PASSES, bool MULTI>
 __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void q3_block_kernel(BlockArgs a) {
-  // LDS: dig[kWaves][kWaveBytes] | wsum[kWaves][kWsumStride]
+  // LDS: dig[kWaves][kAreaBytes] | wsum[kWaves][kWsumStride]
   extern __shared__ uint4 smem[];
+  constexpr int kAreaBytes = kWaveBytes;
   char* dig = reinterpret_cast<char*>(smem);
-  float* wsum = reinterpret_cast<float*>(dig + kWaves * kWaveBytes);
+  float* wsum = reinterpret_cast<float*>(dig + kWaves * kAreaBytes);
   static_assert(kSteps * kStepBytes >= kMaxRows * 64 * 4, "a wave's digit area must hold its final sums");
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -132,9 +129,8 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   const int tile_cols = min(64, a.N - tile * 64);  // multiple of 4
   const uint32_t col_off = (uint32_t)min(4 * c, tile_cols - 4) * 4u;
   const uint32_t row_bytes = (uint32_t)a.N * 4u;
-  char* dig_w = dig + wv * kWaveBytes;
-  unsigned char* sc_tab = reinterpret_cast<unsigned char*>(dig_w + kScaleOff);
-  float* red_w = reinterpret_cast<float*>(dig_w);
+  char* dig_w0 = dig + wv * kAreaBytes;
+  float* red_w = reinterpret_cast<float*>(dig_w0);
   // MFMA column c carries term c % 4 of row c / 4 of the pass
   const int crow = c >> 2, cterm = c & 3;
   f4 keep[PASSES];
@@ -187,9 +183,10 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   for (int s = 0; s < kEarly; ++s) load_step(s);
   __builtin_amdgcn_sched_barrier(0);
 
-#pragma unroll
-  for (int p = 0; p < PASSES; ++p) {
-    // ---- stage the fp8 terms and scales of rows 4p .. 4p+3 -------------------------------------------
+  // ---- stage the fp8 terms and scales of rows 4p .. 4p+3 ---------------------------------------------
+  auto stage = [&](int p) {
+    char* dig_w = dig_w0;
+    unsigned char* sc_tab = reinterpret_cast<unsigned char*>(dig_w + kScaleOff);
 #pragma unroll
     for (int m = 0; m < kPassRows; ++m) {
       if (p == 0 && m > 0) {
@@ -199,54 +196,60 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
         __builtin_amdgcn_sched_barrier(0);
       }
       if (kPassRows * p + m >= M) continue;  // uniform; the operand columns of a missing row feed result columns nobody reads
-      const h8 h = __builtin_bit_cast(h8, xraw[p][m]);
-      float xr[8];
-      float amax = 0.f, asum = 0.f;
+      // The lane's eight activations stay fp16, in pairs (0, 2), (4, 6), (1, 3), (5, 7): even / odd elements of the
+      // k-group go to neighbouring lane quarters of the fp8 operand (see q3.hip), and the conversions below take
+      // and give pairs.
+      const u4v raw = xraw[p][m];
+      const uint32_t w0 = live ? raw.x : 0u, w1 = live ? raw.y : 0u, w2 = live ? raw.z : 0u, w3 = live ? raw.w : 0u;
+      h2v pr[4] = {as_h2(__builtin_amdgcn_perm(w1, w0, 0x05040100u)), as_h2(__builtin_amdgcn_perm(w3, w2, 0x05040100u)),
+                   as_h2(__builtin_amdgcn_perm(w1, w0, 0x07060302u)), as_h2(__builtin_amdgcn_perm(w3, w2, 0x07060302u))};
+      const h2v one = {(_Float16)1.f, (_Float16)1.f};
+      float asum = 0.f;
+      h2v mx = {(_Float16)0.f, (_Float16)0.f};
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        xr[j] = live ? (float)h[j] : 0.f;
-        amax = fmaxf(amax, fabsf(xr[j]));
-        asum += xr[j];
+      for (int i = 0; i < 4; ++i) {
+        asum = __builtin_amdgcn_fdot2(pr[i], one, asum, false);
+        mx = __builtin_elementwise_max(mx, __builtin_elementwise_abs(pr[i]));
       }
+      const float amax = fmaxf((float)mx[0], (float)mx[1]);
       const float gmax = quad_max(amax);  // the k-group's largest magnitude (its four lanes)
       const float total = wave_sum(asum);
       rowsum[p][m] += total;
       // 2^E * max|x| lies in [2^-3, 2^-2): 64 ... 127 subnormal steps of the fp8 format.  fp16 magnitudes: E in -18 ... 21.
       int E = -3 - ((int)((__float_as_uint(gmax) >> 23) & 255u) - 127);
       E = gmax > 0.f ? max(-18, min(21, E)) : 0;
-      const float scaleE = __uint_as_float((uint32_t)(E + 127) << 23);
-      // even / odd elements of the k-group go to neighbouring lane quarters of the fp8 operand (see q3.hip)
-      float ve[4], vo[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        ve[j] = xr[2 * j] * scaleE;
-        vo[j] = xr[2 * j + 1] * scaleE;
-      }
       char* dst = dig_w + step_off(xs) + (kTerms * m) * kRowBytes + (xkb & 1) * 64 + (xkb >> 1) * 16 + xq * 4;
+      // Term t is fp8(what is left * 2^E * 16^t): the conversion divides by the scale 2^-E / 16^t itself, and the
+      // conversion back multiplies by it, so what is left, x - b1 - b2 - ..., stays an fp16 number in the
+      // activation's own units (exactly: every term is the rounded leading part of it).
+      uint32_t sbits = (uint32_t)(127 - E) << 23;
 #pragma unroll
       for (int t = 0; t < kTerms; ++t) {
-        const uint32_t be = to_fp8x4(ve), bo = to_fp8x4(vo);
-        *reinterpret_cast<uint32_t*>(dst + t * kRowBytes) = be;
-        *reinterpret_cast<uint32_t*>(dst + t * kRowBytes + 32) = bo;
-        if (t + 1 < kTerms) {  // what the term left out (at most half its last place), sixteen times: exact in fp32
-          float fe[4], fo[4];
-          from_fp8x4(be, fe);
-          from_fp8x4(bo, fo);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            ve[j] = (ve[j] - fe[j]) * 16.f;
-            vo[j] = (vo[j] - fo[j]) * 16.f;
-          }
+        const float scale = __uint_as_float(sbits);
+        s2v be = {0, 0}, bo = {0, 0};
+        be = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(be, pr[0], scale, false);
+        be = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(be, pr[1], scale, true);
+        bo = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(bo, pr[2], scale, false);
+        bo = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(bo, pr[3], scale, true);
+        const uint32_t ue = __builtin_bit_cast(uint32_t, be), uo = __builtin_bit_cast(uint32_t, bo);
+        *reinterpret_cast<uint32_t*>(dst + t * kRowBytes) = ue;
+        *reinterpret_cast<uint32_t*>(dst + t * kRowBytes + 32) = uo;
+        if (t + 1 < kTerms) {
+          pr[0] -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(ue, scale, false);
+          pr[1] -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(ue, scale, true);
+          pr[2] -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(uo, scale, false);
+          pr[3] -= __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(uo, scale, true);
+          sbits -= 4u << 23;
         }
       }
       // E8M0 scale of term 0: 2^-E for the k-group's power of two, 2^3 for the unit of the fp6 operand (code / 8)
       if (xq == 0) sc_tab[(m * 4 + xkb) * 4 + xs] = (unsigned char)(127 + 3 - E);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-
-    // ---- mask + MFMA -----------------------------------------------------------------------
+  };
+  // ---- mask + MFMA -------------------------------------------------------------------------
+  auto multiply = [&](int p) {
+    char* dig_w = dig_w0;
+    unsigned char* sc_tab = reinterpret_cast<unsigned char*>(dig_w + kScaleOff);
     // The matrix-core operand of the weights (six registers per sixteen MFMAs) is rebuilt in every pass: kept
     // across passes it would double the registers the weights take.  The empty statement hides from the compiler
     // that the weights are the same as in the last pass.
@@ -289,6 +292,14 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
       asm volatile("" : "+v"(v));  // selected here, not where it is stored (four candidates alive until then)
       keep[p][q] += v;
     }
+  };
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    stage(p);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    multiply(p);
     // the next pass rewrites, and the sums below overwrite, the operand and scales this pass's lanes have just read
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_wave_barrier();
@@ -312,7 +323,7 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
     float qx = 0.f, xsum = 0.f;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
-      const float* rw = reinterpret_cast<const float*>(dig + w * kWaveBytes);
+      const float* rw = reinterpret_cast<const float*>(dig + w * kAreaBytes);
       qx += rw[m * 64 + col];
       xsum += wsum[w * kWsumStride + m];
     }
@@ -366,7 +377,7 @@ int launch_block_t(const BlockArgs& a, hipStream_t stream) {
   const size_t smem = (size_t)kWaves * kWaveBytes + (size_t)kWaves * kWsumStride * 4 + 16;
   static const hipError_t attr =
       hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_block_kernel<PASSES, MULTI>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (attr != hipSuccess) return (int)attr;
   hipLaunchKernelGGL((q3_block_kernel<PASSES, MULTI>), dim3((a.N + 63) / 64, a.nsplit), dim3(kWaves * 64), smem, stream, a);
   return hq_launch_status();
