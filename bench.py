@@ -212,7 +212,7 @@ def bench_configs(steps, warmup, windows):
                                                        "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                                                        "frac": round(tf / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None}
     del mats, Ag, og
-    # the headline shape at batches 2, 4 and 8 (extension: one pass over the weights for all rows, 34 rotated buffers)
+    # the headline shape at batches 4 and 8 (extension: one pass over the weights for all rows, 34 rotated buffers)
     Ks, Ns = K, N
     nb = 34
     mats = [torch.randint(-2 ** 31, 2 ** 31 - 1, (3 * Ks // 32, Ns), dtype=torch.int32, device=dev, generator=g)
@@ -220,7 +220,7 @@ def bench_configs(steps, warmup, windows):
     ss = torch.empty(Ns, device=dev).uniform_(0.005, 0.02, generator=g)
     zs = ss * torch.randint(3, 5, (Ns,), device=dev, generator=g).float()
     pm = [vp(m) for m in mats]
-    for Ms in (2, 4, 8):
+    for Ms in (4, 8):
         As = torch.randn(Ms, Ks, device=dev, generator=g).half()
         os_ = torch.empty(Ms, Ns, device=dev)
         pA, pss, pzs, pos = vp(As), vp(ss), vp(zs), vp(os_)
@@ -231,7 +231,7 @@ def bench_configs(steps, warmup, windows):
               "GPTQ 3-bit K=4096 N=11008, %d fp16 activation rows in one call, 34 rotated weight buffers (575 MB)" % Ms,
               3 * Ks // 32 * Ns * 4 + 2 * Ns * 4 + Ms * Ks * 2 + Ms * Ns * 4, secs, steps, "q3_batch%d_4096x11008" % Ms,
               dtype="fp6 x fp8 MFMA, exact integer sums, f32 out",
-              kernel={1: "two rows per pass", 2: "batched GEMM", 3: "four rows per pass"}.get(plan, str(plan)))
+              kernel={2: "batched GEMM", 3: "four rows per pass"}.get(plan, str(plan)))
     del mats
     return out
 

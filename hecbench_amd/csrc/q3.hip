@@ -455,10 +455,6 @@ int launch_matvec(const Q3Args& a, int ntiles, int cus, hipStream_t stream) {
 int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros,
                       float* y, int K, int N, int M, unsigned flags, hipStream_t stream, const HqQ3Scratch* fixed);
 
-int hq_q3_rows_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                      int K, int N, int gpw, int nsplit, float* partial, unsigned* counters, unsigned flags,
-                      hipStream_t stream);
-int hq_q3_rows_groups_per_round(void);
 int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
                        int K, int N, int M, int nsplit, int rpw, float* partial, unsigned* counters, unsigned flags,
                        hipStream_t stream);
@@ -475,15 +471,15 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(unsigned* p, int n) {
 
 namespace {
 // Largest batch the matvec-like kernels take by default, and the most partial-sum rows (tiles x splits x batch)
-// the kernel for 3 ... 8 rows may need: what the fixed scratch of the entry point that allocates nothing holds,
+// the kernel for 2 ... 8 rows may need: what the fixed scratch of the entry point that allocates nothing holds,
 // applied to every caller so that both entry points run the same kernel on the same shape.
 constexpr int kDigitBatchDefault = 8;
 constexpr size_t kBlockPartialRows = 8192;
 
-// How the kernel for 3 ... 8 rows cuts K: up to eight rounds of 4096 elements, one workgroup per round (as the
+// How the kernel for 2 ... 8 rows cuts K: up to eight rounds of 4096 elements, one workgroup per round (as the
 // batch-1 kernel); beyond that as many workgroups per column tile as give every compute unit two, each taking
 // several rounds one after the other.
-void q3_block_split(const HqDevice* dev, int K, int N, int* nsplit, int* rpw) {
+void q3_block_split(const HqDevice* dev, int K, int N, int batch_M, int* nsplit, int* rpw) {
   const int gpr = hq_q3_block_groups_per_round();
   const int rounds = (K / 32 + gpr - 1) / gpr;
   const int ntiles = (N + 63) / 64;
@@ -493,6 +489,8 @@ void q3_block_split(const HqDevice* dev, int K, int N, int* nsplit, int* rpw) {
     if (ns < 1) ns = 1;
     if (ns > rounds) ns = rounds;
   }
+  // no more partial-sum rows than the fixed scratch holds (very wide matrices: fewer, longer ranges of K)
+  while (ns > 1 && (size_t)ntiles * ns * batch_M > kBlockPartialRows) --ns;
   *rpw = (rounds + ns - 1) / ns;
   *nsplit = (rounds + *rpw - 1) / *rpw;
 }
@@ -500,16 +498,15 @@ void q3_block_split(const HqDevice* dev, int K, int N, int* nsplit, int* rpw) {
 int q3_plan(const HqDevice* dev, int K, int N, int batch_M) {
   if (batch_M == 1) return HQ_Q3_PLAN_MATVEC;
   const int limit = hq_tune(HQ_TUNE_Q3_SMALL_BATCH, kDigitBatchDefault);  // 0: every batch takes the GEMM
-  if (batch_M == 2 && limit >= 2) return HQ_Q3_PLAN_ROWS;
-  // 3 ... 8 rows.  Five to eight rows take
+  // 2 ... 8 rows.  Five to eight rows take
   // two passes per workgroup, which beats the GEMM (7.8-12.4 us against 13-19 us at 4096 x 4096 ... 14336 x
   // 4096, 20.7-24.9 against 24.7 at K=8192, N=22016, 26.5-31.9 against 31.6 at K=28672, N=8192) except where
   // the GEMM's 128-column tiles fill the device without a K split (K=8192, N=28672: 27.8-31.1 against 25.3 us).
   int nsplit, rpw;
-  q3_block_split(dev, K, N, &nsplit, &rpw);
+  q3_block_split(dev, K, N, batch_M, &nsplit, &rpw);
   const size_t groups = (size_t)((N + 63) / 64) * nsplit;
   const size_t tiles128 = (size_t)(N + 127) / 128;
-  if (batch_M <= limit && batch_M <= 8 && groups * batch_M <= kBlockPartialRows &&
+  if (batch_M <= limit && batch_M <= 8 && (nsplit == 1 || groups * batch_M <= kBlockPartialRows) &&
       (batch_M <= 4 || (rpw == 1 && 8 * tiles128 < 7 * (size_t)dev->cus)))
     return HQ_Q3_PLAN_BLOCK;
   return HQ_Q3_PLAN_GEMM;
@@ -598,17 +595,10 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
     // Small batches ride on the matvec's digit kernels (one pass over the weights, one launch); everything
     // else takes the batched GEMM.
     const int plan = q3_plan(dev, K, N, batch_M);
-    if (plan == HQ_Q3_PLAN_ROWS) {
-      Q3Split sp;
-      rc = q3_split_k(dev, K / 32, hq_q3_rows_groups_per_round(), (N + 63) / 64, 2, false, fixed, stream, &sp);
-      if (rc != HQ_OK) return rc;
-      return hq_q3_rows_launch(x, qweight, scales, zeros, y, K, N, sp.gpw, sp.nsplit, sp.partial, sp.counters, flags,
-                               stream);
-    }
     if (plan == HQ_Q3_PLAN_BLOCK) {
       Q3Split sp;
       int nsplit, rpw;
-      q3_block_split(dev, K, N, &nsplit, &rpw);
+      q3_block_split(dev, K, N, batch_M, &nsplit, &rpw);
       rc = q3_split_k(dev, K / 32, rpw * hq_q3_block_groups_per_round(), (N + 63) / 64, batch_M, true, fixed, stream, &sp);
       if (rc != HQ_OK) return rc;
       if (sp.nsplit != nsplit) return HQ_ERR_BAD_SHAPE;

@@ -1,8 +1,9 @@
-// GPTQ 3-bit product for small batches (3 ... 8 activation rows) on the matvec's matrix-core kernel, gfx950.
+// GPTQ 3-bit product for small batches (2 ... 8 activation rows) on the matvec's matrix-core kernel, gfx950.
 //
-// q3.hip (batch 1) and q3_rows.hip (batch 2) carry the activations as fixed point relative to the largest
-// magnitude a wave sees in a round, eight or seven 4-bit digits per activation, so one matrix-core pass over
-// the weights serves one or two rows.  Here every k-group (32 consecutive activations of a row) has its own
+// q3.hip (batch 1) carries the activations as fixed point relative to the largest magnitude a wave sees in a
+// round, eight 4-bit digits per activation, so one matrix-core pass over the weights serves one row (a
+// two-row kernel with seven sign-magnitude digits was the first small-batch kernel; this one took its place
+// when it ran a batch of 2 as fast or faster on every shape).  Here every k-group (32 consecutive activations of a row) has its own
 // power of two, applied by the matrix core itself: the fp8 operand of v_mfma_scale_f32_16x16x128_f8f6f4 takes
 // one E8M0 scale per 32 elements of K and column.  And a digit is not a nibble but a small fp8 (e4m3) number:
 // with v = the activation times the power of two that puts the k-group's largest magnitude into [1/8, 1/4),
@@ -388,7 +389,7 @@ int launch_block_t(const BlockArgs& a, hipStream_t stream) {
 // k-groups one workgroup covers (its one round)
 int hq_q3_block_groups_per_round(void) { return kGroupsPerRound; }
 
-// 3 ... 8 fp16 activation rows; the caller has validated the arguments, cut K into nsplit ranges of rpw rounds
+// 2 ... 8 fp16 activation rows; the caller has validated the arguments, cut K into nsplit ranges of rpw rounds
 // of 4096 elements and, for nsplit > 1, provided nsplit * M * 64 floats of partial sums per column tile and
 // one zeroed counter per column tile.
 int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,

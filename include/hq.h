@@ -129,11 +129,7 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  * (src/quant3MatMul-hip/kernels.h:171-217) — pass HQ_FLAG_ACCUMULATE for their
  * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 and has no counterpart in
  * the reference; which kernel serves it (hq_q3_matvec_plan tells):
- *   - batch 2: the matvec's kernel, at about the cost of batch 1, the two rows side
- *     by side in the matrix-core operand (28-bit fixed point relative to the largest
- *     magnitude among each 512 consecutive activations of a row: exact for fp16
- *     entries within 2^17 of it);
- *   - batches 3 ... 4, and 5 ... 8 unless N / 128 is at least 7/8 of the compute units or
+ *   - batches 2 ... 4 (at 0.1 ... 0.6 us more than batch 1), and 5 ... 8 unless N / 128 is at least 7/8 of the compute units or
  *     K is so long that a workgroup takes several rounds of 4096: the matvec's kernel,
  *     four rows side by side;
  *     every activation enters with an error of at most 2^-19 of the largest magnitude
@@ -152,9 +148,8 @@ int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float
  * tunables (for tests and tuning; negative = error code).
  */
 #define HQ_Q3_PLAN_MATVEC 0 /* batch_M == 1 */
-#define HQ_Q3_PLAN_ROWS 1   /* batch_M == 2 on the matvec's digit kernel */
 #define HQ_Q3_PLAN_GEMM 2   /* batched MFMA GEMM */
-#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 3 ... 8: the matvec's kernel, four rows per pass */
+#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 2 ... 8: the matvec's kernel, four rows per pass */
 int hq_q3_matvec_plan(int K, int N, int batch_M);
 
 /*

@@ -1,7 +1,7 @@
-"""Batches 2 ... 16 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): a batch of 2 runs on the
-matvec's digit kernel with the two rows side by side in the matrix-core operand (K split across workgroups
-as for batch 1), batches 3 ... 8 on the same kernel with every activation as four small fp8 terms under one
-scale per 32 activations (four rows per pass over the weights), all others on the batched GEMM.  Every batch size is checked against the CPU oracle through the C ABI,
+"""Batches 2 ... 16 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): batches 2 ... 8 run on the
+matvec's matrix-core kernel with every activation as four small fp8 terms under one scale per 32 activations
+(four rows side by side in the operand per pass over the weights, K split across workgroups as for batch
+1), all others on the batched GEMM.  Every batch size is checked against the CPU oracle through the C ABI,
 and the kernel that ran is asserted through hq_q3_matvec_plan.  The reference has no batched kernel:
 the oracle is the matvec formula applied row by row (parity unpinned by the reference)."""
 import numpy as np
@@ -12,7 +12,7 @@ from tests.tol import FLOOR_F16, rel_err
 
 pytestmark = pytest.mark.gpu
 
-PLAN_MATVEC, PLAN_ROWS, PLAN_GEMM, PLAN_BLOCK = 0, 1, 2, 3
+PLAN_MATVEC, PLAN_GEMM, PLAN_BLOCK = 0, 2, 3
 
 
 def _t(a):
@@ -39,8 +39,8 @@ def _check(y, exact):
 
 
 # wide (N = 257 tiles, the last one 4 columns wide) and narrow (3 tiles, the last one 4 columns wide);
-# K = 4128 is not a multiple of a workgroup's round, so the two-row kernel splits it in two;
-# the long-K shape is there for the two-row kernel and its neighbours only
+# K = 4128 is not a multiple of a workgroup's round, so the kernel splits it in two;
+# the long-K shape is there for the smallest batches only
 _EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)] for M in range(2, 16)
                 if K != 4128 or M <= 4]
 
@@ -49,19 +49,19 @@ _EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)
 def test_every_batch_vs_oracle(hq, oracle, M, K, N):
     codes, scales, zeros, A = oa.make_q3_problem(1000 + 16 * M + (K % 7), K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
-    want_plan = PLAN_ROWS if M == 2 else (PLAN_BLOCK if M <= 8 else PLAN_GEMM)
+    want_plan = PLAN_BLOCK if M <= 8 else PLAN_GEMM
     assert _plan(K, N, M) == want_plan
     y = _run(hq, A, mat, scales, zeros)
     _check(y, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
 
 
-def test_rows_kernel_against_the_gemm_and_the_matvec(hq, oracle, tunable):
-    """The same call with the two-row kernel switched off takes the GEMM; each row also equals the
+def test_batch2_against_the_gemm_and_the_matvec(hq, oracle, tunable):
+    """The same call with the small-batch kernel switched off takes the GEMM; each row also equals the
     batch-1 matvec on that row.  Three kernels, one result (to the accuracy each of them states)."""
     M, K, N = 2, 2048, 16640
     codes, scales, zeros, A = oa.make_q3_problem(500 + M, K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
-    assert _plan(K, N, M) == PLAN_ROWS
+    assert _plan(K, N, M) == PLAN_BLOCK
     y = _run(hq, A, mat, scales, zeros)
     tunable("HQ_Q3_SMALL_BATCH", 0)
     assert _plan(K, N, M) == PLAN_GEMM
@@ -73,7 +73,7 @@ def test_rows_kernel_against_the_gemm_and_the_matvec(hq, oracle, tunable):
 
 
 @pytest.mark.parametrize("scale_exp", [-16, -8, 0, 4])
-def test_rows_kernel_dynamic_range(hq, oracle, scale_exp):
+def test_batch2_dynamic_range(hq, oracle, scale_exp):
     """Two rows of very different magnitude side by side in one matrix-core operand, an all-zero row, a row
     with one large outlier, magnitudes spread over 2^8 inside a row, fp16 subnormals: every row is held
     to the bound the N(0,1) cases meet, measured against that row's own RMS."""
@@ -92,7 +92,7 @@ def test_rows_kernel_dynamic_range(hq, oracle, scale_exp):
     A = A.astype(np.float16)
     for rows in ([0, 1], [2, 4], [3, 5], [6, 7], [4, 8]):
         sub = np.ascontiguousarray(A[rows])
-        assert _plan(K, N, len(rows)) == PLAN_ROWS
+        assert _plan(K, N, len(rows)) == PLAN_BLOCK
         y = _run(hq, sub, mat, scales, zeros)
         exact = oracle.q3_gemm(sub, mat, scales, zeros, mode=0)
         for i, m in enumerate(rows):
@@ -103,7 +103,7 @@ def test_rows_kernel_dynamic_range(hq, oracle, scale_exp):
                 assert rel_err(y[i], exact[i], FLOOR_F16) <= 1e-4, (scale_exp, m)
 
 
-def test_rows_kernel_non_finite_activations(hq, oracle):
+def test_batch2_non_finite_activations(hq, oracle):
     """An infinity or NaN in one row makes that row NaN and leaves the other row alone."""
     K, N = 512, 8192
     codes, scales, zeros, A = oa.make_q3_problem(91, K, N, x_dtype=np.float16, batch=2)
@@ -116,7 +116,7 @@ def test_rows_kernel_non_finite_activations(hq, oracle):
 
 
 def test_config4_shape_batches_2_3_and_11(hq, oracle):
-    """K=8192, N=28672 (the GEMM configuration's weights) at batch 2 (two-row kernel), 3 (four rows per pass)
+    """K=8192, N=28672 (the GEMM configuration's weights) at batches 2 and 3 (four rows per pass)
     and 11 (GEMM): sampled columns against the oracle, all columns against the batch-1 matvec."""
     import torch
     K, N = 8192, 28672
@@ -129,7 +129,7 @@ def test_config4_shape_batches_2_3_and_11(hq, oracle):
     sub = np.ascontiguousarray(mat[:, cols])
     for M in (2, 3, 11):
         A = rng.standard_normal((M, K)).astype(np.float16)
-        assert _plan(K, N, M) == {2: PLAN_ROWS, 3: PLAN_BLOCK, 11: PLAN_GEMM}[M]
+        assert _plan(K, N, M) == {2: PLAN_BLOCK, 3: PLAN_BLOCK, 11: PLAN_GEMM}[M]
         y = hq.q3_gemm(_t(A), dm, ds, dz)
         torch.cuda.synchronize()
         y = y.cpu().numpy()
@@ -139,7 +139,7 @@ def test_config4_shape_batches_2_3_and_11(hq, oracle):
             assert rel_err(y[m], yv) <= 5e-3
 
 
-def test_rows_kernel_accumulates(hq, oracle):
+def test_batch2_accumulates(hq, oracle):
     """HQ_FLAG_ACCUMULATE adds to what y holds, as for batch 1."""
     import torch
     from hecbench_amd import _lib
@@ -149,7 +149,7 @@ def test_rows_kernel_accumulates(hq, oracle):
     rng = np.random.default_rng(5)
     y0 = rng.standard_normal((M, N)).astype(np.float32)
     dA, dm, ds, dz, dy = _t(A), _t(mat), _t(scales), _t(zeros), _t(y0)
-    assert _plan(K, N, M) == PLAN_ROWS
+    assert _plan(K, N, M) == PLAN_BLOCK
     rc = _lib.load().hq_q3_matvec(dA.data_ptr(), 1, dm.data_ptr(), ds.data_ptr(), dz.data_ptr(), dy.data_ptr(),
                                   K, N, M, 1, None)
     assert rc == 0
@@ -161,30 +161,27 @@ def test_rows_kernel_accumulates(hq, oracle):
 
 
 @pytest.mark.parametrize("K", [32, 96, 160])
-def test_rows_kernel_short_k(hq, oracle, K):
+def test_batch2_short_k(hq, oracle, K):
     """Fewer k-groups than a workgroup's waves cover: idle waves, partly filled steps."""
     N = 8200
     codes, scales, zeros, A = oa.make_q3_problem(700 + K, K, N, x_dtype=np.float16, batch=2)
     mat = oracle.q3_pack(codes)
-    assert _plan(K, N, 2) == PLAN_ROWS
+    assert _plan(K, N, 2) == PLAN_BLOCK
     _check(_run(hq, A, mat, scales, zeros), oracle.q3_gemm(A, mat, scales, zeros, mode=0))
 
 
-# (K, N, forced split or 0): K rounds of 4096 -> one workgroup per round up to eight (three for K = 11008,
-# the last one partly filled), beyond that as many workgroups per tile as the compute units allow, each
-# walking several rounds (K = 36864, 64 tiles); a forced single workgroup walks all of K in rounds
-_SPLIT_SHAPES = [(11008, 4096, 0), (36864, 4096, 0), (40960, 1028, 0), (11008, 4096, 1), (8192, 260, 2)]
+# K rounds of 4096 -> one workgroup per round up to eight (three for K = 11008, the last one partly filled),
+# beyond that as many workgroups per tile as give every compute unit two, each walking several rounds
+_SPLIT_SHAPES = [(11008, 4096), (36864, 4096), (40960, 1028), (8192, 260)]
 
 
-@pytest.mark.parametrize("K,N,force", _SPLIT_SHAPES)
-def test_rows_kernel_splits_k(hq, oracle, tunable, K, N, force):
+@pytest.mark.parametrize("K,N", _SPLIT_SHAPES)
+def test_batch2_splits_k(hq, oracle, K, N):
     """Partial sums of both rows per workgroup, added by the last one to arrive: same result as the
     oracle, the same bits on a second call (the counters reset themselves), and as the batch-1 matvec."""
     codes, scales, zeros, A = oa.make_q3_problem(900 + K % 97 + N % 13, K, N, x_dtype=np.float16, batch=2)
     mat = oracle.q3_pack(codes)
-    if force:
-        tunable("HQ_Q3_KSPLIT", force)
-    assert _plan(K, N, 2) == PLAN_ROWS
+    assert _plan(K, N, 2) == PLAN_BLOCK
     y = _run(hq, A, mat, scales, zeros)
     _check(y, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
     assert np.array_equal(_run(hq, A, mat, scales, zeros), y)
@@ -193,7 +190,7 @@ def test_rows_kernel_splits_k(hq, oracle, tunable, K, N, force):
         assert rel_err(y[m], yv) <= 5e-3
 
 
-def test_rows_kernel_split_k_accumulates_and_strict_fences(hq, oracle, tunable):
+def test_batch2_split_k_accumulates_and_strict_fences(hq, oracle, tunable):
     import torch
     from hecbench_amd import _lib
     M, K, N = 2, 12288, 2052
@@ -266,8 +263,8 @@ def test_block_kernel_plan_limits(hq, tunable):
     assert _plan(8192, 28672, 5) == PLAN_GEMM         # two passes: not where the GEMM's 224 tiles fill the device
     assert _plan(8192, 22016, 8) == PLAN_BLOCK        # 172 tiles of 128 columns
     assert _plan(28672, 8192, 8) == PLAN_BLOCK
-    assert _plan(12288, 65536, 2) == PLAN_ROWS
-    assert _plan(12288, 65536, 3) == PLAN_GEMM        # 1024 tiles x 3 rounds x 3 rows = 9216 partial rows
+    assert _plan(12288, 65536, 3) == PLAN_BLOCK       # 1024 tiles x 3 rounds x 3 rows would be 9216 partial rows: two ranges of K
+    assert _plan(12288, 65536, 8) == PLAN_GEMM        # two passes: one round per workgroup only
     tunable("HQ_Q3_SMALL_BATCH", 16)
     assert _plan(4096, 4096, 9) == PLAN_GEMM
     tunable("HQ_Q3_SMALL_BATCH", 4)
