@@ -1,5 +1,5 @@
 """Calls recorded into a HIP graph: after hq_reserve_workspace the entry points that use a workspace (split-K
-matvec, batched GEMM) allocate nothing during capture, and hq_q3_matvec_noalloc never does.  Every replay is
+matvec, a small batch on the same split, batched GEMM) allocate nothing during capture, and hq_q3_matvec_noalloc never does.  Every replay is
 checked against the eager result, with eager work and synchronisations between the replays."""
 import ctypes
 
@@ -31,6 +31,8 @@ def test_replays_match_eager(hq, oracle):
     y = torch.zeros(N, device="cuda:0")
     y_na = torch.zeros(N, device="cuda:0")
     yg = torch.zeros(M, Ng, device="cuda:0")
+    A4 = torch.randn(4, K, device="cuda:0").half()          # batch 4 on the matvec's weights: partial sums of four rows
+    y4 = torch.zeros(4, N, device="cuda:0")
     stream = torch.cuda.Stream()
     vp = lambda t: ctypes.c_void_p(t.data_ptr())
 
@@ -43,23 +45,26 @@ def test_replays_match_eager(hq, oracle):
         assert lib.hq_reserve_workspace(ctypes.c_void_p(stream.cuda_stream), K, N) == 0
         hq.q3_matvec(dx, dm, ds, dz, out=y)
         hq.q3_gemm(dA, dmg, dsg, dzg, out=yg)
+        hq.q3_gemm(A4, dm, ds, dz, out=y4)
         noalloc(stream)
     stream.synchronize()
-    want, want_g, want_na = y.clone(), yg.clone(), y_na.clone()
+    want, want_g, want_na, want_4 = y.clone(), yg.clone(), y_na.clone(), y4.clone()
     assert torch.equal(want, want_na)
 
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=stream):
         hq.q3_matvec(dx, dm, ds, dz, out=y)
         hq.q3_gemm(dA, dmg, dsg, dzg, out=yg)
+        hq.q3_gemm(A4, dm, ds, dz, out=y4)
         noalloc(torch.cuda.current_stream())
     for rep in range(4):
-        y.fill_(float(rep)); yg.fill_(-1.0); y_na.fill_(7.0)       # eager work between the replays
+        y.fill_(float(rep)); yg.fill_(-1.0); y_na.fill_(7.0); y4.fill_(3.0)  # eager work between the replays
         other = hq.q3_matvec(dx, dm, ds, dz)                       # an eager call on another stream's workspace
         torch.cuda.synchronize()
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y, want), rep
         assert torch.equal(yg, want_g), rep
+        assert torch.equal(y4, want_4), rep
         assert torch.equal(y_na, want_na), rep
         assert torch.equal(other, want), rep
