@@ -350,3 +350,21 @@ def test_block_kernel_short_k(hq, oracle, K):
     mat = oracle.q3_pack(codes)
     assert _plan(K, N, 7) == PLAN_BLOCK
     _check(_run(hq, A, mat, scales, zeros), oracle.q3_gemm(A, mat, scales, zeros, mode=0))
+
+
+def test_small_batches_random_shapes(hq, oracle):
+    """Twenty seeded shapes: K any multiple of 32 up to 12 rounds, N any multiple of 4, batches 2 ... 8."""
+    rng = np.random.default_rng(20250)
+    for case in range(20):
+        K = 32 * int(rng.integers(1, 1536 if case % 5 == 0 else 300))
+        N = 4 * int(rng.integers(1, 700))
+        M = int(rng.integers(2, 9))
+        codes, scales, zeros, A = oa.make_q3_problem(3000 + case, K, N, x_dtype=np.float16, batch=M)
+        mat = oracle.q3_pack(codes)
+        if _plan(K, N, M) != PLAN_BLOCK:
+            continue
+        y = _run(hq, A, mat, scales, zeros)
+        exact = oracle.q3_gemm(A, mat, scales, zeros, mode=0)
+        for m in range(M):
+            assert rel_err(y[m], exact[m]) <= 5e-3, (case, K, N, M, m)
+            assert rel_err(y[m], exact[m], FLOOR_F16) <= 1e-4, (case, K, N, M, m)
