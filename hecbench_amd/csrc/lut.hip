@@ -310,7 +310,9 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: addresses of a round stay scalar
   const int c = lane & 15, kb = lane >> 4;
   const int tile = blockIdx.x;
-  const int nquads = a.K >> 7;
+  // K split: workgroup (tile, split) takes the quads of its slice; nquads is where the slice ends
+  const int q_begin = blockIdx.y * (a.kslice >> 7);
+  const int nquads = min(a.K >> 7, q_begin + (a.kslice >> 7));
   const size_t n0 = RAGGED ? (size_t)min(tile * 64, a.N - 64) : (size_t)tile * 64;
   const uint32_t col_off = 4u * c;  // the lane's four columns: weights, alpha and results
   char* xs_w = xs + wv * (QUADS * kDigQuad);
@@ -387,7 +389,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
   // 8.17 -> 6.89 us at K=4096, N=16384, three planes (two quads ahead 7.34, all quads right after the digits
   // are staged 7.70, nothing before that 7.56-8.6).
   Round ra, rb;
-  int q0 = wv * QUADS;
+  int q0 = q_begin + wv * QUADS;
   load_x(q0, ra);
   load_quad(q0, 0, ra);
   __builtin_amdgcn_sched_barrier(0);
@@ -543,7 +545,38 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
       v += poison_w[w];
     }
     // operand units 2^-10, and the sums hold half of sum s*x
-    a.y[n] = (_Float16)(v * 2048.f);
+    if (a.nsplit == 1) a.y[n] = (_Float16)(v * 2048.f);
+    else __hip_atomic_store(&a.partial[((size_t)tile * a.nsplit + blockIdx.y) * 64 + tid], v, __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (a.nsplit > 1) {
+    // Arrival counting as in the table kernel above and in q3.hip: write-through partial sums, every wave waits
+    // for their acknowledgement, a barrier, one device-scope fetch-add per workgroup, and the last workgroup
+    // to arrive adds the partial sums in split order with loads that bypass the non-coherent cache levels.
+    // (the flag lives in the dynamic LDS block: a static variable would move that block off its 16-byte
+    // alignment, and every 128-bit operand read with it)
+    unsigned* s_last = reinterpret_cast<unsigned*>(poison_w + WAVES);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) {
+      const unsigned old = a.strict ? __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT)
+                                    : __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *s_last = (old == (unsigned)(a.nsplit - 1));
+    }
+    __syncthreads();
+    const bool last = *s_last != 0;
+    if (last && a.strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (last) {
+      if (tid < 64 && n < a.N) {
+        float sum = 0.f;
+        for (int s = 0; s < a.nsplit; ++s)
+          sum += __hip_atomic_load(&a.partial[((size_t)tile * a.nsplit + s) * 64 + tid], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        a.y[n] = (_Float16)(sum * 2048.f);
+      }
+      if (tid == 0)  // ready for the next call
+        __hip_atomic_store(&a.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
   }
 }
 
@@ -804,11 +837,32 @@ int launch_bcq_grouped_nb(const LutArgs& a, bool ragged, hipStream_t stream) {
 // Eight waves per workgroup (two per SIMD, up to 256 VGPRs each); QUADS is bounded by the two register
 // sets of a round's loads.
 template <int NB, int QUADS>
-int launch_bcq_planes(const LutArgs& a, bool ragged, hipStream_t stream) {
+int launch_bcq_planes(LutArgs a, bool ragged, int cus, hipStream_t stream) {
   constexpr int WAVES = 8;
-  const dim3 grid((a.N + 63) / 64), block(WAVES * 64);
-  const size_t smem = (size_t)WAVES * QUADS * kDigQuad + (size_t)WAVES * 4 * 64 * 4 + (size_t)WAVES * 4;
-  const bool one_round = a.K <= 128 * QUADS * WAVES;
+  // K split: with fewer column tiles than compute units, whole rounds (128 QUADS WAVES elements of K) go to
+  // workgroups of their own, as many as there are compute units to take them (K=11008, N=4096, three planes:
+  // 64 tiles x 3 rounds)
+  const int ntiles = (a.N + 63) / 64;
+  const int nquads = a.K >> 7;
+  const int rounds = (nquads + WAVES * QUADS - 1) / (WAVES * QUADS);
+  int nsplit = cus / ntiles;
+  if (nsplit > rounds) nsplit = rounds;
+  if (nsplit < 1) nsplit = 1;
+  const int rpw = (rounds + nsplit - 1) / nsplit;
+  nsplit = (rounds + rpw - 1) / rpw;
+  a.kslice = rpw * WAVES * QUADS * 128;
+  a.nsplit = nsplit;
+  a.strict = hq_tune(HQ_TUNE_SPLITK_FENCES, 0);
+  if (nsplit > 1) {
+    HqWorkspace ws;
+    const int rc = hq_get_workspace(stream, (size_t)ntiles * nsplit * 64, (size_t)ntiles, &ws);
+    if (rc != HQ_OK) return rc;
+    a.partial = ws.partial;
+    a.counters = ws.counters;
+  }
+  const dim3 grid(ntiles, nsplit), block(WAVES * 64);
+  const size_t smem = (size_t)WAVES * QUADS * kDigQuad + (size_t)WAVES * 4 * 64 * 4 + (size_t)WAVES * 4 + 16;
+  const bool one_round = rpw == 1;
 #define HQ_LUT_GO(BIAS, RAG)                                                                                        \
   do {                                                                                                              \
     if (one_round) hipLaunchKernelGGL((bcq_planes_kernel<NB, QUADS, WAVES, BIAS, RAG, true>), grid, block, smem, stream, a); \
@@ -857,14 +911,14 @@ extern "C" int hq_lut_gemv(const uint32_t* bW, const void* alpha, const void* q_
     if ((plan & ~HQ_LUT_PLAN_RAGGED) == HQ_LUT_PLAN_MFMA_GROUPED)
       return group_size == 64 ? launch_bcq_grouped_nb<2>(a, ragged, stream) : launch_bcq_grouped_nb<4>(a, ragged, stream);
     switch (nbits) {  // quads per wave per round, bounded by the register budget
-      case 1: return launch_bcq_planes<1, 4>(a, ragged, stream);
-      case 2: return launch_bcq_planes<2, 4>(a, ragged, stream);
-      case 3: return launch_bcq_planes<3, 4>(a, ragged, stream);
-      case 4: return launch_bcq_planes<4, 2>(a, ragged, stream);
-      case 5: return launch_bcq_planes<5, 2>(a, ragged, stream);
-      case 6: return launch_bcq_planes<6, 2>(a, ragged, stream);
-      case 7: return launch_bcq_planes<7, 1>(a, ragged, stream);
-      default: return launch_bcq_planes<8, 1>(a, ragged, stream);
+      case 1: return launch_bcq_planes<1, 4>(a, ragged, dev->cus, stream);
+      case 2: return launch_bcq_planes<2, 4>(a, ragged, dev->cus, stream);
+      case 3: return launch_bcq_planes<3, 4>(a, ragged, dev->cus, stream);
+      case 4: return launch_bcq_planes<4, 2>(a, ragged, dev->cus, stream);
+      case 5: return launch_bcq_planes<5, 2>(a, ragged, dev->cus, stream);
+      case 6: return launch_bcq_planes<6, 2>(a, ragged, dev->cus, stream);
+      case 7: return launch_bcq_planes<7, 1>(a, ragged, dev->cus, stream);
+      default: return launch_bcq_planes<8, 1>(a, ragged, dev->cus, stream);
     }
   }
   const bool pair = (N % 2 == 0) && !((uintptr_t)bW & 7);

@@ -49,6 +49,20 @@ def test_vs_oracle(hq, oracle, tunable, path, K, N, nb, group, zero_bias, seed):
     assert rel_err(y, ref) <= TOL_F16_ACC
 
 
+@pytest.mark.parametrize("K,N,nb", [(11008, 4096, 3), (8192, 1028, 4), (4224, 448, 8)])
+def test_k_split_of_the_plane_kernel(hq, oracle, tunable, K, N, nb):
+    """Fewer column tiles than compute units: whole rounds of K go to workgroups of their own, whose partial
+    sums the last one to arrive adds in split order.  Same result as the oracle, the same bits on a second
+    call and with the formal device-scope fences."""
+    bW, alpha, qbias, x = oa.make_lut_problem(50 + nb, K, N, nb, 128, False)
+    y = _run(hq, bW, alpha, qbias, x, 128)
+    ref = oracle.lut_gemv_f64(bW, alpha, qbias, x, 128)
+    assert rel_err(y, ref, FLOOR_F16) <= 2e-3
+    assert np.array_equal(y, _run(hq, bW, alpha, qbias, x, 128))
+    tunable("HQ_SPLITK_FENCES", 1)
+    assert np.array_equal(y, _run(hq, bW, alpha, qbias, x, 128))
+
+
 def test_plans(hq):
     """Which kernel a shape takes, asked of the library itself: ragged shapes stay on the matrix cores."""
     from hecbench_amd import _lib
