@@ -132,14 +132,14 @@ extern "C" int hq_reserve_workspace(void* stream, int max_K, int max_N) {
   const size_t full_split = tiles * (rounds <= 8 ? rounds : 1);
   const size_t per_cu = tiles + 2 * (size_t)d->cus;
   size_t split_floats = (full_split > per_cu ? full_split : per_cu) * 64 * 2;
-  // batches 3 ... 8 on the matvec-like kernel: one partial row per tile, round of K and activation row, at most 8192
+  // batches 2 ... 12 on the matvec-like kernel: one partial row per tile, round of K and activation row, at most 8192
   size_t block_splits = rounds;
   if (rounds > 8) {  // longer K: two workgroups per compute unit
     block_splits = 2 * (size_t)d->cus / (tiles ? tiles : 1);
     if (block_splits < 1) block_splits = 1;
     if (block_splits > rounds) block_splits = rounds;
   }
-  const size_t block_rows = tiles * block_splits * 8 < 8192 ? tiles * block_splits * 8 : 8192;
+  const size_t block_rows = tiles * block_splits * 12 < 8192 ? tiles * block_splits * 12 : 8192;
   if (block_rows * 64 > split_floats) split_floats = block_rows * 64;
   HqWorkspace ws;
   return hq_get_workspace((hipStream_t)stream, gemm_floats > split_floats ? gemm_floats : split_floats,

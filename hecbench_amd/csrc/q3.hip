@@ -473,7 +473,7 @@ namespace {
 // Largest batch the matvec-like kernels take by default, and the most partial-sum rows (tiles x splits x batch)
 // the kernel for 2 ... 8 rows may need: what the fixed scratch of the entry point that allocates nothing holds,
 // applied to every caller so that both entry points run the same kernel on the same shape.
-constexpr int kDigitBatchDefault = 8;
+constexpr int kDigitBatchDefault = 12;
 constexpr size_t kBlockPartialRows = 8192;
 
 // How the kernel for 2 ... 8 rows cuts K: up to eight rounds of 4096 elements, one workgroup per round (as the
@@ -509,6 +509,9 @@ int q3_plan(const HqDevice* dev, int K, int N, int batch_M) {
   if (batch_M <= limit && batch_M <= 8 && (nsplit == 1 || groups * batch_M <= kBlockPartialRows) &&
       (batch_M <= 4 || (rpw == 1 && 8 * tiles128 < 7 * (size_t)dev->cus)))
     return HQ_Q3_PLAN_BLOCK;
+  // 9 ... 12 rows, three passes: where the launch has at most one workgroup per compute unit (it is a matter
+  // of latency there, and the GEMM needs three launches)
+  if (batch_M <= limit && batch_M <= 12 && rpw == 1 && groups <= (size_t)dev->cus) return HQ_Q3_PLAN_BLOCK;
   return HQ_Q3_PLAN_GEMM;
 }
 

@@ -1,4 +1,4 @@
-// GPTQ 3-bit product for small batches (2 ... 8 activation rows) on the matvec's matrix-core kernel, gfx950.
+// GPTQ 3-bit product for small batches (2 ... 12 activation rows) on the matvec's matrix-core kernel, gfx950.
 //
 // q3.hip (batch 1) carries the activations as fixed point relative to the largest magnitude a wave sees in a
 // round, eight 4-bit digits per activation, so one matrix-core pass over the weights serves one row (a
@@ -21,10 +21,8 @@
 // activation's own exponent all the way - exact fp16 in fifteen columns for five rows - were built as well:
 // the matrix core does not add products that far apart exactly, 5e-5 of the output RMS was lost.)
 // Five to eight rows take two passes over the weights held in registers: terms of four rows staged in LDS,
-// sixteen MFMAs per wave, the pass's sums folded into four registers, next four rows.  (Three and four
-// passes no longer fit the 128 registers that let two workgroups share a compute unit, and from nine rows on
-// the activations a workgroup reads outweigh its weights: 13.0-21.8 us against the batched GEMM's 13.3-18.0
-// us on 4096 x 4096 ... 8192 x 8192.)
+// sixteen MFMAs per wave, the pass's sums folded into four registers, next four rows; nine to twelve rows
+// take three passes where the launch is small (see q3_block_kernel_many below).
 // Everything else follows q3.hip: a workgroup owns a 64-column tile and one round of K (8 waves x 4 steps x
 // 4 k-groups = 4096 elements), a wave's 16-lane quarter streams one k-group per step as three 128-bit loads,
 // every wave stages its own operand behind a wave-local fence, the waves meet once at the end, and K beyond
@@ -94,8 +92,8 @@ constexpr int kPassRows = 4;                  // rows of activations per pass: s
 constexpr int kStepBytes = 16 * kRowBytes;    // sixteen operand rows
 constexpr int kScaleOff = kSteps * kStepBytes + 160;  // behind the last step and its skew
 constexpr int kWaveBytes = (kScaleOff + 64 + 127) / 128 * 128;  // + scales[4 rows][4 quarters][4 steps], one byte each
-constexpr int kMaxRows = 2 * kPassRows;
-constexpr int kWsumStride = 8;
+constexpr int kMaxRows = 3 * kPassRows;
+constexpr int kWsumStride = 16;
 // the four steps are written by the four lane quarters of one instruction: 32-byte slots 0, 1, 4, 5 of a 256-byte bank period
 __device__ __forceinline__ constexpr int step_off(int s) {
   return s * kStepBytes + (s & 1) * 32 + ((s >> 1) & 1) * 128;
@@ -109,7 +107,7 @@ __device__ __forceinline__ constexpr int step_off(int s) {
 // at most one workgroup per compute unit - changes nothing: a pass costs its ~450 VALU instructions per wave
 // wherever they stand.)
 template <int PASSES, bool MULTI>
-__global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void q3_block_kernel(BlockArgs a) {
+__device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
   // LDS: dig[kWaves][kAreaBytes] | wsum[kWaves][kWsumStride]
   extern __shared__ uint4 smem[];
   constexpr int kAreaBytes = kWaveBytes;
@@ -373,14 +371,26 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   }
 }
 
+// One and two passes: at most 128 registers, so that two workgroups share a compute unit.
 template <int PASSES, bool MULTI>
-int launch_block_t(const BlockArgs& a, hipStream_t stream) {
+__global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void q3_block_kernel(BlockArgs a) {
+  q3_block_body<PASSES, MULTI>(a);
+}
+// Three passes (9 ... 12 rows) take 127 registers and more time than two workgroups per compute unit leave
+// room for; they run where the launch has at most one workgroup per compute unit and is a matter of latency
+// (K=4096, N=11008: 11.2-12.7 us against the batched GEMM's 14.7; four passes: 16.1 against 14.9 at 16 rows).
+template <int PASSES>
+__global__ __launch_bounds__(kWaves * 64) void q3_block_kernel_many(BlockArgs a) {
+  q3_block_body<PASSES, false>(a);
+}
+
+template <auto KERNEL>
+int launch_block(const BlockArgs& a, hipStream_t stream) {
   const size_t smem = (size_t)kWaves * kWaveBytes + (size_t)kWaves * kWsumStride * 4 + 16;
   static const hipError_t attr =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_block_kernel<PASSES, MULTI>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+      hipFuncSetAttribute(reinterpret_cast<const void*>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (attr != hipSuccess) return (int)attr;
-  hipLaunchKernelGGL((q3_block_kernel<PASSES, MULTI>), dim3((a.N + 63) / 64, a.nsplit), dim3(kWaves * 64), smem, stream, a);
+  hipLaunchKernelGGL(KERNEL, dim3((a.N + 63) / 64, a.nsplit), dim3(kWaves * 64), smem, stream, a);
   return hq_launch_status();
 }
 
@@ -389,7 +399,7 @@ int launch_block_t(const BlockArgs& a, hipStream_t stream) {
 // k-groups one workgroup covers (its one round)
 int hq_q3_block_groups_per_round(void) { return kGroupsPerRound; }
 
-// 2 ... 8 fp16 activation rows; the caller has validated the arguments, cut K into nsplit ranges of rpw rounds
+// 2 ... 12 fp16 activation rows; the caller has validated the arguments, cut K into nsplit ranges of rpw rounds
 // of 4096 elements and, for nsplit > 1, provided nsplit * M * 64 floats of partial sums per column tile and
 // one zeroed counter per column tile.
 int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
@@ -402,6 +412,8 @@ int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scale
   a.w = reinterpret_cast<const uint32_t*>(qweight);
   a.scales = scales; a.zeros = zeros; a.y = y; a.partial = partial; a.counters = counters; a.K = K; a.N = N; a.M = M;
   a.nsplit = nsplit; a.rpw = rpw; a.flags = flags & (HQ_FLAG_ACCUMULATE | HQ_FLAG_STRICT_FENCES);
-  if (rpw > 1) return M <= kPassRows ? launch_block_t<1, true>(a, stream) : HQ_ERR_BAD_SHAPE;
-  return M <= kPassRows ? launch_block_t<1, false>(a, stream) : launch_block_t<2, false>(a, stream);
+  if (rpw > 1) return M <= kPassRows ? launch_block<&q3_block_kernel<1, true>>(a, stream) : HQ_ERR_BAD_SHAPE;
+  if (M <= kPassRows) return launch_block<&q3_block_kernel<1, false>>(a, stream);
+  if (M <= 2 * kPassRows) return launch_block<&q3_block_kernel<2, false>>(a, stream);
+  return launch_block<&q3_block_kernel_many<3>>(a, stream);
 }

@@ -129,7 +129,8 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  * (src/quant3MatMul-hip/kernels.h:171-217) — pass HQ_FLAG_ACCUMULATE for their
  * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 and has no counterpart in
  * the reference; which kernel serves it (hq_q3_matvec_plan tells):
- *   - batches 2 ... 4 (at 0.1 ... 0.6 us more than batch 1), and 5 ... 8 unless N / 128 is at least 7/8 of the compute units or
+ *   - batches 2 ... 4 (at 0.1 ... 0.6 us more than batch 1), 9 ... 12 where the launch has at
+ *     most one workgroup per compute unit (N / 64 times K / 4096), and 5 ... 8 unless N / 128 is at least 7/8 of the compute units or
  *     K is so long that a workgroup takes several rounds of 4096: the matvec's kernel,
  *     four rows side by side;
  *     every activation enters with an error of at most 2^-19 of the largest magnitude
@@ -149,7 +150,7 @@ int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float
  */
 #define HQ_Q3_PLAN_MATVEC 0 /* batch_M == 1 */
 #define HQ_Q3_PLAN_GEMM 2   /* batched MFMA GEMM */
-#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 2 ... 8: the matvec's kernel, four rows per pass */
+#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 2 ... 12: the matvec's kernel, four rows per pass */
 int hq_q3_matvec_plan(int K, int N, int batch_M);
 
 /*

@@ -23,7 +23,7 @@ def test_replays_match_eager(hq, oracle):
     K, N = 8192, 8256                       # two rounds of K: split over two workgroups per tile (workspace)
     codes, scales, zeros, x = oa.make_q3_problem(901, K, N)
     mat = oracle.q3_pack(codes)
-    Kg, Ng, M = 1024, 516, 16               # batched GEMM: pre-pass and main kernel meet in the workspace
+    Kg, Ng, M = 1024, 516, 24               # batched GEMM: pre-pass and main kernel meet in the workspace
     codes_g, scales_g, zeros_g, A = oa.make_q3_problem(902, Kg, Ng, x_dtype=np.float16, batch=M)
     mat_g = oracle.q3_pack(codes_g)
     dx, dm, ds, dz = _t(x), _t(mat), _t(scales), _t(zeros)

@@ -1,7 +1,7 @@
-"""Batches 2 ... 16 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): batches 2 ... 8 run on the
-matvec's matrix-core kernel with every activation as four small fp8 terms under one scale per 32 activations
-(four rows side by side in the operand per pass over the weights, K split across workgroups as for batch
-1), all others on the batched GEMM.  Every batch size is checked against the CPU oracle through the C ABI,
+"""Batches 2 ... 16 of the GPTQ 3-bit product (hq_q3_matvec with batch_M > 1): batches 2 ... 8 (up to 12 on
+small launches) run on the matvec's matrix-core kernel with every activation as four small fp8 terms under
+one scale per 32 activations (four rows side by side in the operand per pass over the weights, K split across
+workgroups as for batch 1), all others on the batched GEMM.  Every batch size is checked against the CPU oracle through the C ABI,
 and the kernel that ran is asserted through hq_q3_matvec_plan.  The reference has no batched kernel:
 the oracle is the matvec formula applied row by row (parity unpinned by the reference)."""
 import numpy as np
@@ -49,7 +49,8 @@ _EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)
 def test_every_batch_vs_oracle(hq, oracle, M, K, N):
     codes, scales, zeros, A = oa.make_q3_problem(1000 + 16 * M + (K % 7), K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
-    want_plan = PLAN_BLOCK if M <= 8 else PLAN_GEMM
+    # 9 ... 12 rows: three passes, where the launch has at most one workgroup per compute unit
+    want_plan = PLAN_BLOCK if (M <= 8 or (M <= 12 and N < 1000)) else PLAN_GEMM
     assert _plan(K, N, M) == want_plan
     y = _run(hq, A, mat, scales, zeros)
     _check(y, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
@@ -213,7 +214,7 @@ def test_batch2_split_k_accumulates_and_strict_fences(hq, oracle, tunable):
             assert rel_err(got[m] - y0[m], exact[m], FLOOR_F16) <= 1e-3
 
 
-@pytest.mark.parametrize("M,K,N", [(M, K, N) for (K, N) in [(1024, 196), (4128, 8192)] for M in (2, 3, 4, 5, 8)])
+@pytest.mark.parametrize("M,K,N", [(M, K, N) for (K, N) in [(1024, 196), (4128, 8192)] for M in (2, 3, 4, 5, 8, 11)])
 def test_small_batches_on_the_gemm(hq, oracle, tunable, M, K, N):
     """HQ_Q3_SMALL_BATCH=0 keeps the digit kernels out: the GEMM serves the small batches as well."""
     tunable("HQ_Q3_SMALL_BATCH", 0)
@@ -227,7 +228,8 @@ def test_small_batches_on_the_gemm(hq, oracle, tunable, M, K, N):
 # (two workgroups per tile), eight rounds, and more (workgroups that take several rounds, the last one partly
 # filled); N with a 4-column last tile
 _BLOCK_CASES = [(M, K, N) for (K, N) in [(4128, 1028), (160, 16388)] for M in (3, 4, 5, 6, 7, 8)] + \
-               [(6, 32768, 260), (8, 16384, 196), (4, 8192, 4096), (4, 36864, 1028), (3, 49184, 260)]
+               [(6, 32768, 260), (8, 16384, 196), (4, 8192, 4096), (4, 36864, 1028), (3, 49184, 260)] + \
+               [(M, K, N) for (K, N) in [(4128, 1028), (512, 4100)] for M in (9, 10, 11, 12)]
 
 
 @pytest.mark.parametrize("M,K,N", _BLOCK_CASES)
@@ -258,7 +260,11 @@ def test_block_kernel_plan_limits(hq, tunable):
     assert _plan(49152, 12288, 8) == PLAN_GEMM        # twelve rounds, 192 tiles: six rounds per workgroup, one pass only
     assert _plan(49152, 12288, 4) == PLAN_BLOCK
     assert _plan(4096, 4096, 8) == PLAN_BLOCK
-    assert _plan(4096, 4096, 9) == PLAN_GEMM
+    assert _plan(4096, 4096, 12) == PLAN_BLOCK        # three passes: 64 workgroups
+    assert _plan(4096, 4096, 13) == PLAN_GEMM
+    assert _plan(4096, 16448, 12) == PLAN_GEMM        # 257 workgroups
+    assert _plan(8192, 8192, 12) == PLAN_BLOCK        # 128 tiles x 2 rounds
+    assert _plan(8192, 8256, 12) == PLAN_GEMM
     assert _plan(8192, 28672, 4) == PLAN_BLOCK        # one pass per workgroup: always
     assert _plan(8192, 28672, 5) == PLAN_GEMM         # two passes: not where the GEMM's 224 tiles fill the device
     assert _plan(8192, 22016, 8) == PLAN_BLOCK        # 172 tiles of 128 columns
@@ -266,7 +272,7 @@ def test_block_kernel_plan_limits(hq, tunable):
     assert _plan(12288, 65536, 3) == PLAN_BLOCK       # 1024 tiles x 3 rounds x 3 rows would be 9216 partial rows: two ranges of K
     assert _plan(12288, 65536, 8) == PLAN_GEMM        # two passes: one round per workgroup only
     tunable("HQ_Q3_SMALL_BATCH", 16)
-    assert _plan(4096, 4096, 9) == PLAN_GEMM
+    assert _plan(4096, 4096, 13) == PLAN_GEMM
     tunable("HQ_Q3_SMALL_BATCH", 4)
     assert _plan(4096, 4096, 4) == PLAN_BLOCK
     assert _plan(4096, 4096, 5) == PLAN_GEMM
