@@ -59,9 +59,6 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float lane_f(float v, int l) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
-}
 __device__ __forceinline__ float quad_max(float v) {
   v = fmaxf(v, dpp_f<0xB1>(v));  // quad_perm [1,0,3,2]
   return fmaxf(v, dpp_f<0x4E>(v));  // quad_perm [2,3,0,1]
@@ -69,12 +66,6 @@ __device__ __forceinline__ float quad_max(float v) {
 __device__ __forceinline__ float quad_sum(float v) {
   v += dpp_f<0xB1>(v);
   return v + dpp_f<0x4E>(v);
-}
-__device__ __forceinline__ float wave_sum(float v) {
-  v = quad_sum(v);
-  v += dpp_f<0x141>(v);  // row_half_mirror
-  v += dpp_f<0x140>(v);  // row_mirror
-  return (lane_f(v, 0) + lane_f(v, 16)) + (lane_f(v, 32) + lane_f(v, 48));
 }
 
 constexpr uint32_t low3_mask(int word) {
@@ -133,13 +124,16 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
   // MFMA column c carries term c % 4 of row c / 4 of the pass
   const int crow = c >> 2, cterm = c & 3;
   f4 keep[PASSES];
-  float rowsum[PASSES][kPassRows];  // uniform
+  float rowsum[PASSES];  // sum of the activations of row crow of the pass over this wave's k-groups
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     keep[p] = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int m = 0; m < kPassRows; ++m) rowsum[p][m] = 0.f;
+    rowsum[p] = 0.f;
   }
+  // The sums of the activations (for the zero term) come from the matrix core as well: one more MFMA per step
+  // with a weight operand of all 1/8 (fp6 000001) adds up every operand column, i.e. every term of every row,
+  // with the same scales - the sum of exactly the activations the products see.
+  const v8i eighths = {0x41041041, 0x10410410, 0x04104104, 0x41041041, 0x10410410, 0x04104104, 0, 0};
   constexpr uint32_t M0 = low3_mask(0), M1 = low3_mask(1), M2 = low3_mask(2);
 
   // A workgroup's rounds run one after the other, nothing of the next round in flight during this one: two
@@ -202,18 +196,11 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
       const uint32_t w0 = live ? raw.x : 0u, w1 = live ? raw.y : 0u, w2 = live ? raw.z : 0u, w3 = live ? raw.w : 0u;
       h2v pr[4] = {as_h2(__builtin_amdgcn_perm(w1, w0, 0x05040100u)), as_h2(__builtin_amdgcn_perm(w3, w2, 0x05040100u)),
                    as_h2(__builtin_amdgcn_perm(w1, w0, 0x07060302u)), as_h2(__builtin_amdgcn_perm(w3, w2, 0x07060302u))};
-      const h2v one = {(_Float16)1.f, (_Float16)1.f};
-      float asum = 0.f;
       h2v mx = {(_Float16)0.f, (_Float16)0.f};
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        asum = __builtin_amdgcn_fdot2(pr[i], one, asum, false);
-        mx = __builtin_elementwise_max(mx, __builtin_elementwise_abs(pr[i]));
-      }
+      for (int i = 0; i < 4; ++i) mx = __builtin_elementwise_max(mx, __builtin_elementwise_abs(pr[i]));
       const float amax = fmaxf((float)mx[0], (float)mx[1]);
       const float gmax = quad_max(amax);  // the k-group's largest magnitude (its four lanes)
-      const float total = wave_sum(asum);
-      rowsum[p][m] += total;
       // 2^E * max|x| lies in [2^-3, 2^-2): 64 ... 127 subnormal steps of the fp8 format.  fp16 magnitudes: E in -18 ... 21.
       int E = -3 - ((int)((__float_as_uint(gmax) >> 23) & 255u) - 127);
       E = gmax > 0.f ? max(-18, min(21, E)) : 0;
@@ -262,7 +249,7 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
     }
     // the scales of the column's row for this lane quarter's k-group in the four steps, times 16^-term
     const uint32_t sc4 = *reinterpret_cast<const uint32_t*>(sc_tab + (crow * 4 + kb) * 4) - (uint32_t)cterm * 0x04040404u;
-    f4 acc[4];
+    f4 acc[4], colsum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int q = 0; q < 4; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -272,6 +259,7 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
       const u4v b0 = bp[0], b1 = bp[1];
       const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
       const int scale_b = (int)(sc4 >> (8 * s));  // byte 0: this step's scale
+      colsum = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(eighths, B, colsum, 2, 0, 0, 0x7f7f7f7f, 0, scale_b);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const uint32_t w0 = wreg[s][0][q], w1 = wreg[s][1][q], w2 = wreg[s][2][q];
@@ -291,6 +279,7 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
       asm volatile("" : "+v"(v));  // selected here, not where it is stored (four candidates alive until then)
       keep[p][q] += v;
     }
+    rowsum[p] += quad_sum(colsum[0]);  // every result row holds the column sums
   };
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
@@ -307,9 +296,7 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
     *reinterpret_cast<f4*>(red_w + (kPassRows * p + crow) * 64 + 4 * (4 * kb + cterm)) = keep[p];
-#pragma unroll
-    for (int m = 0; m < kPassRows; ++m)
-      if (lane == 0) wsum[wv * kWsumStride + kPassRows * p + m] = rowsum[p][m];
+    if (kb == 0 && cterm == 0) wsum[wv * kWsumStride + kPassRows * p + crow] = rowsum[p];
   }
   __syncthreads();
 
