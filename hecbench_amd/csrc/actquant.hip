@@ -27,10 +27,14 @@ typedef uint32_t u2v __attribute__((ext_vector_type(2)));
 struct bf16_t { uint16_t bits; };  // bfloat16 = the upper half of an fp32
 
 // src/quantVLLM-cuda/utils.h:9-24
+// The saturation is done on the converted integer (the hardware conversion saturates at the int32 range
+// and turns a NaN into 0, as the conversion of the clamped float did): one integer median instead of
+// two compares and two selects per element.
 __device__ __forceinline__ int float_to_int8_rn(float x) {
-  float dst = rintf(x);
-  dst = dst < -128.f ? -128.f : (127.f < dst ? 127.f : dst);
-  return (int)dst;
+  const float dst = rintf(x);
+  int r;
+  asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(dst));
+  return min(max(r, -128), 127);
 }
 // src/quantVLLM-cuda/utils.h:26-50: round to nearest even, saturating at the int32 range.  The
 // hardware conversion saturates by itself (and turns a NaN into 0); it is written as an instruction
@@ -94,6 +98,13 @@ __device__ __forceinline__ void forget(Raw<T>& r) {
     asm volatile("" : "+v"(r.w[i]));
 }
 
+// The low bytes of four integers as one word, a first: byte selects instead of masks and shifts.
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+  const uint32_t lo = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);
+  const uint32_t hi = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x04000c0cu);
+  return lo | hi;
+}
+
 // Stores elements [lo, hi) of a unit's eight results; all eight as one 64-bit store.  STREAM: as a
 // write-through nontemporal store, which the one-pass static kernels gain from (14.2 -> 13.5 us at 4096 x 5137
 // fp16) and the two-pass dynamic kernels lose by (18.5 -> 22.9 us).
@@ -103,20 +114,16 @@ __device__ __forceinline__ void store_unit(int8_t* __restrict__ out, int64_t uni
   int8_t* p = out + unit * kVec;
   if (lo == 0 && hi == kVec && aligned) {
     u2v w;
-    w.x = (uint32_t)(q[0] & 255) | ((uint32_t)(q[1] & 255) << 8) | ((uint32_t)(q[2] & 255) << 16) |
-          ((uint32_t)(q[3] & 255) << 24);
-    w.y = (uint32_t)(q[4] & 255) | ((uint32_t)(q[5] & 255) << 8) | ((uint32_t)(q[6] & 255) << 16) |
-          ((uint32_t)(q[7] & 255) << 24);
+    w.x = pack4(q[0], q[1], q[2], q[3]);
+    w.y = pack4(q[4], q[5], q[6], q[7]);
     if (STREAM) hq_store_stream(reinterpret_cast<hq_u2v*>(p), w);
     else __builtin_nontemporal_store(w, reinterpret_cast<u2v*>(p));
   } else if (aligned) {
     // a unit shared with the neighbouring row: the fewest naturally aligned pieces that cover [lo, hi)
     // (a store instruction costs the same whatever it carries, and the other lanes wait for it)
     uint32_t w[2];
-    w[0] = (uint32_t)(q[0] & 255) | ((uint32_t)(q[1] & 255) << 8) | ((uint32_t)(q[2] & 255) << 16) |
-           ((uint32_t)(q[3] & 255) << 24);
-    w[1] = (uint32_t)(q[4] & 255) | ((uint32_t)(q[5] & 255) << 8) | ((uint32_t)(q[6] & 255) << 16) |
-           ((uint32_t)(q[7] & 255) << 24);
+    w[0] = pack4(q[0], q[1], q[2], q[3]);
+    w[1] = pack4(q[4], q[5], q[6], q[7]);
 #pragma unroll
     for (int d = 0; d < 2; ++d) {
       const bool whole = lo <= 4 * d && hi >= 4 * d + 4;
@@ -139,10 +146,11 @@ __device__ __forceinline__ void store_unit(int8_t* __restrict__ out, int64_t uni
   }
 }
 
-// Division by a scale that many elements share.  y = v * (1 / s) differs from the rounded quotient by
-// at most 2 ulp (half an ulp each for the reciprocal, the product and the quotient itself, rounded up),
-// so both round to the same integer unless y is within 2^-21 |y| of a tie; where the result saturates
-// the quotient need not be known at all.  The reciprocal must be a normal number for that bound.
+// Division by a scale that many elements share.  y = v * (1 / s) differs from the rounded quotient q by
+// less than 1.5 * 2^-23 |q| (2^-24 relative each for the reciprocal, the product and the quotient itself),
+// so both round to the same integer unless y is within that of a tie; the checks below allow twice as
+// much, 3 * 2^-23 |y|, which also covers their own rounding.  Where the result saturates the quotient
+// need not be known at all.  The reciprocal must be a normal number for that bound.
 struct Divisor {
   float s, r;
   bool usable;
@@ -155,23 +163,54 @@ struct Divisor {
 // float_to_int8_rn(v / s) or, with AZP, int32_to_int8(float_to_int32_rn(v / s) + azp), for eight values.
 template <bool AZP>
 __device__ __forceinline__ void quantise8(const float (&v)[kVec], const Divisor& d, int azp, int (&q)[kVec]) {
-  bool exact = !d.usable;
-  float y[kVec];
+  if (!AZP) {
+    // Without a zero point only |y| < 129 can end anywhere but at a bound, and there 3 * 2^-23 |y| is less
+    // than 2^-15: one constant margin for all eight, taken on the largest distance of a product from its
+    // nearest integer.  The subtraction is exact and must stay one (contracted into a multiply-add it
+    // would return the rounding error of products beyond 2^23 and send those to the division).  A NaN
+    // distance - an infinite or NaN input - drops out of the maximum: such a product converts to the same
+    // bound, or to 0, as the quotient.
+#pragma clang fp contract(off)
+    float n[kVec], worst = 0.f;
 #pragma unroll
-  for (int i = 0; i < kVec; ++i) {
-    y[i] = v[i] * d.r;
-    const float dist = fabsf(y[i] - rintf(y[i]));  // distance to the nearest integer
-    // false for a NaN and for |y| >= 2^20; the constant margin covers quotients too small for a relative bound
-    const bool clear = fmaf(fabsf(y[i]), 0x1p-21f, dist) < 0.5f - 0x1p-20f;
-    // without a zero point everything beyond +-129 saturates whichever way it rounds
-    exact |= AZP ? !clear : !(clear || fabsf(y[i]) > 130.f);
+    for (int i = 0; i < kVec; ++i) {
+      const float y = v[i] * d.r;
+      n[i] = rintf(y);
+      worst = fmaxf(worst, fabsf(y - n[i]));
+    }
+    const bool exact = !d.usable || !(worst <= 0.5f - 0x1p-15f);
+    if (__builtin_amdgcn_ballot_w64(exact)) {
+#pragma unroll
+      for (int i = 0; i < kVec; ++i) n[i] = rintf(v[i] / d.s);
+    }
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+      int r;
+      asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(n[i]));
+      q[i] = min(max(r, -128), 127);
+    }
+    return;
   }
+  // With a zero point any quotient may matter: the margin is relative (a subnormal product has no
+  // relative bound and no tie near it either); it reaches 0.5, i.e. sends the unit to the division, from
+  // |y| = 2^20.4 on.  One comparison for the largest of the eight; a NaN drops out as above.
+  float y[kVec], worst = 0.f;
+  {
+#pragma clang fp contract(off)
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+      y[i] = v[i] * d.r;
+      const float dist = fabsf(y[i] - rintf(y[i]));  // distance to the nearest integer
+      worst = fmaxf(worst, fmaf(fabsf(y[i]), 0x1.8p-22f, dist));
+    }
+  }
+  const bool exact = !d.usable || !(worst < 0.5f - 0x1p-24f);
   if (__builtin_amdgcn_ballot_w64(exact)) {
 #pragma unroll
     for (int i = 0; i < kVec; ++i) y[i] = v[i] / d.s;
   }
 #pragma unroll
-  for (int i = 0; i < kVec; ++i) q[i] = AZP ? int32_to_int8(float_to_int32_rn(y[i]) + azp) : float_to_int8_rn(y[i]);
+  for (int i = 0; i < kVec; ++i) q[i] = int32_to_int8(float_to_int32_rn(y[i]) + azp);
 }
 
 // ---- static scale: elementwise over the whole tensor ---------------------------------------------

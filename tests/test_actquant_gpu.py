@@ -69,9 +69,17 @@ def test_static_division_ties_and_extreme_scales(hq, oracle, scale):
         ties = ((k + 0.5) * np.float64(s)).astype(np.float32)
         ints = (k * np.float64(s)).astype(np.float32)
         base = np.concatenate([ties, ints])
-        x = np.concatenate([base, np.nextafter(base, np.float32(np.inf)), np.nextafter(base, np.float32(-np.inf)),
+        beside = []  # one to six floats either side: the window in which product and quotient can round apart
+        up, down = base, base
+        for _ in range(6):
+            up, down = np.nextafter(up, np.float32(np.inf)), np.nextafter(down, np.float32(-np.inf))
+            beside += [up, down]
+        x = np.concatenate([base] + beside + [
                             np.array([0.0, -0.0, np.inf, -np.inf, 3e38, -3e38, 1e-45, 1e30, -1e30], np.float32),
-                            np.random.default_rng(3).standard_normal(3000).astype(np.float32) * np.float32(abs(scale)) * 60])
+                            np.random.default_rng(3).standard_normal(3000).astype(np.float32) * np.float32(abs(scale)) * 60,
+                            (np.arange(-2.0 ** 20, 2.0 ** 20, 2049.0) + 0.5) * np.float64(s),
+                            (k + 0.5 + 2000000.0) * np.float64(s), (k + 0.5 - 2000000.0) * np.float64(s),
+                            (k + 0.5 + 100.0) * np.float64(s), (k + 0.5 - 54.0) * np.float64(s)]).astype(np.float32)
     x = np.ascontiguousarray(np.resize(x, (4, x.size // 4)))
     dx = _dev(x)
     for azp in (None, 0, 54, -100, 2000000, -2000000):
