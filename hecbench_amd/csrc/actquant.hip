@@ -12,8 +12,8 @@
 // (the reference's run size is 5137); a unit that straddles a row boundary is masked.
 //   static : no row structure at all, a flat grid-stride loop over the units.
 //   dynamic: a wave per row up to 1536 elements, a workgroup per row beyond; the row stays in registers
-//            between the max / min pass and the quantise pass (one read of x, up to 10240 elements),
-//            and the next row is already being loaded meanwhile.
+//            between the max / min pass and the quantise pass (one read of x, up to 10240 elements);
+//            one launch slot per row, many workgroups per CU.
 // The division by a scale shared by many elements is done as a multiplication by its reciprocal
 // wherever that provably rounds to the same integer (the product is further from a tie than its error
 // bound, or saturates either way); the other lanes divide.
@@ -245,176 +245,132 @@ __global__ __launch_bounds__(256) void static_quant_kernel(const T* __restrict__
 }
 
 // ---- dynamic scale: LANES threads per row --------------------------------------------------------
-// Maximum of a[r] and minimum of b[r], r < R, over the LANES threads of a row.
-template <int LANES, int R>
-__device__ __forceinline__ void rows_max_min(float (&a)[R], float (&b)[R], float* lds) {
+// Maximum of a and minimum of b over the LANES threads of a row.
+template <int LANES>
+__device__ __forceinline__ void row_max_min(float& a, float& b, float* lds) {
 #pragma unroll
-  for (int r = 0; r < R; ++r)
-#pragma unroll
-    for (int m = 32; m > 0; m >>= 1) {
-      a[r] = fmaxf(a[r], __shfl_xor(a[r], m));
-      b[r] = fminf(b[r], __shfl_xor(b[r], m));
-    }
-  if (LANES > 64) {  // the rows span the workgroup: one exchange for all of them
+  for (int m = 32; m > 0; m >>= 1) {
+    a = fmaxf(a, __shfl_xor(a, m));
+    b = fminf(b, __shfl_xor(b, m));
+  }
+  if (LANES > 64) {  // the row spans the workgroup
     const int wv = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) {
-#pragma unroll
-      for (int r = 0; r < R; ++r) { lds[8 * r + wv] = a[r]; lds[8 * r + 4 + wv] = b[r]; }
-    }
+    if ((threadIdx.x & 63) == 0) { lds[wv] = a; lds[4 + wv] = b; }
     __syncthreads();
 #pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int w = 0; w < LANES / 64; ++w) { a[r] = fmaxf(a[r], lds[8 * r + w]); b[r] = fminf(b[r], lds[8 * r + 4 + w]); }
+    for (int w = 0; w < LANES / 64; ++w) { a = fmaxf(a, lds[w]); b = fminf(b, lds[4 + w]); }
   }
 }
 
-constexpr int kMaxRows = 3;
-
-// LANES threads per row (a wave, or the workgroup), so 256 / LANES row slots per workgroup, and R rows
-// in turn per slot and trip.  KEEP units per thread and row stay in registers between the max / min
-// pass and the quantise pass; a longer row streams the rest twice.  The next trip's rows are requested
-// as soon as this trip's have been scanned, so their loads are in flight during the reduction, the
-// quantisation and the stores: R is chosen so that this is enough data to cover the memory latency.
+// LANES threads per row (a wave, or the workgroup), so 256 / LANES rows per workgroup and one workgroup
+// for every 256 / LANES rows: nothing loops over rows.  KEEP units per thread stay in registers between
+// the max / min pass and the quantise pass; a longer row streams the rest twice.  (Workgroups that walked
+// over several rows, the next rows' loads in flight during the reduction, the quantisation and the stores,
+// needed twice the registers for half the waves per CU and measured 18.8 us where this takes 14.0, 4096
+// rows of 5137 fp16: the hardware overlaps one row's stores with another's loads by itself when enough
+// workgroups fit a CU.)
 // VEC: both pointers are aligned and the tensor is a whole number of units, so every unit is loaded whole.
-template <typename T, bool AZP, int LANES, int KEEP, int R, bool VEC>
+template <typename T, bool AZP, int LANES, int KEEP, bool VEC>
 __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict__ in, int8_t* __restrict__ out,
                                                            float* __restrict__ scales, int32_t* __restrict__ azps,
                                                            int64_t tokens, int hidden) {
   constexpr bool aligned = VEC;
-  __shared__ float lds[8 * kMaxRows];
+  __shared__ float lds[8];
   const int lane = threadIdx.x % LANES;
   const int64_t total = tokens * hidden;
-  // the loop bounds are uniform over the wave (LANES == 64) or the workgroup
-  const int64_t slot = LANES == 64 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
-  const int64_t slots = LANES == 64 ? (int64_t)gridDim.x * 4 : gridDim.x;
-  // A row's units, and the multiple of 64 at or before its first: lanes are laid over the units from
+  // uniform over the wave (LANES == 64) or the workgroup
+  const int64_t token = LANES == 64 ? (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
+  if (token >= tokens) return;
+  // The row's units, and the multiple of 64 at or before its first: lanes are laid over the units from
   // there, so that a wave's loads and stores cover whole 128-byte lines of the output (256 of the
   // input) except at the row's ends.  Everything per row is uniform: base pointers at that multiple of
   // 64, and 32-bit unit numbers j relative to it (valid in [first, end)).
-  struct Row { const T* in; int8_t* out; int64_t ubase; int first, end, head; };
-  auto row_of = [&](int64_t token) {
-    Row w;
-    const int64_t g0 = token * hidden;
-    const int64_t u_first = g0 / kVec;
-    w.ubase = u_first & ~(int64_t)63;
-    w.first = (int)(u_first - w.ubase);
-    w.end = (int)((g0 + hidden + kVec - 1) / kVec - w.ubase);
-    w.head = (int)(g0 - u_first * kVec);  // elements of the first unit that belong to the row before
-    w.in = in + w.ubase * kVec;
-    w.out = out + w.ubase * kVec;
-    return w;
-  };
-  auto fetch = [&](const Row& w, int j) {
-    return VEC ? load_unit(w.in, j) : load_unit_tail(in, w.ubase + j, total);
-  };
-  auto load_row = [&](int64_t token, Raw<T> (&buf)[KEEP]) {
-    const Row w = row_of(token);
-#pragma unroll
-    for (int k = 0; k < KEEP; ++k) {
-      const int j = lane + k * LANES;
-      // whole units are loaded without a branch, so that the loads stay one straight run the waits can
-      // count; a unit outside the row repeats the row's first or last
-      if (VEC) buf[k] = load_unit(w.in, min(max(j, w.first), w.end - 1));
-      else if (j >= w.first && j < w.end) buf[k] = fetch(w, j);
-    }
-  };
-  Raw<T> keep[R][KEEP], ahead[R][KEEP];
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-    if (slot + r * slots < tokens) load_row(slot + r * slots, keep[r]);
-  for (int64_t first = slot; first < tokens; first += slots * R) {
-    float mx[R], mn[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      // reference initial values: max starts at FLT_MIN (smallest positive normal), min at FLT_MAX
-      // (reference.h:71-72); the symmetric variant starts its absmax at 0 (reference.h:43)
-      mx[r] = AZP ? 1.17549435e-38f : 0.f;
-      mn[r] = 3.40282347e+38f;
-      const int64_t token = first + r * slots;
-      if (token >= tokens) continue;
-      const Row w = row_of(token);
-      auto scan = [&](const Raw<T>& raw, int j) {
-        float v[kVec];
-        unpack(raw, v);
-        const int rel = (j - w.first) * kVec - w.head;  // row position of the unit's element 0
-        const int lo = max(-rel, 0), hi = min(hidden - rel, kVec);
-        if (lo == 0 && hi == kVec) {  // all but the row's first and last unit
-#pragma unroll
-          for (int i = 0; i < kVec; ++i) {
-            if (AZP) { mx[r] = fmaxf(mx[r], v[i]); mn[r] = fminf(mn[r], v[i]); }
-            else mx[r] = fmaxf(mx[r], fabsf(v[i]));
-          }
-        } else {
-#pragma unroll
-          for (int i = 0; i < kVec; ++i)
-            if (i >= lo && i < hi) {
-              if (AZP) { mx[r] = fmaxf(mx[r], v[i]); mn[r] = fminf(mn[r], v[i]); }
-              else mx[r] = fmaxf(mx[r], fabsf(v[i]));
-            }
-        }
-      };
-#pragma unroll
-      for (int k = 0; k < KEEP; ++k) {
-        const int j = lane + k * LANES;
-        if (j >= w.first && j < w.end) scan(keep[r][k], j);
-      }
-      for (int j = lane + KEEP * LANES; j < w.end; j += LANES) scan(fetch(w, j), j);
-    }
-    // the next trip's loads go out here, behind nothing this trip still waits for
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int64_t token = first + (R + r) * slots;
-      if (token < tokens) load_row(token, ahead[r]);
-    }
-    rows_max_min<LANES, R>(mx, mn, lds);
+  const int64_t g0 = token * hidden;
+  const int64_t u_first = g0 / kVec;
+  const int64_t ubase = u_first & ~(int64_t)63;
+  const int first = (int)(u_first - ubase);
+  const int end = (int)((g0 + hidden + kVec - 1) / kVec - ubase);
+  const int head = (int)(g0 - u_first * kVec);  // elements of the first unit that belong to the row before
+  const T* row_in = in + ubase * kVec;
+  int8_t* row_out = out + ubase * kVec;
+  auto fetch = [&](int j) { return VEC ? load_unit(row_in, j) : load_unit_tail(in, ubase + j, total); };
 
+  Raw<T> keep[KEEP];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int64_t token = first + r * slots;
-      if (token >= tokens) continue;
-      const Row w = row_of(token);
-      float scale_val, mul = 0.f;
-      int azp_val = 0;
-      if (AZP) {
-        scale_val = (mx[r] - mn[r]) / 255.0f;
-        azp_val = (int)rintf(-128.0f - mn[r] / scale_val);
-      } else {
-        scale_val = mx[r] / 127.0f;
-        mul = 127.0f / mx[r];
-      }
-      if (lane == 0) {
-        scales[token] = scale_val;
-        if (AZP) azps[token] = azp_val;
-      }
-      const Divisor d(scale_val);
-      auto emit = [&](Raw<T> raw, int j) {
-        float v[kVec];
-        int q[kVec];
-        forget(raw);
-        unpack(raw, v);
-        if (AZP) {
-          quantise8<true>(v, d, azp_val, q);
-        } else {
-#pragma unroll
-          for (int i = 0; i < kVec; ++i) q[i] = float_to_int8_rn(v[i] * mul);
-        }
-        const int rel = (j - w.first) * kVec - w.head;
-        store_unit<false>(w.out, j, q, max(-rel, 0), min(hidden - rel, kVec), aligned);
-      };
-#pragma unroll
-      for (int k = 0; k < KEEP; ++k) {
-        const int j = lane + k * LANES;
-        if (j >= w.first && j < w.end) emit(keep[r][k], j);
-      }
-      for (int j = lane + KEEP * LANES; j < w.end; j += LANES) emit(fetch(w, j), j);
-    }
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int k = 0; k < KEEP; ++k) keep[r][k] = ahead[r][k];
-    if (LANES > 64) __syncthreads();  // the exchange buffer is reused by the next trip
+  for (int k = 0; k < KEEP; ++k) {
+    const int j = lane + k * LANES;
+    // whole units are loaded without a branch, so that the loads stay one straight run the waits can
+    // count; a unit outside the row repeats the row's first or last
+    if (VEC) keep[k] = load_unit(row_in, min(max(j, first), end - 1));
+    else if (j >= first && j < end) keep[k] = fetch(j);
   }
+
+  // reference initial values: max starts at FLT_MIN (smallest positive normal), min at FLT_MAX
+  // (reference.h:71-72); the symmetric variant starts its absmax at 0 (reference.h:43)
+  float mx = AZP ? 1.17549435e-38f : 0.f;
+  float mn = 3.40282347e+38f;
+  auto scan = [&](const Raw<T>& raw, int j) {
+    float v[kVec];
+    unpack(raw, v);
+    const int rel = (j - first) * kVec - head;  // row position of the unit's element 0
+    const int lo = max(-rel, 0), hi = min(hidden - rel, kVec);
+    if (lo == 0 && hi == kVec) {  // all but the row's first and last unit
+#pragma unroll
+      for (int i = 0; i < kVec; ++i) {
+        if (AZP) { mx = fmaxf(mx, v[i]); mn = fminf(mn, v[i]); }
+        else mx = fmaxf(mx, fabsf(v[i]));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kVec; ++i)
+        if (i >= lo && i < hi) {
+          if (AZP) { mx = fmaxf(mx, v[i]); mn = fminf(mn, v[i]); }
+          else mx = fmaxf(mx, fabsf(v[i]));
+        }
+    }
+  };
+#pragma unroll
+  for (int k = 0; k < KEEP; ++k) {
+    const int j = lane + k * LANES;
+    if (j >= first && j < end) scan(keep[k], j);
+  }
+  for (int j = lane + KEEP * LANES; j < end; j += LANES) scan(fetch(j), j);
+  row_max_min<LANES>(mx, mn, lds);
+
+  float scale_val, mul = 0.f;
+  int azp_val = 0;
+  if (AZP) {
+    scale_val = (mx - mn) / 255.0f;
+    azp_val = (int)rintf(-128.0f - mn / scale_val);
+  } else {
+    scale_val = mx / 127.0f;
+    mul = 127.0f / mx;
+  }
+  if (lane == 0) {
+    scales[token] = scale_val;
+    if (AZP) azps[token] = azp_val;
+  }
+  const Divisor d(scale_val);
+  auto emit = [&](Raw<T> raw, int j) {
+    float v[kVec];
+    int q[kVec];
+    forget(raw);
+    unpack(raw, v);
+    if (AZP) {
+      quantise8<true>(v, d, azp_val, q);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kVec; ++i) q[i] = float_to_int8_rn(v[i] * mul);
+    }
+    const int rel = (j - first) * kVec - head;
+    store_unit<false>(row_out, j, q, max(-rel, 0), min(hidden - rel, kVec), aligned);
+  };
+#pragma unroll
+  for (int k = 0; k < KEEP; ++k) {
+    const int j = lane + k * LANES;
+    if (j >= first && j < end) emit(keep[k], j);
+  }
+  for (int j = lane + KEEP * LANES; j < end; j += LANES) emit(fetch(j), j);
 }
 
 // The 128-bit loads and 64-bit stores need both base pointers on their grid; other pointers are served
@@ -444,25 +400,24 @@ int launch_static(const T* in, int8_t* out, int64_t tokens, int hidden, float sc
 template <typename T, bool AZP, bool VEC>
 void launch_dynamic_vec(const T* in, int8_t* out, float* scales, int32_t* azps, int64_t tokens, int hidden,
                         const HqDevice* dev, hipStream_t stream) {
-  // short rows get a wave each, the others the workgroup; the units a thread must keep pick the kernel,
-  // and shorter rows go several to a trip
+  // short rows get a wave each, the others the workgroup; the units a thread must keep pick the kernel
   const bool wave_rows = hidden <= 64 * kVec * 3;
   const int lanes = wave_rows ? 64 : 256;
   const int span = (hidden + kVec - 1) / kVec + 1 + 63;  // units from the 64-unit boundary before a ragged row to its end
   const int need = (span + lanes - 1) / lanes;
   const int64_t groups = wave_rows ? (tokens + 3) / 4 : tokens;
-  const dim3 grid((unsigned)std::min<int64_t>(groups, (int64_t)dev->cus * hq_tune(HQ_TUNE_ACTQ_GROUPS, 8))), block(256);
-#define HQ_ROWS(LANES, KEEP, R)                                                                                   \
-  hipLaunchKernelGGL((dynamic_quant_kernel<T, AZP, LANES, KEEP, R, VEC>), grid, block, 0, stream, in, out, scales, \
+  const dim3 grid((unsigned)groups), block(256);
+#define HQ_ROWS(LANES, KEEP)                                                                                    \
+  hipLaunchKernelGGL((dynamic_quant_kernel<T, AZP, LANES, KEEP, VEC>), grid, block, 0, stream, in, out, scales, \
                      azps, tokens, hidden)
   if (wave_rows) {
-    if (need <= 2) HQ_ROWS(64, 2, 3);
-    else if (need <= 3) HQ_ROWS(64, 3, 2);
-    else HQ_ROWS(64, 5, 1);
+    if (need <= 2) HQ_ROWS(64, 2);
+    else if (need <= 3) HQ_ROWS(64, 3);
+    else HQ_ROWS(64, 5);
   } else {
-    if (need <= 2) HQ_ROWS(256, 2, 3);
-    else if (need <= 3) HQ_ROWS(256, 3, 2);
-    else HQ_ROWS(256, 5, 1);
+    if (need <= 2) HQ_ROWS(256, 2);
+    else if (need <= 3) HQ_ROWS(256, 3);
+    else HQ_ROWS(256, 5);
   }
 #undef HQ_ROWS
 }
