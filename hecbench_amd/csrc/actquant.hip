@@ -89,6 +89,61 @@ __device__ __forceinline__ void unpack(const Raw<bf16_t>& r, float (&v)[kVec]) {
     v[i] = __uint_as_float((i & 1) ? (r.w[0][i >> 1] & 0xffff0000u) : (r.w[0][i >> 1] << 16));
 }
 
+// y[i] = element i * m.  An fp16 element is converted and multiplied by one mixed-precision instruction
+// (the added +0 only turns a product of -0 into +0, which rounds to the same integer).
+template <typename T>
+__device__ __forceinline__ void products(const Raw<T>& r, float m, float (&y)[kVec]) {
+  float v[kVec];
+  unpack(r, v);
+#pragma unroll
+  for (int i = 0; i < kVec; ++i) y[i] = v[i] * m;
+}
+__device__ __forceinline__ void products(const Raw<_Float16>& r, float m, float (&y)[kVec]) {
+#pragma unroll
+  for (int i = 0; i < kVec / 2; ++i) {
+    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(y[2 * i]) : "v"(r.w[0][i]), "v"(m));
+    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(y[2 * i + 1]) : "v"(r.w[0][i]), "v"(m));
+  }
+}
+
+// Running maximum and minimum of whole units.  fp16 units are scanned as packed halves (the maximum of
+// magnitudes on the bits with the signs cleared), everything else as converted floats.
+typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+template <typename T, bool AZP>
+struct UnitScan {
+  __device__ __forceinline__ void add(const Raw<T>& r, float& mx, float& mn) {
+    float v[kVec];
+    unpack(r, v);
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) {
+      if (AZP) { mx = fmaxf(mx, v[i]); mn = fminf(mn, v[i]); }
+      else mx = fmaxf(mx, fabsf(v[i]));
+    }
+  }
+  __device__ __forceinline__ void fold(float&, float&) {}
+};
+template <bool AZP>
+struct UnitScan<_Float16, AZP> {
+  h2v hi, lo;
+  __device__ __forceinline__ UnitScan() {
+    const _Float16 inf = (_Float16)__builtin_inff();
+    hi = AZP ? h2v{-inf, -inf} : h2v{(_Float16)0.f, (_Float16)0.f};
+    lo = h2v{inf, inf};
+  }
+  __device__ __forceinline__ void add(const Raw<_Float16>& r, float&, float&) {
+#pragma unroll
+    for (int i = 0; i < kVec / 2; ++i) {
+      const h2v x = __builtin_bit_cast(h2v, AZP ? r.w[0][i] : (r.w[0][i] & 0x7fff7fffu));
+      hi = __builtin_elementwise_max(hi, x);
+      if (AZP) lo = __builtin_elementwise_min(lo, x);
+    }
+  }
+  __device__ __forceinline__ void fold(float& mx, float& mn) {
+    mx = fmaxf(mx, fmaxf((float)hi.x, (float)hi.y));
+    if (AZP) mn = fminf(mn, fminf((float)lo.x, (float)lo.y));
+  }
+};
+
 // Makes the compiler forget what it knows about a unit's bits, so that the values converted for the
 // first pass are not kept alive (at twice the registers of the raw data) for the second.
 template <typename T>
@@ -161,8 +216,16 @@ struct Divisor {
 };
 
 // float_to_int8_rn(v / s) or, with AZP, int32_to_int8(float_to_int32_rn(v / s) + azp), for eight values.
-template <bool AZP>
-__device__ __forceinline__ void quantise8(const float (&v)[kVec], const Divisor& d, int azp, int (&q)[kVec]) {
+template <bool AZP, typename T>
+__device__ __forceinline__ void quantise8(const Raw<T>& raw, const Divisor& d, int azp, int (&q)[kVec]) {
+  float y[kVec];
+  products(raw, d.r, y);
+  auto divide = [&]() {
+    float v[kVec];
+    unpack(raw, v);
+#pragma unroll
+    for (int i = 0; i < kVec; ++i) y[i] = v[i] / d.s;
+  };
   if (!AZP) {
     // Without a zero point only |y| < 129 can end anywhere but at a bound, and there 3 * 2^-23 |y| is less
     // than 2^-15: one constant margin for all eight, taken on the largest distance of a product from its
@@ -171,44 +234,29 @@ __device__ __forceinline__ void quantise8(const float (&v)[kVec], const Divisor&
     // distance - an infinite or NaN input - drops out of the maximum: such a product converts to the same
     // bound, or to 0, as the quotient.
 #pragma clang fp contract(off)
-    float n[kVec], worst = 0.f;
+    float worst = 0.f;
 #pragma unroll
-    for (int i = 0; i < kVec; ++i) {
-      const float y = v[i] * d.r;
-      n[i] = rintf(y);
-      worst = fmaxf(worst, fabsf(y - n[i]));
-    }
+    for (int i = 0; i < kVec; ++i) worst = fmaxf(worst, fabsf(y[i] - rintf(y[i])));
     const bool exact = !d.usable || !(worst <= 0.5f - 0x1p-15f);
-    if (__builtin_amdgcn_ballot_w64(exact)) {
+    if (__builtin_amdgcn_ballot_w64(exact)) divide();
 #pragma unroll
-      for (int i = 0; i < kVec; ++i) n[i] = rintf(v[i] / d.s);
-    }
-#pragma unroll
-    for (int i = 0; i < kVec; ++i) {
-      int r;
-      asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(n[i]));
-      q[i] = min(max(r, -128), 127);
-    }
+    for (int i = 0; i < kVec; ++i) q[i] = float_to_int8_rn(y[i]);
     return;
   }
   // With a zero point any quotient may matter: the margin is relative (a subnormal product has no
   // relative bound and no tie near it either); it reaches 0.5, i.e. sends the unit to the division, from
   // |y| = 2^20.4 on.  One comparison for the largest of the eight; a NaN drops out as above.
-  float y[kVec], worst = 0.f;
+  float worst = 0.f;
   {
 #pragma clang fp contract(off)
 #pragma unroll
     for (int i = 0; i < kVec; ++i) {
-      y[i] = v[i] * d.r;
       const float dist = fabsf(y[i] - rintf(y[i]));  // distance to the nearest integer
       worst = fmaxf(worst, fmaf(fabsf(y[i]), 0x1.8p-22f, dist));
     }
   }
   const bool exact = !d.usable || !(worst < 0.5f - 0x1p-24f);
-  if (__builtin_amdgcn_ballot_w64(exact)) {
-#pragma unroll
-    for (int i = 0; i < kVec; ++i) y[i] = v[i] / d.s;
-  }
+  if (__builtin_amdgcn_ballot_w64(exact)) divide();
 #pragma unroll
   for (int i = 0; i < kVec; ++i) q[i] = int32_to_int8(float_to_int32_rn(y[i]) + azp);
 }
@@ -235,10 +283,8 @@ __global__ __launch_bounds__(256) void static_quant_kernel(const T* __restrict__
 #pragma unroll
     for (int k = 0; k < kStaticUnroll; ++k) {
       const int64_t u = u0 + k * stride;
-      float v[kVec];
       int q[kVec];
-      unpack(raw[k], v);
-      quantise8<AZP>(v, d, azp, q);
+      quantise8<AZP>(raw[k], d, azp, q);
       if (u < units) store_unit<true>(out, u, q, 0, (int)min((int64_t)kVec, total - u * kVec), aligned);
     }
   }
@@ -309,18 +355,15 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict_
   // (reference.h:71-72); the symmetric variant starts its absmax at 0 (reference.h:43)
   float mx = AZP ? 1.17549435e-38f : 0.f;
   float mn = 3.40282347e+38f;
+  UnitScan<T, AZP> whole;
   auto scan = [&](const Raw<T>& raw, int j) {
-    float v[kVec];
-    unpack(raw, v);
     const int rel = (j - first) * kVec - head;  // row position of the unit's element 0
     const int lo = max(-rel, 0), hi = min(hidden - rel, kVec);
     if (lo == 0 && hi == kVec) {  // all but the row's first and last unit
-#pragma unroll
-      for (int i = 0; i < kVec; ++i) {
-        if (AZP) { mx = fmaxf(mx, v[i]); mn = fminf(mn, v[i]); }
-        else mx = fmaxf(mx, fabsf(v[i]));
-      }
+      whole.add(raw, mx, mn);
     } else {
+      float v[kVec];
+      unpack(raw, v);
 #pragma unroll
       for (int i = 0; i < kVec; ++i)
         if (i >= lo && i < hi) {
@@ -335,6 +378,7 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict_
     if (j >= first && j < end) scan(keep[k], j);
   }
   for (int j = lane + KEEP * LANES; j < end; j += LANES) scan(fetch(j), j);
+  whole.fold(mx, mn);
   row_max_min<LANES>(mx, mn, lds);
 
   float scale_val, mul = 0.f;
@@ -352,15 +396,15 @@ __global__ __launch_bounds__(256) void dynamic_quant_kernel(const T* __restrict_
   }
   const Divisor d(scale_val);
   auto emit = [&](Raw<T> raw, int j) {
-    float v[kVec];
     int q[kVec];
     forget(raw);
-    unpack(raw, v);
     if (AZP) {
-      quantise8<true>(v, d, azp_val, q);
+      quantise8<true>(raw, d, azp_val, q);
     } else {
+      float y[kVec];
+      products(raw, mul, y);
 #pragma unroll
-      for (int i = 0; i < kVec; ++i) q[i] = float_to_int8_rn(v[i] * mul);
+      for (int i = 0; i < kVec; ++i) q[i] = float_to_int8_rn(y[i]);
     }
     const int rel = (j - first) * kVec - head;
     store_unit<false>(row_out, j, q, max(-rel, 0), min(hidden - rel, kVec), aligned);

@@ -56,6 +56,57 @@ def test_ragged_rows_wave_and_group_paths(hq, oracle, dtype, tokens, hidden):
         assert np.array_equal(got.cpu().numpy(), want), with_azp
 
 
+def test_fp16_subnormals_and_special_values(hq, oracle):
+    """fp16 rows made of subnormal halves, of the largest halves, and rows that hold -0, infinities (static
+    scale only) and isolated NaNs next to ordinary values (NaN is ignored by the reference's max / min and its quantised
+    value is left out of the comparison): the fp16 kernels multiply the packed halves directly."""
+    import torch
+    rng = np.random.default_rng(77)
+    rows = [rng.standard_normal(5137) * 3e-6,                       # all subnormal
+            rng.standard_normal(5137) * 6e-5,                       # around the smallest normal half
+            np.clip(rng.standard_normal(5137) * 2e4, -65504, 65504),  # up to the largest halves
+            np.where(rng.random(5137) < 0.5, 5.96e-8, -5.96e-8),    # the smallest subnormal, both signs
+            np.where(rng.random(5137) < 0.01, 0.0, rng.standard_normal(5137)) * np.where(rng.random(5137) < 0.5, 1, -1),
+            rng.standard_normal(5137) + 3.0]
+    x = np.stack(rows).astype(np.float16)
+    x[4, 17] = np.float16(-0.0)
+    x = np.concatenate([x, x[:, ::-1]], axis=0)
+    dx = _dev(x)
+    for scale in (1e-7, 3e-6, 0.5, 300.0):
+        for azp in (None, 54):
+            xs = x.copy()
+            if azp is None:  # infinities saturate; with a dynamic scale or a zero point they are undefined
+                xs[2, 5], xs[2, 4000] = np.float16(np.inf), np.float16(-np.inf)
+            if azp is not None:  # int32 overflow of quotient + zero point is undefined in the reference as well
+                with np.errstate(all="ignore"):
+                    xs = np.where(np.abs(x.astype(np.float64) / scale) < 2.0e9, x, np.float16(0))
+            got = hq.static_scaled_int8_quant(_dev(xs), scale, azp)
+            torch.cuda.synchronize()
+            assert np.array_equal(got.cpu().numpy(), oracle.int8_quant_static(xs, scale, azp)), (scale, azp)
+    for with_azp in (False, True):
+        got, gs, gz = hq.dynamic_scaled_int8_quant(dx, with_azp)
+        torch.cuda.synchronize()
+        want, ws, wz = oracle.int8_quant_dynamic(x, with_azp)
+        assert np.array_equal(gs.cpu().numpy(), ws)
+        if with_azp:
+            assert np.array_equal(gz.cpu().numpy(), wz)
+        assert np.array_equal(got.cpu().numpy(), want), with_azp
+    # NaN elements: the row's scale comes from the others, and the others quantise as without the NaN
+    y = x.copy()
+    y[:, 100] = np.float16(np.nan)
+    y[:, 4001] = np.float16(np.nan)
+    keep = np.ones(y.shape[1], bool)
+    keep[[100, 4001]] = False
+    for with_azp in (False, True):
+        got, gs, gz = hq.dynamic_scaled_int8_quant(_dev(y), with_azp)
+        torch.cuda.synchronize()
+        want, ws, wz = oracle.int8_quant_dynamic(y, with_azp)
+        assert np.array_equal(gs.cpu().numpy(), ws)
+        if with_azp:
+            assert np.array_equal(gz.cpu().numpy(), wz)
+        assert np.array_equal(got.cpu().numpy()[:, keep], want[:, keep]), with_azp
+
+
 @pytest.mark.parametrize("scale", [0.1, 0.25, 0.3, 1.0 / 3.0, 7.0, 1e-3, 123.456, 2.0 ** -100, 2.0 ** 100, 2.0 ** -101,
                                    2.0 ** 101, 1e-40, 3e38, -0.5])
 def test_static_division_ties_and_extreme_scales(hq, oracle, scale):
