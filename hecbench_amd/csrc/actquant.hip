@@ -292,13 +292,29 @@ __global__ __launch_bounds__(256) void static_quant_kernel(const T* __restrict__
 
 // ---- dynamic scale: LANES threads per row --------------------------------------------------------
 // Maximum of a and minimum of b over the LANES threads of a row.
+// (Neither is a NaN: the scans drop them.)  Within a wave: lane exchanges inside rows of 16 lanes on the
+// data path of the instruction (DPP), then the four rows through scalar registers; six rounds of
+// shuffles through the LDS crossbar took about three times as long.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float lane_f(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+template <bool MAX>
+__device__ __forceinline__ float wave_extreme(float v) {
+  auto pick = [](float x, float y) { return MAX ? fmaxf(x, y) : fminf(x, y); };
+  v = pick(v, dpp_f<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = pick(v, dpp_f<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = pick(v, dpp_f<0x141>(v));  // row_half_mirror
+  v = pick(v, dpp_f<0x140>(v));  // row_mirror
+  return pick(pick(lane_f(v, 0), lane_f(v, 16)), pick(lane_f(v, 32), lane_f(v, 48)));
+}
 template <int LANES>
 __device__ __forceinline__ void row_max_min(float& a, float& b, float* lds) {
-#pragma unroll
-  for (int m = 32; m > 0; m >>= 1) {
-    a = fmaxf(a, __shfl_xor(a, m));
-    b = fminf(b, __shfl_xor(b, m));
-  }
+  a = wave_extreme<true>(a);
+  b = wave_extreme<false>(b);
   if (LANES > 64) {  // the row spans the workgroup
     const int wv = threadIdx.x >> 6;
     if ((threadIdx.x & 63) == 0) { lds[wv] = a; lds[4 + wv] = b; }
