@@ -5,9 +5,11 @@ Headline (the fields `metric`, `value`, `ms_per_step`, `roofline`): the GPTQ 3-b
 with fp32 activations - achieved HBM GB/s (algorithmic bytes / time per call) and microseconds per call,
 weights rotated over more than 512 MB of distinct buffers so that no call is served from the 256 MB
 Infinity Cache.  The same line carries, under `configs`, the other four benchmark configurations (NF4
-dequantisation, LUT-GEMM, AQLM, batched 3-bit GEMM), each timed the same way with its own roofline object.
+dequantisation, LUT-GEMM, AQLM, batched 3-bit GEMM), each timed the same way with its own roofline object,
+and under `other_kernels` the kernels of the neighbouring benchmarks (gemv fp16 / int8 / int4, mxfp4, the int8
+activation quantisers, the 8-bit dynamic-map quantiser) at the reference programs' run sizes.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--windows R] [--no-cpu] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--windows R] [--no-cpu] [--no-others] [--all]
 
 A step is one library call.  After W warm-up calls, R windows of exactly K back-to-back calls are enqueued
 with a HIP event between windows (on the stream the kernels are launched on); `ms_per_step` is the MEDIAN
@@ -362,6 +364,11 @@ def bench_others(steps, warmup, windows):
     b = 5.0 * nq + 1024
     out["quantize_dynamic8_16777216"] = {"us": secs / st * 1e6, "GBps": b * st / secs / 1e9,
                                          "frac_hbm": b * st / secs / 1e9 / HBM_PEAK_GBS}
+    for name, e in out.items():
+        algo = int(round(e["GBps"] * e["us"] * 1e3))
+        e["algorithmic_bytes_per_call"] = algo
+        e["roofline"] = _roofline_hbm(algo, e["us"], name)
+        e["us"], e["GBps"], e["frac_hbm"] = round(e["us"], 3), round(e["GBps"], 1), round(e["frac_hbm"], 4)
     return out
 
 
@@ -459,7 +466,10 @@ def main():
                     help="timed windows of --steps calls (default: 11, more when --steps is small)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-configs", action="store_true", help="time the headline configuration only")
-    ap.add_argument("--all", action="store_true", help="also time the kernels of the neighbouring benchmarks")
+    ap.add_argument("--no-others", action="store_true",
+                    help="skip the kernels of the neighbouring benchmarks (gemv, mxfp4, quantVLLM, quantBnB)")
+    ap.add_argument("--all", action="store_true",
+                    help="also time the CPU restatements of the other configurations and kernels")
     ap.add_argument("--no-hot", action="store_true", help="skip the hot-cache (single buffer) timing")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 20 plain device copies of 256 MiB (reference point for rocprofv3 "
@@ -516,9 +526,11 @@ def main():
         # the other four benchmark configurations: a few thousand calls each at most
         st = max(1, min(args.steps, 1000))
         result["configs"] = bench_configs(st, min(args.warmup, 100), _windows_for(st, args.windows))
-    if args.all:
+    if not args.no_others:
+        # the kernels of the neighbouring benchmarks (gemv, mxfp4, quantVLLM, quantBnB), shorter loops
         st = max(20, min(args.steps // 4, 500))
-        result["other_kernels"] = bench_others(st, 20, 11)
+        result["other_kernels"] = bench_others(st, 20, _windows_for(st, args.windows) if args.steps < 200 else 11)
+    if args.all and not args.no_others:
         if not args.no_cpu:
             cpu = cpu_others()
             for name, c in cpu.items():
