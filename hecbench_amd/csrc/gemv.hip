@@ -66,6 +66,88 @@ __device__ __forceinline__ float sum8(u4v v, float acc) {
   return acc;
 }
 
+// One step of a wave: R matrix units m[r] (16 bytes per lane and row) against the matching pieces v[] of the
+// vector.  SUM: also add the pieces' elements to vsum (needed once per wave, not once per row group).
+template <int MODE, int R, bool SUM>
+__device__ __forceinline__ void gemv_step(const u4v (&m)[R], const u4v (&v)[Geom<MODE>::kVecUnits], float (&acc)[R],
+                                          float (&acc16)[R], float& vsum) {
+  using G = Geom<MODE>;
+  uint32_t vw[4 * G::kVecUnits];
+#pragma unroll
+  for (int i = 0; i < G::kVecUnits; ++i) { vw[4 * i] = v[i].x; vw[4 * i + 1] = v[i].y; vw[4 * i + 2] = v[i].z; vw[4 * i + 3] = v[i].w; }
+
+  if (MODE == kF16) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const uint32_t mw[4] = {m[r].x, m[r].y, m[r].z, m[r].w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[r] = __builtin_amdgcn_fdot2(as_h2(mw[i]), as_h2(vw[i]), acc[r], false);
+    }
+  } else if (MODE == kI8) {
+    if (SUM) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) vsum = sum8(v[i], vsum);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const uint32_t mw[4] = {m[r].x, m[r].y, m[r].z, m[r].w};
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        // bytes 0..3 of word d are columns 4d..4d+3: vector halves vw[2d].lo, .hi, vw[2d+1].lo, .hi
+        const h2v x01 = as_h2(vw[2 * d]), x23 = as_h2(vw[2 * d + 1]);
+        acc[r] = fmaf((float)x01[0], (float)(int8_t)(mw[d] & 0xffu), acc[r]);
+        acc[r] = fmaf((float)x01[1], (float)(int8_t)((mw[d] >> 8) & 0xffu), acc[r]);
+        acc[r] = fmaf((float)x23[0], (float)(int8_t)((mw[d] >> 16) & 0xffu), acc[r]);
+        acc[r] = fmaf((float)x23[1], (float)(int8_t)(mw[d] >> 24), acc[r]);
+      }
+    }
+  } else {
+    if (SUM) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) vsum = sum8(v[i], vsum);
+    }
+    // word d holds columns 8d..8d+7 in nibbles 0..7; `(w >> 4i) & 0x000f000f` pairs columns
+    // i and i+4, so the vector halves are paired the same way once for all rows
+    uint32_t pv[4][4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      pv[d][0] = __builtin_amdgcn_perm(vw[4 * d + 2], vw[4 * d], 0x05040100u);      // v0 v4
+      pv[d][1] = __builtin_amdgcn_perm(vw[4 * d + 2], vw[4 * d], 0x07060302u);      // v1 v5
+      pv[d][2] = __builtin_amdgcn_perm(vw[4 * d + 3], vw[4 * d + 1], 0x05040100u);  // v2 v6
+      pv[d][3] = __builtin_amdgcn_perm(vw[4 * d + 3], vw[4 * d + 1], 0x07060302u);  // v3 v7
+    }
+    // nibbles 1 and 3 are masked where they stand, four bits up, which makes them 16 times too large:
+    // they go to a second sum that is divided by 16 at the end (5 instead of 7 shift / mask
+    // instructions per word)
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const uint32_t mw[4] = {m[r].x, m[r].y, m[r].z, m[r].w};
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const uint32_t up = mw[d] >> 8;
+        acc[r] = __builtin_amdgcn_fdot2(as_h2(mw[d] & 0x000f000fu), as_h2(pv[d][0]), acc[r], false);
+        acc16[r] = __builtin_amdgcn_fdot2(as_h2(mw[d] & 0x00f000f0u), as_h2(pv[d][1]), acc16[r], false);
+        acc[r] = __builtin_amdgcn_fdot2(as_h2(up & 0x000f000fu), as_h2(pv[d][2]), acc[r], false);
+        acc16[r] = __builtin_amdgcn_fdot2(as_h2(up & 0x00f000f0u), as_h2(pv[d][3]), acc16[r], false);
+      }
+    }
+  }
+}
+
+// Lane sums, zero point and scale, one rounding to fp16: rows row0 .. row0 + R - 1 of a wave.
+template <int MODE, int R>
+__device__ __forceinline__ void gemv_finish(const GemvArgs& a, int row0, const float (&acc)[R], const float (&acc16)[R],
+                                            float vs) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float s = wave_sum(MODE == kI4 ? fmaf(acc16[r], 0.0625f, acc[r]) : acc[r]);
+    if (MODE == kI8) s = a.scale * (s - a.zp * vs);
+    if (MODE == kI4) s = a.scale * (s * 16777216.f - a.zp * vs);  // codes were fp16 subnormals code * 2^-24
+    if (lane == 0 && row0 + r < a.rows) a.res[row0 + r] = (_Float16)s;
+  }
+}
+
 template <int MODE, int R>
 __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
   using G = Geom<MODE>;
@@ -91,72 +173,83 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
     u4v v[G::kVecUnits];
 #pragma unroll
     for (int i = 0; i < G::kVecUnits; ++i) v[i] = a.vec[(size_t)u * G::kVecUnits + i];
-    uint32_t vw[4 * G::kVecUnits];
-#pragma unroll
-    for (int i = 0; i < G::kVecUnits; ++i) { vw[4 * i] = v[i].x; vw[4 * i + 1] = v[i].y; vw[4 * i + 2] = v[i].z; vw[4 * i + 3] = v[i].w; }
+    gemv_step<MODE, R, true>(m, v, acc, acc16, vsum);
+  }
 
-    if (MODE == kF16) {
+  gemv_finish<MODE, R>(a, row0, acc, acc16, MODE == kF16 ? 0.f : wave_sum(vsum));
+}
+
+// The vector in LDS, the workgroups persistent.  A CU returns its loads in issue order and holds about
+// 64 KB of them, whichever cache serves them: every piece of the vector a wave loads next to its matrix
+// rows (as many bytes as the rows themselves for int8 with two rows per wave and int4 with four) takes a
+// place in that queue from the matrix.  Here a workgroup of sixteen waves copies the vector into LDS once
+// (piece i of matrix unit u at [i][u], so that a wave's reads of one piece are contiguous) and then walks
+// over groups of R rows, one group per wave and trip, with nothing but the matrix in the load queue.
+template <int MODE, int R>
+__global__ __launch_bounds__(1024) void gemv_lds_kernel(GemvArgs a, int groups) {
+  using G = Geom<MODE>;
+  extern __shared__ u4v vl[];
+  const int lane = threadIdx.x & 63;
+  const int units = a.n / G::kPerUnit;  // 16-byte units per matrix row
+  const size_t row_bytes = (size_t)units * 16;
+  const int waves = gridDim.x * 16;
+  int grp = blockIdx.x * 16 + (threadIdx.x >> 6);
+
+  auto rows_of = [&](int g, const u4v* (&rowp)[R]) {
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const uint32_t mw[4] = {m[r].x, m[r].y, m[r].z, m[r].w};
+    for (int r = 0; r < R; ++r)
+      rowp[r] = reinterpret_cast<const u4v*>(a.mat + (size_t)min(g * R + r, a.rows - 1) * row_bytes);
+  };
+  // the first matrix units are on their way while the vector is copied
+  const u4v* rowp[R];
+  u4v m[R];
+  rows_of(min(grp, groups - 1), rowp);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[r] = __builtin_amdgcn_fdot2(as_h2(mw[i]), as_h2(vw[i]), acc[r], false);
-      }
-    } else if (MODE == kI8) {
+  for (int r = 0; r < R; ++r) m[r] = __builtin_nontemporal_load(rowp[r] + min(lane, units - 1));
+  for (int t = threadIdx.x; t < units * G::kVecUnits; t += 1024) {
+    const int u = t / G::kVecUnits, i = t % G::kVecUnits;
+    vl[i * units + u] = a.vec[t];
+  }
+  __syncthreads();
+
+  float vs = 0.f;
+  bool first = true;
+  for (; grp < groups; grp += waves) {
+    float acc[R], acc16[R], vsum = 0.f;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) vsum = sum8(v[i], vsum);
+    for (int r = 0; r < R; ++r) acc[r] = acc16[r] = 0.f;
+    for (int u = lane; u < units; u += 64) {
+      u4v cur[R], v[G::kVecUnits];
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const uint32_t mw[4] = {m[r].x, m[r].y, m[r].z, m[r].w};
+      for (int r = 0; r < R; ++r) cur[r] = m[r];
+      // the next step's units (the next group's first ones at the end of a row) before this step's arithmetic
+      if (u + 64 >= units) rows_of(min(grp + waves, groups - 1), rowp);
+      const int un = u + 64 < units ? u + 64 : min(lane, units - 1);
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          // bytes 0..3 of word d are columns 4d..4d+3: vector halves vw[2d].lo, .hi, vw[2d+1].lo, .hi
-          const h2v x01 = as_h2(vw[2 * d]), x23 = as_h2(vw[2 * d + 1]);
-          acc[r] = fmaf((float)x01[0], (float)(int8_t)(mw[d] & 0xffu), acc[r]);
-          acc[r] = fmaf((float)x01[1], (float)(int8_t)((mw[d] >> 8) & 0xffu), acc[r]);
-          acc[r] = fmaf((float)x23[0], (float)(int8_t)((mw[d] >> 16) & 0xffu), acc[r]);
-          acc[r] = fmaf((float)x23[1], (float)(int8_t)(mw[d] >> 24), acc[r]);
-        }
-      }
-    } else {
+      for (int r = 0; r < R; ++r) m[r] = __builtin_nontemporal_load(rowp[r] + un);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) vsum = sum8(v[i], vsum);
-      // word d holds columns 8d..8d+7 in nibbles 0..7; `(w >> 4i) & 0x000f000f` pairs columns
-      // i and i+4, so the vector halves are paired the same way once for all rows
-      uint32_t pv[4][4];
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        pv[d][0] = __builtin_amdgcn_perm(vw[4 * d + 2], vw[4 * d], 0x05040100u);      // v0 v4
-        pv[d][1] = __builtin_amdgcn_perm(vw[4 * d + 2], vw[4 * d], 0x07060302u);      // v1 v5
-        pv[d][2] = __builtin_amdgcn_perm(vw[4 * d + 3], vw[4 * d + 1], 0x05040100u);  // v2 v6
-        pv[d][3] = __builtin_amdgcn_perm(vw[4 * d + 3], vw[4 * d + 1], 0x07060302u);  // v3 v7
-      }
-      // nibbles 1 and 3 are masked where they stand, four bits up, which makes them 16 times too large:
-      // they go to a second sum that is divided by 16 at the end (5 instead of 7 shift / mask
-      // instructions per word)
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const uint32_t mw[4] = {m[r].x, m[r].y, m[r].z, m[r].w};
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          const uint32_t up = mw[d] >> 8;
-          acc[r] = __builtin_amdgcn_fdot2(as_h2(mw[d] & 0x000f000fu), as_h2(pv[d][0]), acc[r], false);
-          acc16[r] = __builtin_amdgcn_fdot2(as_h2(mw[d] & 0x00f000f0u), as_h2(pv[d][1]), acc16[r], false);
-          acc[r] = __builtin_amdgcn_fdot2(as_h2(up & 0x000f000fu), as_h2(pv[d][2]), acc[r], false);
-          acc16[r] = __builtin_amdgcn_fdot2(as_h2(up & 0x00f000f0u), as_h2(pv[d][3]), acc16[r], false);
-        }
-      }
+      for (int i = 0; i < G::kVecUnits; ++i) v[i] = vl[i * units + u];
+      if (first) gemv_step<MODE, R, true>(cur, v, acc, acc16, vsum);
+      else gemv_step<MODE, R, false>(cur, v, acc, acc16, vsum);
     }
+    if (first && MODE != kF16) vs = wave_sum(vsum);
+    first = false;
+    gemv_finish<MODE, R>(a, grp * R, acc, acc16, vs);
   }
+}
 
-  const float vs = MODE == kF16 ? 0.f : wave_sum(vsum);
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    float s = wave_sum(MODE == kI4 ? fmaf(acc16[r], 0.0625f, acc[r]) : acc[r]);
-    if (MODE == kI8) s = a.scale * (s - a.zp * vs);
-    if (MODE == kI4) s = a.scale * (s * 16777216.f - a.zp * vs);  // codes were fp16 subnormals code * 2^-24
-    if (lane == 0 && row0 + r < a.rows) a.res[row0 + r] = (_Float16)s;
-  }
+constexpr size_t kMaxVectorLds = 128 * 1024;  // bytes of the vector the LDS kernel takes (n <= 65536)
+
+template <int MODE, int R>
+int launch_gemv_lds(const GemvArgs& a, int cus, hipStream_t stream) {
+  const size_t smem = (size_t)a.n * 2;
+  static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_lds_kernel<MODE, R>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxVectorLds);
+  if (attr != hipSuccess) return (int)attr;
+  const int groups = (a.rows + R - 1) / R;
+  const int wgs = (groups + 15) / 16;
+  hipLaunchKernelGGL((gemv_lds_kernel<MODE, R>), dim3(wgs < cus ? wgs : cus), dim3(1024), smem, stream, a, groups);
+  return hq_launch_status();
 }
 
 template <int MODE>
@@ -180,6 +273,18 @@ int launch_gemv(const void* mat, const void* vec, void* res, int rows, int n, fl
   // (int4 reads four times as many bytes of the vector per byte of the matrix as fp16: rows per wave pay
   // there even when they leave only eight waves per compute unit - 8192 x 28672: 33.1 us with one row per
   // wave, 25.0 with two, 20.6 with four; fp16 at 4096 x 16384: 23.7 us with one row, 28.0 with two)
+  // The LDS kernel pays where a wave loads as many bytes of the vector as of the matrix and walks over several
+  // row groups: int4 with four rows per wave (32768 x 8192 29.0 -> 24.2 us, 28672 x 8192 25.7 -> 22.5,
+  // 16384 x 28672 41.7 -> 38.8, 16384 x 16384 25.8 -> 25.5); fp16 and int8 gain on some shapes and lose on
+  // others (fp16 16384 x 16384 88.7 -> 83.0 us but 28672 x 8192 70.6 -> 79.0), fewer rows lose throughout.
+  // HQ_GEMV_LDS: 0 never, 1 wherever the vector fits, unset: the rule above.
+  const int lds = hq_tune(HQ_TUNE_GEMV_LDS, -1);
+  const int full = dev->cus * 16;  // waves of a full launch of the LDS kernel
+  if ((size_t)n * 2 <= kMaxVectorLds && (lds == 1 || (lds < 0 && MODE == kI4 && rows >= full * 4))) {
+    if (rows >= full * 4) return launch_gemv_lds<MODE, 4>(a, dev->cus, stream);
+    if (rows >= full * 2) return launch_gemv_lds<MODE, 2>(a, dev->cus, stream);
+    return launch_gemv_lds<MODE, 1>(a, dev->cus, stream);
+  }
   constexpr int RMAX = MODE == kI4 ? 4 : 2;
   constexpr int kMinWaves = MODE == kI4 ? 8 : 16;  // per compute unit
   if (rows >= dev->cus * kMinWaves * RMAX) {

@@ -46,6 +46,34 @@ def test_vs_oracle(hq, oracle, rows, n, mode):
 
 
 @pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("rows,n", [(512, 512), (37, 1024), (1, 32), (9000, 2048), (16390, 64), (4099, 4096),
+                                    (16385, 1056), (40, 65536)])
+def test_vector_in_lds_kernel(hq, oracle, tunable, rows, n, mode):
+    """The persistent kernel that keeps the vector in LDS (by default only int4 with many rows), forced on
+    shapes with one, two and four rows per wave, ragged row counts, rows shorter than one step of a wave
+    and the longest vector it takes; and the ordinary kernel forced where the rule would pick the other:
+    both must give the same bits, and the oracle's result."""
+    import torch
+    mat, vec = gemv_problem(rows * 3 + n + mode, rows, n, mode)
+    _, r64 = oracle.gemv(mat, mode, vec, SCALE, ZP)
+    tunable("HQ_GEMV_LDS", 1)
+    lds, _, _ = _run(hq, mat, vec, mode)
+    _check(lds, r64)
+    tunable("HQ_GEMV_LDS", 0)
+    plain, _, _ = _run(hq, mat, vec, mode)
+    assert np.array_equal(lds.view(np.uint16), plain.view(np.uint16))
+
+
+def test_vector_too_long_for_lds(hq, oracle, tunable):
+    """Beyond 65536 elements the vector does not fit: the ordinary kernel runs even when the other is asked for."""
+    mat, vec = gemv_problem(5, 24, 65536 + 32, 2)
+    tunable("HQ_GEMV_LDS", 1)
+    got, _, _ = _run(hq, mat, vec, 2)
+    _, r64 = oracle.gemv(mat, 2, vec, SCALE, ZP)
+    _check(got, r64)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2])
 def test_signed_data_and_extremes(hq, oracle, mode):
     """Signed vector entries (cancellation) and the extreme codes -128 / 127 / 0 / 15."""
     rng = np.random.default_rng(3)
