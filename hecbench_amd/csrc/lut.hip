@@ -300,7 +300,13 @@ constexpr int kDigQuad = 4 * 4 * 32 + 16;  // digits of one quad [k-word][digit]
 constexpr int planes_of_set(int nb, int s) { return nb - 3 * s < 3 ? nb - 3 * s : 3; }
 
 template <int NB, int QUADS, int WAVES, bool BIAS, bool RAGGED, bool ONE_ROUND>
-__global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(LutArgs a) {
+__global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(
+    const uint32_t* bW_, const _Float16* x_, const _Float16* alpha_, int K_, int N_, int nb_, int G_, int kslice_,
+    int nsplit_, int strict_, const _Float16* qbias_, _Float16* y_, float* partial_, unsigned* counters_) {
+  // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
+  LutArgs a;
+  a.bW = bW_; a.alpha = alpha_; a.qbias = qbias_; a.x = x_; a.y = y_; a.partial = partial_; a.counters = counters_;
+  a.K = K_; a.N = N_; a.nb = nb_; a.G = G_; a.kslice = kslice_; a.nsplit = nsplit_; a.strict = strict_;
   constexpr int SETS = (NB + 2) / 3;
   extern __shared__ float lds[];
   char* xs = reinterpret_cast<char*>(lds);                                   // [waves][QUADS][kDigQuad]
@@ -599,7 +605,13 @@ constexpr int kGroupedQuadBytes = 20 * kLutRow;  // sixteen digit rows and up to
 constexpr int kGroupedRedBytes = 20 * 64 * 4;  // a wave's final sums: twenty columns of 64 outputs
 
 template <int NB, int GS, int QUADS, int WAVES, bool BIAS, bool RAGGED>
-__global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(LutArgs a) {
+__global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(
+    const uint32_t* bW_, const _Float16* x_, const _Float16* alpha_, int K_, int N_, int nb_, int G_, int kslice_,
+    int nsplit_, int strict_, const _Float16* qbias_, _Float16* y_, float* partial_, unsigned* counters_) {
+  // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
+  LutArgs a;
+  a.bW = bW_; a.alpha = alpha_; a.qbias = qbias_; a.x = x_; a.y = y_; a.partial = partial_; a.counters = counters_;
+  a.K = K_; a.N = N_; a.nb = nb_; a.G = G_; a.kslice = kslice_; a.nsplit = nsplit_; a.strict = strict_;
   constexpr int kWaveBytes = QUADS * kGroupedQuadBytes > kGroupedRedBytes ? QUADS * kGroupedQuadBytes : kGroupedRedBytes;
   extern __shared__ float lds[];
   char* xs = reinterpret_cast<char*>(lds);  // [waves][kWaveBytes]: operands in the loop, the final sums after it
@@ -814,7 +826,7 @@ int launch_bcq_grouped(const LutArgs& a, bool ragged, hipStream_t stream) {
   const size_t smem = (size_t)WAVES * kWaveBytes + (size_t)WAVES * 4;
   const dim3 grid((a.N + 63) / 64), block(WAVES * 64);
 #define HQ_LUT_GO(BIAS, RAG) \
-  hipLaunchKernelGGL((bcq_mfma_grouped_kernel<NB, GS, QUADS, WAVES, BIAS, RAG>), grid, block, smem, stream, a)
+  hipLaunchKernelGGL((bcq_mfma_grouped_kernel<NB, GS, QUADS, WAVES, BIAS, RAG>), grid, block, smem, stream, a.bW, a.x, a.alpha, a.K, a.N, a.nb, a.G, a.kslice, a.nsplit, a.strict, a.qbias, a.y, a.partial, a.counters)
   if (a.qbias) { if (ragged) HQ_LUT_GO(true, true); else HQ_LUT_GO(true, false); }
   else { if (ragged) HQ_LUT_GO(false, true); else HQ_LUT_GO(false, false); }
 #undef HQ_LUT_GO
@@ -865,8 +877,10 @@ int launch_bcq_planes(LutArgs a, bool ragged, int cus, hipStream_t stream) {
   const bool one_round = rpw == 1;
 #define HQ_LUT_GO(BIAS, RAG)                                                                                        \
   do {                                                                                                              \
-    if (one_round) hipLaunchKernelGGL((bcq_planes_kernel<NB, QUADS, WAVES, BIAS, RAG, true>), grid, block, smem, stream, a); \
-    else hipLaunchKernelGGL((bcq_planes_kernel<NB, QUADS, WAVES, BIAS, RAG, false>), grid, block, smem, stream, a); \
+    if (one_round) hipLaunchKernelGGL((bcq_planes_kernel<NB, QUADS, WAVES, BIAS, RAG, true>), grid, block, smem, stream, \
+                                       a.bW, a.x, a.alpha, a.K, a.N, a.nb, a.G, a.kslice, a.nsplit, a.strict, a.qbias, a.y, a.partial, a.counters); \
+    else hipLaunchKernelGGL((bcq_planes_kernel<NB, QUADS, WAVES, BIAS, RAG, false>), grid, block, smem, stream, \
+                            a.bW, a.x, a.alpha, a.K, a.N, a.nb, a.G, a.kslice, a.nsplit, a.strict, a.qbias, a.y, a.partial, a.counters); \
   } while (0)
   if (a.qbias) { if (ragged) HQ_LUT_GO(true, true); else HQ_LUT_GO(true, false); }
   else { if (ragged) HQ_LUT_GO(false, true); else HQ_LUT_GO(false, false); }

@@ -119,7 +119,15 @@ __device__ __forceinline__ constexpr int step_off(int s) {
 // with only the first step's loads at the top of a round and step s + 1 of the next round before the
 // arithmetic of step s.
 template <int WAVES, int STEPS, bool XF16, int ROUNDS>
-__global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(Q3Args a) {
+__global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w_, const void* x_, int K_, int N_, int gpw_,
+                                                              int nsplit_, int x_f16_, unsigned flags_,
+                                                              const float* scales_, const float* zeros_, float* y_,
+                                                              float* partial_, unsigned* counters_) {
+  // leading scalars rather than the struct: those are preloaded into scalar registers (the first 14 dwords,
+  // i.e. everything the loads and the staging need; y, partial and counters are fetched for the tail)
+  Q3Args a;
+  a.x = x_; a.w = w_; a.scales = scales_; a.zeros = zeros_; a.y = y_; a.partial = partial_; a.counters = counters_;
+  a.K = K_; a.N = N_; a.gpw = gpw_; a.nsplit = nsplit_; a.x_f16 = x_f16_; a.flags = flags_;
   // LDS: dig[WAVES][STEPS * kStepBytes] | red[WAVES][8][kRedStride] | part[WAVES][64] | xsum[WAVES]
   extern __shared__ uint4 smem[];
   char* dig = reinterpret_cast<char*>(smem);
@@ -430,7 +438,8 @@ int launch_matvec_t(const Q3Args& a, int ntiles, hipStream_t stream) {
                           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
   if (attr != hipSuccess) return (int)attr;
   hipLaunchKernelGGL((q3_matvec_kernel<WAVES, STEPS, XF16, ROUNDS>), dim3(ntiles, a.nsplit), dim3(WAVES * 64), smem,
-                     stream, a);
+                     stream, a.w, a.x, a.K, a.N, a.gpw, a.nsplit, a.x_f16, a.flags, a.scales, a.zeros, a.y, a.partial,
+                     a.counters);
   return hq_launch_status();
 }
 template <int WAVES, int STEPS>

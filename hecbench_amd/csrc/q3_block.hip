@@ -360,14 +360,26 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
 
 // One and two passes: at most 128 registers, so that two workgroups share a compute unit.
 template <int PASSES, bool MULTI>
-__global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void q3_block_kernel(BlockArgs a) {
+__global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void q3_block_kernel(
+                   const uint32_t* w_, const _Float16* x_, int K_, int N_, int M_, int nsplit_, int rpw_, unsigned flags_,
+                   const float* scales_, const float* zeros_, float* y_, float* partial_, unsigned* counters_) {
+  // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
+  BlockArgs a;
+  a.x = x_; a.w = w_; a.scales = scales_; a.zeros = zeros_; a.y = y_; a.partial = partial_; a.counters = counters_;
+  a.K = K_; a.N = N_; a.M = M_; a.nsplit = nsplit_; a.rpw = rpw_; a.flags = flags_;
   q3_block_body<PASSES, MULTI>(a);
 }
 // Three passes (9 ... 12 rows) take 127 registers and more time than two workgroups per compute unit leave
 // room for; they run where the launch has at most one workgroup per compute unit and is a matter of latency
 // (K=4096, N=11008: 11.2-12.7 us against the batched GEMM's 14.7; four passes: 16.1 against 14.9 at 16 rows).
 template <int PASSES>
-__global__ __launch_bounds__(kWaves * 64) void q3_block_kernel_many(BlockArgs a) {
+__global__ __launch_bounds__(kWaves * 64) void q3_block_kernel_many(
+                   const uint32_t* w_, const _Float16* x_, int K_, int N_, int M_, int nsplit_, int rpw_, unsigned flags_,
+                   const float* scales_, const float* zeros_, float* y_, float* partial_, unsigned* counters_) {
+  // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
+  BlockArgs a;
+  a.x = x_; a.w = w_; a.scales = scales_; a.zeros = zeros_; a.y = y_; a.partial = partial_; a.counters = counters_;
+  a.K = K_; a.N = N_; a.M = M_; a.nsplit = nsplit_; a.rpw = rpw_; a.flags = flags_;
   q3_block_body<PASSES, false>(a);
 }
 
@@ -377,7 +389,8 @@ int launch_block(const BlockArgs& a, hipStream_t stream) {
   static const hipError_t attr =
       hipFuncSetAttribute(reinterpret_cast<const void*>(KERNEL), hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (attr != hipSuccess) return (int)attr;
-  hipLaunchKernelGGL(KERNEL, dim3((a.N + 63) / 64, a.nsplit), dim3(kWaves * 64), smem, stream, a);
+  hipLaunchKernelGGL(KERNEL, dim3((a.N + 63) / 64, a.nsplit), dim3(kWaves * 64), smem, stream, a.w, a.x, a.K, a.N, a.M,
+                     a.nsplit, a.rpw, a.flags, a.scales, a.zeros, a.y, a.partial, a.counters);
   return hq_launch_status();
 }
 
