@@ -46,7 +46,14 @@ __device__ __forceinline__ float dot8(u4v e, u4v xv, float acc) {
 }
 
 template <int ROWS>
-__global__ __launch_bounds__(256) void aqlm_matvec_kernel(AqlmArgs a) {
+__global__ __launch_bounds__(256) void aqlm_matvec_kernel(const u4v* codes_, const u4v* codebooks_, const u4v* x_, int M_, int K_, int cb_stride_,
+                                                         int cb0_, int cb1_, int cb2_, int cb3_,
+                                                         const _Float16* scales_, _Float16* y_) {
+  // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
+  AqlmArgs a;
+  a.codes = codes_; a.codebooks = codebooks_; a.scales = scales_; a.x = x_; a.y = y_;
+  a.M = M_; a.K = K_; a.cb_stride = cb_stride_;
+  a.cb_sizes[0] = cb0_; a.cb_sizes[1] = cb1_; a.cb_sizes[2] = cb2_; a.cb_sizes[3] = cb3_;
   const int lane = threadIdx.x & 63;
   // Workgroups b, b + 8, b + 16, ... run on the same XCD; inside every 64 of them the row blocks are dealt
   // out so that the eight workgroups whose results share a 128-byte line of y are on one XCD (its L2 then
@@ -133,8 +140,8 @@ extern "C" int hq_aqlm_matvec(const int16_t* codes, const void* codebooks, const
   }
   const int nwaves = (M + rows - 1) / rows;
   const int blocks = (nwaves + 3) / 4;
-  if (rows == 4) hipLaunchKernelGGL(aqlm_matvec_kernel<4>, dim3(blocks), dim3(256), 0, stream, a);
-  else if (rows == 2) hipLaunchKernelGGL(aqlm_matvec_kernel<2>, dim3(blocks), dim3(256), 0, stream, a);
-  else hipLaunchKernelGGL(aqlm_matvec_kernel<1>, dim3(blocks), dim3(256), 0, stream, a);
+  if (rows == 4) hipLaunchKernelGGL(aqlm_matvec_kernel<4>, dim3(blocks), dim3(256), 0, stream, a.codes, a.codebooks, a.x, a.M, a.K, a.cb_stride, a.cb_sizes[0], a.cb_sizes[1], a.cb_sizes[2], a.cb_sizes[3], a.scales, a.y);
+  else if (rows == 2) hipLaunchKernelGGL(aqlm_matvec_kernel<2>, dim3(blocks), dim3(256), 0, stream, a.codes, a.codebooks, a.x, a.M, a.K, a.cb_stride, a.cb_sizes[0], a.cb_sizes[1], a.cb_sizes[2], a.cb_sizes[3], a.scales, a.y);
+  else hipLaunchKernelGGL(aqlm_matvec_kernel<1>, dim3(blocks), dim3(256), 0, stream, a.codes, a.codebooks, a.x, a.M, a.K, a.cb_stride, a.cb_sizes[0], a.cb_sizes[1], a.cb_sizes[2], a.cb_sizes[3], a.scales, a.y);
   return hq_launch_status();
 }

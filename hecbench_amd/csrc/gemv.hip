@@ -149,7 +149,11 @@ __device__ __forceinline__ void gemv_finish(const GemvArgs& a, int row0, const f
 }
 
 template <int MODE, int R>
-__global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
+__global__ __launch_bounds__(256) void gemv_kernel(const char* mat_, const u4v* vec_, _Float16* res_, int rows_, int n_, float scale_,
+                                                  float zp_) {
+  // leading scalars, not the struct: the arguments arrive preloaded in scalar registers
+  GemvArgs a;
+  a.mat = mat_; a.vec = vec_; a.res = res_; a.rows = rows_; a.n = n_; a.scale = scale_; a.zp = zp_;
   using G = Geom<MODE>;
   const int lane = threadIdx.x & 63;
   const int wave = (blockIdx.x * 256 + threadIdx.x) >> 6;
@@ -186,7 +190,11 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
 // (piece i of matrix unit u at [i][u], so that a wave's reads of one piece are contiguous) and then walks
 // over groups of R rows, one group per wave and trip, with nothing but the matrix in the load queue.
 template <int MODE, int R>
-__global__ __launch_bounds__(1024) void gemv_lds_kernel(GemvArgs a, int groups) {
+__global__ __launch_bounds__(1024) void gemv_lds_kernel(const char* mat_, const u4v* vec_, _Float16* res_, int rows_, int n_, float scale_,
+                                                       float zp_, int groups) {
+  // leading scalars, not the struct: the arguments arrive preloaded in scalar registers
+  GemvArgs a;
+  a.mat = mat_; a.vec = vec_; a.res = res_; a.rows = rows_; a.n = n_; a.scale = scale_; a.zp = zp_;
   using G = Geom<MODE>;
   extern __shared__ u4v vl[];
   const int lane = threadIdx.x & 63;
@@ -248,7 +256,7 @@ int launch_gemv_lds(const GemvArgs& a, int cus, hipStream_t stream) {
   if (attr != hipSuccess) return (int)attr;
   const int groups = (a.rows + R - 1) / R;
   const int wgs = (groups + 15) / 16;
-  hipLaunchKernelGGL((gemv_lds_kernel<MODE, R>), dim3(wgs < cus ? wgs : cus), dim3(1024), smem, stream, a, groups);
+  hipLaunchKernelGGL((gemv_lds_kernel<MODE, R>), dim3(wgs < cus ? wgs : cus), dim3(1024), smem, stream, a.mat, a.vec, a.res, a.rows, a.n, a.scale, a.zp, groups);
   return hq_launch_status();
 }
 
@@ -289,12 +297,12 @@ int launch_gemv(const void* mat, const void* vec, void* res, int rows, int n, fl
   constexpr int kMinWaves = MODE == kI4 ? 8 : 16;  // per compute unit
   if (rows >= dev->cus * kMinWaves * RMAX) {
     const int waves = (rows + RMAX - 1) / RMAX;
-    hipLaunchKernelGGL((gemv_kernel<MODE, RMAX>), dim3((waves + 3) / 4), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((gemv_kernel<MODE, RMAX>), dim3((waves + 3) / 4), dim3(256), 0, stream, a.mat, a.vec, a.res, a.rows, a.n, a.scale, a.zp);
   } else if (RMAX > 2 && rows >= dev->cus * kMinWaves * 2) {
     const int waves = (rows + 1) / 2;
-    hipLaunchKernelGGL((gemv_kernel<MODE, 2>), dim3((waves + 3) / 4), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((gemv_kernel<MODE, 2>), dim3((waves + 3) / 4), dim3(256), 0, stream, a.mat, a.vec, a.res, a.rows, a.n, a.scale, a.zp);
   } else {
-    hipLaunchKernelGGL((gemv_kernel<MODE, 1>), dim3((rows + 3) / 4), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((gemv_kernel<MODE, 1>), dim3((rows + 3) / 4), dim3(256), 0, stream, a.mat, a.vec, a.res, a.rows, a.n, a.scale, a.zp);
   }
   return hq_launch_status();
 }

@@ -163,7 +163,15 @@ struct GemmArgs {
 // depth itself, 2 to 5 steps, changes little: what a workgroup moves through its CU's L1 - all of the
 // re-ordered activations, 1 MB, next to 0.4 MB of weights - bounds the loop, not the latency.)
 template <int MB>  // 32-row blocks of activations
-__global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(GemmArgs a) {
+__global__ __launch_bounds__(kWaves * 64) void q3_gemm_kernel(const uint32_t* w_, const u4v* Ap_, int M_, int K_, int N_,
+                                                             int Gpad_, int nsplit_, int spp_, unsigned flags_,
+                                                             const float* scales_, const float* zeros_,
+                                                             const float* rowsum_, const float* rowinv_, float* out_,
+                                                             float* partial_) {
+  // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
+  GemmArgs a;
+  a.w = w_; a.Ap = Ap_; a.rowsum = rowsum_; a.rowinv = rowinv_; a.scales = scales_; a.zeros = zeros_; a.out = out_;
+  a.partial = partial_; a.M = M_; a.K = K_; a.N = N_; a.Gpad = Gpad_; a.nsplit = nsplit_; a.spp = spp_; a.flags = flags_;
   constexpr int Mpad = 32 * MB;
   extern __shared__ u4v lds[];  // used by the final reduction only
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
@@ -313,7 +321,8 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream) {
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (attr != hipSuccess) return (int)attr;
   const int ntiles = (a.N + kTileN - 1) / kTileN;
-  hipLaunchKernelGGL((q3_gemm_kernel<MB>), dim3(ntiles, a.nsplit), dim3(kWaves * 64), smem, stream, a);
+  hipLaunchKernelGGL((q3_gemm_kernel<MB>), dim3(ntiles, a.nsplit), dim3(kWaves * 64), smem, stream, a.w, a.Ap, a.M, a.K,
+                     a.N, a.Gpad, a.nsplit, a.spp, a.flags, a.scales, a.zeros, a.rowsum, a.rowinv, a.out, a.partial);
   int rc = hq_launch_status();
   if (rc != HQ_OK || a.nsplit == 1) return rc;
   hipLaunchKernelGGL(q3_gemm_reduce, dim3(ntiles, (a.M + 7) / 8 < 8 ? (a.M + 7) / 8 : 8), dim3(256), 0, stream, a, 32 * MB);
