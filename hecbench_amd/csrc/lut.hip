@@ -301,9 +301,10 @@ constexpr int planes_of_set(int nb, int s) { return nb - 3 * s < 3 ? nb - 3 * s 
 
 template <int NB, int QUADS, int WAVES, bool BIAS, bool RAGGED, bool ONE_ROUND>
 __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(
-    const uint32_t* bW_, const _Float16* x_, const _Float16* alpha_, int K_, int N_, int nb_, int G_, int kslice_,
-    int nsplit_, int strict_, const _Float16* qbias_, _Float16* y_, float* partial_, unsigned* counters_) {
-  // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
+    const uint32_t* bW_, const _Float16* x_, const _Float16* alpha_, const _Float16* qbias_, int K_, int N_, int nb_,
+    int G_, int kslice_, int nsplit_, int strict_, _Float16* y_, float* partial_, unsigned* counters_) {
+  // leading scalars, not the struct: the first 14 dwords of the arguments (all that the loads need) arrive
+  // preloaded in scalar registers
   LutArgs a;
   a.bW = bW_; a.alpha = alpha_; a.qbias = qbias_; a.x = x_; a.y = y_; a.partial = partial_; a.counters = counters_;
   a.K = K_; a.N = N_; a.nb = nb_; a.G = G_; a.kslice = kslice_; a.nsplit = nsplit_; a.strict = strict_;
@@ -606,9 +607,10 @@ constexpr int kGroupedRedBytes = 20 * 64 * 4;  // a wave's final sums: twenty co
 
 template <int NB, int GS, int QUADS, int WAVES, bool BIAS, bool RAGGED>
 __global__ __launch_bounds__(WAVES * 64) void bcq_mfma_grouped_kernel(
-    const uint32_t* bW_, const _Float16* x_, const _Float16* alpha_, int K_, int N_, int nb_, int G_, int kslice_,
-    int nsplit_, int strict_, const _Float16* qbias_, _Float16* y_, float* partial_, unsigned* counters_) {
-  // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
+    const uint32_t* bW_, const _Float16* x_, const _Float16* alpha_, const _Float16* qbias_, int K_, int N_, int nb_,
+    int G_, int kslice_, int nsplit_, int strict_, _Float16* y_, float* partial_, unsigned* counters_) {
+  // leading scalars, not the struct: the first 14 dwords of the arguments (all that the loads need) arrive
+  // preloaded in scalar registers
   LutArgs a;
   a.bW = bW_; a.alpha = alpha_; a.qbias = qbias_; a.x = x_; a.y = y_; a.partial = partial_; a.counters = counters_;
   a.K = K_; a.N = N_; a.nb = nb_; a.G = G_; a.kslice = kslice_; a.nsplit = nsplit_; a.strict = strict_;
@@ -826,7 +828,7 @@ int launch_bcq_grouped(const LutArgs& a, bool ragged, hipStream_t stream) {
   const size_t smem = (size_t)WAVES * kWaveBytes + (size_t)WAVES * 4;
   const dim3 grid((a.N + 63) / 64), block(WAVES * 64);
 #define HQ_LUT_GO(BIAS, RAG) \
-  hipLaunchKernelGGL((bcq_mfma_grouped_kernel<NB, GS, QUADS, WAVES, BIAS, RAG>), grid, block, smem, stream, a.bW, a.x, a.alpha, a.K, a.N, a.nb, a.G, a.kslice, a.nsplit, a.strict, a.qbias, a.y, a.partial, a.counters)
+  hipLaunchKernelGGL((bcq_mfma_grouped_kernel<NB, GS, QUADS, WAVES, BIAS, RAG>), grid, block, smem, stream, a.bW, a.x, a.alpha, a.qbias, a.K, a.N, a.nb, a.G, a.kslice, a.nsplit, a.strict, a.y, a.partial, a.counters)
   if (a.qbias) { if (ragged) HQ_LUT_GO(true, true); else HQ_LUT_GO(true, false); }
   else { if (ragged) HQ_LUT_GO(false, true); else HQ_LUT_GO(false, false); }
 #undef HQ_LUT_GO
@@ -878,9 +880,9 @@ int launch_bcq_planes(LutArgs a, bool ragged, int cus, hipStream_t stream) {
 #define HQ_LUT_GO(BIAS, RAG)                                                                                        \
   do {                                                                                                              \
     if (one_round) hipLaunchKernelGGL((bcq_planes_kernel<NB, QUADS, WAVES, BIAS, RAG, true>), grid, block, smem, stream, \
-                                       a.bW, a.x, a.alpha, a.K, a.N, a.nb, a.G, a.kslice, a.nsplit, a.strict, a.qbias, a.y, a.partial, a.counters); \
+                                       a.bW, a.x, a.alpha, a.qbias, a.K, a.N, a.nb, a.G, a.kslice, a.nsplit, a.strict, a.y, a.partial, a.counters); \
     else hipLaunchKernelGGL((bcq_planes_kernel<NB, QUADS, WAVES, BIAS, RAG, false>), grid, block, smem, stream, \
-                            a.bW, a.x, a.alpha, a.K, a.N, a.nb, a.G, a.kslice, a.nsplit, a.strict, a.qbias, a.y, a.partial, a.counters); \
+                            a.bW, a.x, a.alpha, a.qbias, a.K, a.N, a.nb, a.G, a.kslice, a.nsplit, a.strict, a.y, a.partial, a.counters); \
   } while (0)
   if (a.qbias) { if (ragged) HQ_LUT_GO(true, true); else HQ_LUT_GO(true, false); }
   else { if (ragged) HQ_LUT_GO(false, true); else HQ_LUT_GO(false, false); }
