@@ -208,11 +208,13 @@ extern "C" int hq_dequant_nf4(const uint8_t* packed, const float* absmax, void* 
   if (mode == MM)                                                                                            \
     hipLaunchKernelGGL((dequant4_kernel<U, MM, NT>), dim3((unsigned)blocks), dim3(256), 0, stream, pw, absmax, \
                        (u4v*)out_fp16, nwords, blocksize, shift, table);
-    // Pipelined variant, eight (large inputs: four) workgroups per CU: measured 7.2 us against 7.5 us for the
-    // one-shot grid at 4096x4096 and 25.5 against 27.0 us at 2^26 elements; from 2^28 elements on the one-shot
-    // grid is the faster one (484 against 507 us at 2^30), so the variant is kept to the mid sizes.
+    // Pipelined variant, up to eight workgroups per CU, fewer for larger inputs (us per call, one-shot grid /
+    // 2 / 4 / 8 workgroups per CU): 2^19 elements 5.17 / 4.11 / 4.13 / 4.11, 2^21 5.23 / 3.97 / 3.94 / 3.96,
+    // 2^23 5.87 / 4.86 / 4.74 / 4.70, 2^24 (4096 x 4096) 7.78 / 7.44 / 7.10 / 7.20, 2^25 14.4 / 13.2 / 13.1 / 13.3,
+    // 2^26 26.8 / 24.7 / 25.3 / 25.3, 2^27 51.5 / 47.3 / 49.8 / -; from 2^28 elements on the one-shot grid is the
+    // faster one (121.0 against 122.6 with four and 168 with two; 484 against 507 us at 2^30).
     int pipe = hq_tune(HQ_TUNE_NF4_PIPE, -1);
-    if (pipe < 0) pipe = nwords < (1 << 19) || nwords > (1 << 25) ? 0 : (nwords <= (1 << 21) ? 8 : 4);
+    if (pipe < 0) pipe = nwords >= (1 << 25) ? 0 : (nwords <= (1 << 20) ? 8 : (nwords <= (1 << 22) ? 4 : 2));
     if (mode == 0 && pipe > 0 && shift >= 3 && nwords < ((int64_t)1 << 31)) {
       constexpr int PU = 4;
       const int64_t nch = (nwords + 256 * PU - 1) / (256 * PU);

@@ -25,6 +25,18 @@ def test_bit_exact(hq, oracle, n, blocksize, table):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("pipe", [0, 1, 2, 8])
+@pytest.mark.parametrize("n,blocksize", [(1 << 20, 64), (4096 * 1100 + 8 * 37 + 3, 64), (8, 8), (1032, 128), (100000, 64)])
+def test_both_launch_variants(hq, oracle, tunable, n, blocksize, pipe):
+    """The one-shot grid (by default only beyond 2^28 elements) and the persistent variant with one, two and
+    eight workgroups per compute unit, forced on sizes from one word up: same bits."""
+    tunable("HQ_NF4_PIPE", pipe)
+    packed, absmax = oa.make_nf4_problem(n + pipe, n, blocksize)
+    got = _run(hq, packed, absmax, n, blocksize, 0)
+    want = oracle.dequant_4bit(packed, absmax, n, blocksize, 0).view(np.uint16)
+    assert np.array_equal(got, want)
+
+
 def test_all_codes_all_roundings(hq, oracle):
     """Every byte value against absmax values that exercise fp16 rounding,
     fp16 subnormal results and overflow to infinity."""
