@@ -279,7 +279,9 @@ extern "C" int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* 
   if (rc != HQ_OK) return rc;
   const int vec_ok = !((uintptr_t)A & 15) && !((uintptr_t)out & 3);
   int64_t blocks = (n / 4 + 256 * kQuads - 1) / (256 * kQuads);  // one trip of the fast path each, or grid-stride
-  const int64_t cap = (int64_t)dev->cus * hq_tune(HQ_TUNE_Q8_WGS, 5);
+  // workgroups per CU of the persistent fast path: five up to 2^24 elements (16.5 us; two 17.8, eight 19.2),
+  // two from 2^25 on (2^25: 30.5 against 31.4 us with five, 2^26: 55.4 against 59.7, 2^27: 108.6 against 123.2)
+  const int64_t cap = (int64_t)dev->cus * hq_tune(HQ_TUNE_Q8_WGS, n >= ((int64_t)1 << 25) ? 2 : 5);
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(quantize8_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, code, A, out, n,
