@@ -12,7 +12,8 @@ activation quantisers, the 8-bit dynamic-map quantiser) at the reference program
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--windows R] [--no-cpu] [--no-others] [--all]
 
 A step is one library call.  After W warm-up calls, R windows of exactly K back-to-back calls are enqueued
-with a HIP event between windows (on the stream the kernels are launched on); `ms_per_step` is the MEDIAN
+with a HIP event between windows (on the stream the kernels are launched on; timing-only events without a
+system-scope fence); `ms_per_step` is the MEDIAN
 window divided by K, the fastest and slowest windows are reported next to it.  Prints ONE JSON line."""
 import argparse
 import ctypes
@@ -53,6 +54,35 @@ def _windows_for(steps, windows):
     return max(11, min(201, (20000 // max(steps, 1)) | 1))
 
 
+_HIP = None
+
+
+def _hip_runtime():
+    """The HIP runtime this process already runs on (the copy torch loaded), for events created with
+    hipEventDisableSystemFence: events that only measure time need no system-scope fence, whose cache
+    write-back and invalidation would otherwise be charged to the first call of the next window (0.1 us per
+    call in windows of 20 calls).  None if it cannot be found."""
+    global _HIP
+    if _HIP is None:
+        _HIP = False
+        try:
+            with open("/proc/self/maps") as maps:
+                paths = {line.split()[-1] for line in maps if "libamdhip64.so" in line}
+            if len(paths) == 1:
+                lib = ctypes.CDLL(paths.pop())
+                lib.hipEventCreateWithFlags.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint]
+                lib.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+                lib.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+                lib.hipEventDestroy.argtypes = [ctypes.c_void_p]
+                _HIP = lib
+        except (OSError, AttributeError):
+            _HIP = False
+    return _HIP or None
+
+
+HIP_EVENT_DISABLE_SYSTEM_FENCE = 0x20000000
+
+
 def _time_windows(fn, n_buffers, steps, warmup, windows):
     """R windows of `steps` back-to-back calls on torch's current stream (the stream the kernels are
     enqueued on), a HIP event between windows, one synchronisation at the end.  Returns the sorted list of
@@ -61,16 +91,44 @@ def _time_windows(fn, n_buffers, steps, warmup, windows):
     for i in range(warmup):
         fn(i % n_buffers)
     torch.cuda.synchronize()
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(windows + 1)]
+    hip = _hip_runtime()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    raw = []
+    if hip is not None:
+        for _ in range(windows + 1):
+            e = ctypes.c_void_p()
+            if hip.hipEventCreateWithFlags(ctypes.byref(e), HIP_EVENT_DISABLE_SYSTEM_FENCE) != 0:
+                for made in raw:
+                    hip.hipEventDestroy(made)
+                raw, hip = [], None
+                break
+            raw.append(e)
+    if hip is None:
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(windows + 1)]
+        record = lambda j: ev[j].record()
+    else:
+        def record(j):
+            if hip.hipEventRecord(raw[j], stream) != 0:
+                raise RuntimeError("hipEventRecord failed")
     k = 0
-    ev[0].record()
+    record(0)
     for w in range(windows):
         for _ in range(steps):
             fn(k % n_buffers)
             k += 1
-        ev[w + 1].record()
+        record(w + 1)
     torch.cuda.synchronize()
-    return sorted(ev[w].elapsed_time(ev[w + 1]) * 1e-3 for w in range(windows))
+    if hip is None:
+        return sorted(ev[w].elapsed_time(ev[w + 1]) * 1e-3 for w in range(windows))
+    secs = []
+    ms = ctypes.c_float()
+    for w in range(windows):
+        if hip.hipEventElapsedTime(ctypes.byref(ms), raw[w], raw[w + 1]) != 0:
+            raise RuntimeError("hipEventElapsedTime failed")
+        secs.append(ms.value * 1e-3)
+    for e in raw:
+        hip.hipEventDestroy(e)
+    return sorted(secs)
 
 
 def _summary(secs, steps):
@@ -511,7 +569,8 @@ def main():
         "config": {"workload": "GPTQ 3-bit matvec K=4096 N=11008 batch 1, fp32 x, weights rotated over 34 "
                                "distinct 16.9 MB buffers (575 MB)", "algorithmic_bytes_per_call": ALGO_BYTES},
         "windows": windows, "ms_per_step_min": round(us_min * 1e-3, 6), "ms_per_step_max": round(us_max * 1e-3, 6),
-        "timing": f"median of {windows} windows of {args.steps} back-to-back calls, HIP events on the launch stream",
+        "timing": f"median of {windows} windows of {args.steps} back-to-back calls, HIP events on the launch stream "
+                  f"({'created with hipEventDisableSystemFence' if _hip_runtime() else 'torch events'})",
         "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2),
         "effective_fp16_weight_GBps": round(K * N * 2 / us / 1e3, 1),
         "hot_cache_us_per_call": None if hot_us is None else round(hot_us, 3),
