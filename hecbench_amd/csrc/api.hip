@@ -24,7 +24,7 @@ std::vector<std::pair<int, void*>> g_retired;  // outgrown buffers, freed by hq_
 // with one relaxed atomic load, never the environment.
 namespace {
 const char* const kTunableNames[HQ_TUNE_COUNT] = {
-    "HQ_Q3_WAVES", "HQ_Q3_STEPS", "HQ_Q3_KSPLIT", "HQ_Q3_SMALL_BATCH", "HQ_LUT_PATH", "HQ_LUT_KSPLIT", "HQ_NF4_PIPE",
+    "HQ_Q3_WAVES", "HQ_Q3_STEPS", "HQ_Q3_KSPLIT", "HQ_Q3_SMALL_BATCH", "HQ_Q3_ROW_BLOCKS", "HQ_LUT_PATH", "HQ_LUT_KSPLIT", "HQ_NF4_PIPE",
     "HQ_AQLM_ROWS", "HQ_Q8_WGS", "HQ_Q8_FAST", "HQ_GEMV_LDS", "HQ_SPLITK_FENCES"};
 constexpr int kUnset = INT_MIN;
 std::atomic<int> g_tunables[HQ_TUNE_COUNT];
@@ -132,18 +132,19 @@ extern "C" int hq_reserve_workspace(void* stream, int max_K, int max_N) {
   const size_t full_split = tiles * (rounds <= 8 ? rounds : 1);
   const size_t per_cu = tiles + 2 * (size_t)d->cus;
   size_t split_floats = (full_split > per_cu ? full_split : per_cu) * 64 * 2;
-  // batches 2 ... 12 on the matvec-like kernel: one partial row per tile, round of K and activation row, at most 8192
+  // batches 2 ... 32 on the matvec-like kernel: one partial row per tile, round of K and activation row, at most 8192
   size_t block_splits = rounds;
   if (rounds > 8) {  // longer K: two workgroups per compute unit
     block_splits = 2 * (size_t)d->cus / (tiles ? tiles : 1);
     if (block_splits < 1) block_splits = 1;
     if (block_splits > rounds) block_splits = rounds;
   }
-  const size_t block_rows = tiles * block_splits * 12 < 8192 ? tiles * block_splits * 12 : 8192;
+  // (up to 32 rows as row blocks of four: the same bound, and a counter per tile and row block)
+  const size_t block_rows = tiles * block_splits * 32 < 8192 ? tiles * block_splits * 32 : 8192;
   if (block_rows * 64 > split_floats) split_floats = block_rows * 64;
   HqWorkspace ws;
   return hq_get_workspace((hipStream_t)stream, gemm_floats > split_floats ? gemm_floats : split_floats,
-                          tiles > 1 ? tiles : 1, &ws);
+                          tiles > 1 ? tiles * 8 : 8, &ws);
 }
 
 extern "C" int hq_shutdown(void) {

@@ -465,8 +465,8 @@ int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales
                       float* y, int K, int N, int M, unsigned flags, hipStream_t stream, const HqQ3Scratch* fixed);
 
 int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                       int K, int N, int M, int nsplit, int rpw, float* partial, unsigned* counters, unsigned flags,
-                       hipStream_t stream);
+                       int K, int N, int M, int nsplit, int rpw, int mblocks, float* partial, unsigned* counters,
+                       unsigned flags, hipStream_t stream);
 int hq_q3_block_groups_per_round(void);
 
 namespace {
@@ -482,7 +482,6 @@ namespace {
 // Largest batch the matvec-like kernels take by default, and the most partial-sum rows (tiles x splits x batch)
 // the kernel for 2 ... 8 rows may need: what the fixed scratch of the entry point that allocates nothing holds,
 // applied to every caller so that both entry points run the same kernel on the same shape.
-constexpr int kDigitBatchDefault = 12;
 constexpr size_t kBlockPartialRows = 8192;
 
 // How the kernel for 2 ... 8 rows cuts K: up to eight rounds of 4096 elements, one workgroup per round (as the
@@ -504,23 +503,53 @@ void q3_block_split(const HqDevice* dev, int K, int N, int batch_M, int* nsplit,
   *nsplit = (rounds + *rpw - 1) / *rpw;
 }
 
+constexpr int kRowBlockBatchMax = 32;  // rows a batch may have as row blocks of four
+
+// Row blocks (workgroups per column tile, four rows each) of a batch of more than four rows; 1: passes inside
+// one workgroup; 0: the four-rows-per-pass kernel does not take this batch at all.
+int q3_block_row_blocks(const HqDevice* dev, int K, int N, int batch_M, int nsplit, int rpw) {
+  (void)K;
+  // Measured (us per call, passes in one workgroup or the GEMM -> row blocks): with a CU for every workgroup,
+  // K=4096, N=4096: 5 rows 7.2 -> 5.2, 8 rows 8.4 -> 5.3, 12 rows 11.7 -> 5.3, 16 rows 12.7 -> 5.6; with up to
+  // four workgroups per CU, K=4096, N=4096, 32 rows 12.8 -> 8.4; K=4096, N=11008: 8 rows 9.0 -> 8.5, 12 rows
+  // 12.3 -> 11.0, 16 rows 14.3 -> 11.4; K=11008, N=4096: 12 rows 15.0 -> 12.8, 16 rows 17.6 -> 13.0; K=4096,
+  // N=22016: 7 rows 14.4 -> 11.9, 8 rows 15.2 -> 11.7; K=8192, N=8192: 16 rows 16.5 -> 16.2.  Five and six
+  // rows in more workgroups than CUs do not gain (K=4096, N=11008, 5 rows: 7.8 -> 8.4): the second block's one
+  // or two rows cost a whole workgroup where a second pass costs two rows of staging.
+  const int mode = hq_tune(HQ_TUNE_Q3_ROW_BLOCKS, -1);  // 0: never, 1: wherever possible (tests)
+  if (batch_M <= 4) return 1;
+  const int mb = (batch_M + 3) / 4;
+  const size_t groups = (size_t)((N + 63) / 64) * nsplit;
+  const bool possible = mode != 0 && rpw == 1 && nsplit <= 8 && batch_M <= kRowBlockBatchMax &&
+                        (nsplit == 1 || groups * mb * 4 <= kBlockPartialRows);
+  if (possible) {
+    const size_t wgs = groups * mb;
+    if (mode == 1 || wgs <= (size_t)dev->cus || (batch_M >= 7 && wgs <= 4 * (size_t)dev->cus)) return mb;
+  }
+  return batch_M <= 12 ? 1 : 0;
+}
+
 int q3_plan(const HqDevice* dev, int K, int N, int batch_M) {
   if (batch_M == 1) return HQ_Q3_PLAN_MATVEC;
-  const int limit = hq_tune(HQ_TUNE_Q3_SMALL_BATCH, kDigitBatchDefault);  // 0: every batch takes the GEMM
-  // 2 ... 8 rows.  Five to eight rows take
+  const int limit = hq_tune(HQ_TUNE_Q3_SMALL_BATCH, kRowBlockBatchMax);  // 0: every batch takes the GEMM
+  int nsplit, rpw;
+  q3_block_split(dev, K, N, batch_M, &nsplit, &rpw);
+  if (batch_M > limit) return HQ_Q3_PLAN_GEMM;
+  const int mb = q3_block_row_blocks(dev, K, N, batch_M, nsplit, rpw);
+  if (mb > 1) return HQ_Q3_PLAN_BLOCK;
+  if (mb == 0) return HQ_Q3_PLAN_GEMM;
+  // 2 ... 8 rows in one workgroup per tile and K range.  Five to eight rows take
   // two passes per workgroup, which beats the GEMM (7.8-12.4 us against 13-19 us at 4096 x 4096 ... 14336 x
   // 4096, 20.7-24.9 against 24.7 at K=8192, N=22016, 26.5-31.9 against 31.6 at K=28672, N=8192) except where
   // the GEMM's 128-column tiles fill the device without a K split (K=8192, N=28672: 27.8-31.1 against 25.3 us).
-  int nsplit, rpw;
-  q3_block_split(dev, K, N, batch_M, &nsplit, &rpw);
   const size_t groups = (size_t)((N + 63) / 64) * nsplit;
   const size_t tiles128 = (size_t)(N + 127) / 128;
-  if (batch_M <= limit && batch_M <= 8 && (nsplit == 1 || groups * batch_M <= kBlockPartialRows) &&
+  if (batch_M <= 8 && (nsplit == 1 || groups * batch_M <= kBlockPartialRows) &&
       (batch_M <= 4 || (rpw == 1 && 8 * tiles128 < 7 * (size_t)dev->cus)))
     return HQ_Q3_PLAN_BLOCK;
   // 9 ... 12 rows, three passes: where the launch has at most one workgroup per compute unit (it is a matter
   // of latency there, and the GEMM needs three launches)
-  if (batch_M <= limit && batch_M <= 12 && rpw == 1 && groups <= (size_t)dev->cus) return HQ_Q3_PLAN_BLOCK;
+  if (batch_M <= 12 && rpw == 1 && groups <= (size_t)dev->cus) return HQ_Q3_PLAN_BLOCK;
   return HQ_Q3_PLAN_GEMM;
 }
 
@@ -611,11 +640,16 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
       Q3Split sp;
       int nsplit, rpw;
       q3_block_split(dev, K, N, batch_M, &nsplit, &rpw);
-      rc = q3_split_k(dev, K / 32, rpw * hq_q3_block_groups_per_round(), (N + 63) / 64, batch_M, true, fixed, stream, &sp);
+      int mblocks = q3_block_row_blocks(dev, K, N, batch_M, nsplit, rpw);
+      if (mblocks < 1) mblocks = 1;
+      if (mblocks > 1)
+        rc = q3_split_k(dev, K / 32, hq_q3_block_groups_per_round(), (N + 63) / 64 * mblocks, 4, true, fixed, stream, &sp);
+      else
+        rc = q3_split_k(dev, K / 32, rpw * hq_q3_block_groups_per_round(), (N + 63) / 64, batch_M, true, fixed, stream, &sp);
       if (rc != HQ_OK) return rc;
       if (sp.nsplit != nsplit) return HQ_ERR_BAD_SHAPE;
-      return hq_q3_block_launch(x, qweight, scales, zeros, y, K, N, batch_M, nsplit, rpw, sp.partial, sp.counters, flags,
-                                stream);
+      return hq_q3_block_launch(x, qweight, scales, zeros, y, K, N, batch_M, nsplit, rpw, mblocks, sp.partial, sp.counters,
+                                flags, stream);
     }
     return hq_q3_gemm_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream, fixed);
   }

@@ -53,6 +53,7 @@ struct BlockArgs {
   int nsplit;         // workgroups per column tile
   int rpw;            // rounds of K per workgroup
   unsigned flags;
+  int prow;            // rows of partial sums a (virtual) column tile has per split
 };
 
 template <int CTRL>
@@ -98,7 +99,7 @@ __device__ __forceinline__ constexpr int step_off(int s) {
 // at most one workgroup per compute unit - changes nothing: a pass costs its ~450 VALU instructions per wave
 // wherever they stand.)
 template <int PASSES, bool MULTI>
-__device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
+__device__ __forceinline__ void q3_block_body(const BlockArgs& a, const int tile, const int vtile) {
   // LDS: dig[kWaves][kAreaBytes] | wsum[kWaves][kWsumStride]
   extern __shared__ uint4 smem[];
   constexpr int kAreaBytes = kWaveBytes;
@@ -109,7 +110,7 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 15, kb = lane >> 4;
-  const int tile = blockIdx.x, split = blockIdx.y;
+  const int split = blockIdx.y;
   const int g_begin = split * a.rpw * kGroupsPerRound;
   const int g_count = min(a.rpw * kGroupsPerRound, (a.K >> 5) - g_begin);  // k-groups of this workgroup
   const int M = a.M;
@@ -321,7 +322,7 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
         const float y_old = (a.flags & HQ_FLAG_ACCUMULATE) ? *yp : 0.f;
         __hip_atomic_store(yp, y_old + val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       } else {
-        __hip_atomic_store(&a.partial[(((size_t)tile * a.nsplit + split) * M + m) * 64 + col], val, __ATOMIC_RELAXED,
+        __hip_atomic_store(&a.partial[(((size_t)vtile * a.nsplit + split) * a.prow + m) * 64 + col], val, __ATOMIC_RELAXED,
                            __HIP_MEMORY_SCOPE_AGENT);
       }
     }
@@ -335,8 +336,8 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (tid == 0) {
-      const unsigned old = strict ? __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT)
-                                  : __hip_atomic_fetch_add(&a.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned old = strict ? __hip_atomic_fetch_add(&a.counters[vtile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT)
+                                  : __hip_atomic_fetch_add(&a.counters[vtile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       s_last = (old == (unsigned)(a.nsplit - 1));
     }
     __syncthreads();
@@ -346,14 +347,14 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a) {
         for (int m = tid >> 6; m < M; m += kWaves) {
           float sum = 0.f;
           for (int s = 0; s < a.nsplit; ++s)
-            sum += __hip_atomic_load(&a.partial[(((size_t)tile * a.nsplit + s) * M + m) * 64 + col], __ATOMIC_RELAXED,
+            sum += __hip_atomic_load(&a.partial[(((size_t)vtile * a.nsplit + s) * a.prow + m) * 64 + col], __ATOMIC_RELAXED,
                                      __HIP_MEMORY_SCOPE_AGENT);
           float* yp = &a.y[(size_t)m * a.N + ncol];
           *yp = (a.flags & HQ_FLAG_ACCUMULATE) ? *yp + sum : sum;
         }
       }
       if (tid == 0)  // ready for the next call
-        __hip_atomic_store(&a.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&a.counters[vtile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
 }
@@ -366,8 +367,26 @@ __global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 
   // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
   BlockArgs a;
   a.x = x_; a.w = w_; a.scales = scales_; a.zeros = zeros_; a.y = y_; a.partial = partial_; a.counters = counters_;
-  a.K = K_; a.N = N_; a.M = M_; a.nsplit = nsplit_; a.rpw = rpw_; a.flags = flags_;
-  q3_block_body<PASSES, MULTI>(a);
+  a.K = K_; a.N = N_; a.M = M_; a.nsplit = nsplit_; a.rpw = rpw_; a.flags = flags_; a.prow = M_;
+  q3_block_body<PASSES, MULTI>(a, blockIdx.x, blockIdx.x);
+}
+// More than four rows as several workgroups per column tile, each with up to four rows of its own (one pass):
+// the rows need no exchange, a launch that leaves compute units idle has room for the workgroups, and the
+// workgroups of a tile run on one XCD, close in time (workgroup b runs on XCD b mod 8: slot b / 8 of an XCD
+// is row block slot % mblocks of tile (slot / mblocks) * 8 + b mod 8), so the tile's weights come out of
+// that XCD's L2 for all but the first of them.
+__global__ __launch_bounds__(kWaves * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void q3_block_rows_kernel(
+                   const uint32_t* w_, const _Float16* x_, int K_, int N_, int M_, int nsplit_, int mblocks_, unsigned flags_,
+                   const float* scales_, const float* zeros_, float* y_, float* partial_, unsigned* counters_) {
+  const int slot = blockIdx.x >> 3;
+  const int tile = (slot / mblocks_) * 8 + (blockIdx.x & 7), mb = slot % mblocks_;
+  if (tile * 64 >= N_) return;  // the last group of eight tiles may be short
+  BlockArgs a;
+  a.x = x_ + (size_t)mb * kPassRows * K_;
+  a.y = y_ + (size_t)mb * kPassRows * N_;
+  a.w = w_; a.scales = scales_; a.zeros = zeros_; a.partial = partial_; a.counters = counters_;
+  a.K = K_; a.N = N_; a.M = min(kPassRows, M_ - mb * kPassRows); a.nsplit = nsplit_; a.rpw = 1; a.flags = flags_; a.prow = kPassRows;
+  q3_block_body<1, false>(a, tile, tile * mblocks_ + mb);
 }
 // Three passes (9 ... 12 rows) take 127 registers and more time than two workgroups per compute unit leave
 // room for; they run where the launch has at most one workgroup per compute unit and is a matter of latency
@@ -379,8 +398,8 @@ __global__ __launch_bounds__(kWaves * 64) void q3_block_kernel_many(
   // leading scalars, not the struct: the first 14 dwords of the arguments arrive preloaded in scalar registers
   BlockArgs a;
   a.x = x_; a.w = w_; a.scales = scales_; a.zeros = zeros_; a.y = y_; a.partial = partial_; a.counters = counters_;
-  a.K = K_; a.N = N_; a.M = M_; a.nsplit = nsplit_; a.rpw = rpw_; a.flags = flags_;
-  q3_block_body<PASSES, false>(a);
+  a.K = K_; a.N = N_; a.M = M_; a.nsplit = nsplit_; a.rpw = rpw_; a.flags = flags_; a.prow = M_;
+  q3_block_body<PASSES, false>(a, blockIdx.x, blockIdx.x);
 }
 
 template <auto KERNEL>
@@ -403,15 +422,26 @@ int hq_q3_block_groups_per_round(void) { return kGroupsPerRound; }
 // of 4096 elements and, for nsplit > 1, provided nsplit * M * 64 floats of partial sums per column tile and
 // one zeroed counter per column tile.
 int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
-                       int K, int N, int M, int nsplit, int rpw, float* partial, unsigned* counters, unsigned flags,
-                       hipStream_t stream) {
+                       int K, int N, int M, int nsplit, int rpw, int mblocks, float* partial, unsigned* counters,
+                       unsigned flags, hipStream_t stream) {
   const int rounds = (K / 32 + kGroupsPerRound - 1) / kGroupsPerRound;
-  if (M < 1 || M > kMaxRows || rpw < 1 || nsplit != (rounds + rpw - 1) / rpw) return HQ_ERR_BAD_SHAPE;
+  if (M < 1 || (M > kMaxRows && mblocks <= 1) || rpw < 1 || nsplit != (rounds + rpw - 1) / rpw) return HQ_ERR_BAD_SHAPE;
   BlockArgs a;
   a.x = reinterpret_cast<const _Float16*>(x);
   a.w = reinterpret_cast<const uint32_t*>(qweight);
   a.scales = scales; a.zeros = zeros; a.y = y; a.partial = partial; a.counters = counters; a.K = K; a.N = N; a.M = M;
-  a.nsplit = nsplit; a.rpw = rpw; a.flags = flags & (HQ_FLAG_ACCUMULATE | HQ_FLAG_STRICT_FENCES);
+  a.nsplit = nsplit; a.rpw = rpw; a.flags = flags & (HQ_FLAG_ACCUMULATE | HQ_FLAG_STRICT_FENCES); a.prow = M;
+  if (mblocks > 1) {
+    if (rpw != 1 || mblocks != (M + kPassRows - 1) / kPassRows) return HQ_ERR_BAD_SHAPE;
+    const size_t smem = (size_t)kWaves * kWaveBytes + (size_t)kWaves * kWsumStride * 4 + 16;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_block_rows_kernel),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (attr != hipSuccess) return (int)attr;
+    const int groups8 = ((N + 63) / 64 + 7) / 8;
+    hipLaunchKernelGGL(q3_block_rows_kernel, dim3(groups8 * mblocks * 8, nsplit), dim3(kWaves * 64), smem, stream, a.w, a.x,
+                       a.K, a.N, a.M, a.nsplit, mblocks, a.flags, a.scales, a.zeros, a.y, a.partial, a.counters);
+    return hq_launch_status();
+  }
   if (rpw > 1) return M <= kPassRows ? launch_block<&q3_block_kernel<1, true>>(a, stream) : HQ_ERR_BAD_SHAPE;
   if (M <= kPassRows) return launch_block<&q3_block_kernel<1, false>>(a, stream);
   if (M <= 2 * kPassRows) return launch_block<&q3_block_kernel<2, false>>(a, stream);

@@ -81,7 +81,7 @@ int hq_reserve_workspace(void* stream, int max_K, int max_N);
 int hq_shutdown(void);
 
 /* Launch-shape override for tests and sweeps, not part of the stable interface: name is one of
- * HQ_Q3_WAVES, HQ_Q3_STEPS, HQ_Q3_KSPLIT, HQ_Q3_SMALL_BATCH, HQ_LUT_PATH, HQ_LUT_KSPLIT, HQ_NF4_PIPE,
+ * HQ_Q3_WAVES, HQ_Q3_STEPS, HQ_Q3_KSPLIT, HQ_Q3_SMALL_BATCH, HQ_Q3_ROW_BLOCKS, HQ_LUT_PATH, HQ_LUT_KSPLIT, HQ_NF4_PIPE,
  * HQ_AQLM_ROWS, HQ_Q8_WGS, HQ_Q8_FAST, HQ_GEMV_LDS, HQ_SPLITK_FENCES (an environment variable of the same name seeds
  * the knob once per process); clear != 0 returns the knob to the library's own choice.  Results
  * never depend on a knob beyond the documented tolerances. */
@@ -129,10 +129,11 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  * (src/quant3MatMul-hip/kernels.h:171-217) — pass HQ_FLAG_ACCUMULATE for their
  * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 and has no counterpart in
  * the reference; which kernel serves it (hq_q3_matvec_plan tells):
- *   - batches 2 ... 4 (at 0.1 ... 0.6 us more than batch 1), 9 ... 12 where the launch has at
- *     most one workgroup per compute unit (N / 64 times K / 4096), and 5 ... 8 unless N / 128 is at least 7/8 of the compute units or
- *     K is so long that a workgroup takes several rounds of 4096: the matvec's kernel,
- *     four rows side by side;
+ *   - the matvec's kernel, four rows side by side: batches 2 ... 4 (at 0.1 ... 0.6 us more than
+ *     batch 1); batches up to 32 as row blocks of four, one workgroup per column tile, 4096
+ *     elements of K and row block, where that makes at most four workgroups per compute unit
+ *     (5 and 6 rows: at most one) and K <= 32768; otherwise 5 ... 8 rows as two passes of one
+ *     workgroup unless N / 128 is at least 7/8 of the compute units or K is longer than that;
  *     every activation enters with an error of at most 2^-19 of the largest magnitude
  *     among its 32 neighbours (exactly, if within 2^8 of it);
  *   - everything else: the MFMA GEMM path, which pre-scales every activation row by a
@@ -150,7 +151,7 @@ int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float
  */
 #define HQ_Q3_PLAN_MATVEC 0 /* batch_M == 1 */
 #define HQ_Q3_PLAN_GEMM 2   /* batched MFMA GEMM */
-#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 2 ... 12: the matvec's kernel, four rows per pass */
+#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 2 ... 32: the matvec's kernel, four rows per pass or workgroup */
 int hq_q3_matvec_plan(int K, int N, int batch_M);
 
 /*

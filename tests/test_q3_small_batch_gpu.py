@@ -41,16 +41,17 @@ def _check(y, exact):
 # wide (N = 257 tiles, the last one 4 columns wide) and narrow (3 tiles, the last one 4 columns wide);
 # K = 4128 is not a multiple of a workgroup's round, so the kernel splits it in two;
 # the long-K shape is there for the smallest batches only
-_EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)] for M in range(2, 16)
-                if K != 4128 or M <= 4]
+_EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)] for M in range(2, 35)
+                if (K == 512 and M <= 15) or (K == 4128 and M <= 4) or K == 1024]
 
 
 @pytest.mark.parametrize("M,K,N", _EVERY_BATCH)
 def test_every_batch_vs_oracle(hq, oracle, M, K, N):
     codes, scales, zeros, A = oa.make_q3_problem(1000 + 16 * M + (K % 7), K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
-    # 9 ... 12 rows: three passes, where the launch has at most one workgroup per compute unit
-    want_plan = PLAN_BLOCK if (M <= 8 or (M <= 12 and N < 1000)) else PLAN_GEMM
+    # more than four rows: row blocks of four where that makes at most four workgroups per compute unit (the
+    # wide shape: up to three blocks of its 257 tiles), up to 32 rows
+    want_plan = PLAN_BLOCK if M <= (12 if N > 1000 else 32) else PLAN_GEMM
     assert _plan(K, N, M) == want_plan
     y = _run(hq, A, mat, scales, zeros)
     _check(y, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
@@ -251,28 +252,64 @@ def test_block_kernel_vs_oracle(hq, oracle, M, K, N):
         assert rel_err(y[m], yv) <= 1e-3
 
 
+@pytest.mark.parametrize("M,K,N", [(5, 4128, 1028), (8, 512, 4100), (11, 4128, 1028), (12, 160, 16388), (13, 1024, 132),
+                                   (16, 8192, 260), (23, 4096, 516), (32, 32768, 68), (32, 160, 4100)])
+def test_row_blocks_and_passes_agree(hq, oracle, tunable, M, K, N):
+    """More than four rows as row blocks of four (one workgroup each; forced here whatever the launch size, with
+    and without a K split, with a last block of one to four rows) against the oracle, against the same batch
+    as passes of one workgroup (up to twelve rows) and, row by row, against the batch-1 matvec."""
+    codes, scales, zeros, A = oa.make_q3_problem(1700 + 16 * M + K % 13, K, N, x_dtype=np.float16, batch=M)
+    mat = oracle.q3_pack(codes)
+    exact = oracle.q3_gemm(A, mat, scales, zeros, mode=0)
+    tunable("HQ_Q3_ROW_BLOCKS", 1)
+    assert _plan(K, N, M) == PLAN_BLOCK
+    y = _run(hq, A, mat, scales, zeros)
+    for m in range(M):
+        assert rel_err(y[m], exact[m]) <= 1e-3, m
+    assert np.array_equal(_run(hq, A, mat, scales, zeros), y)  # partial sums and counters are left ready
+    dm, ds, dz = _t(mat), _t(scales), _t(zeros)
+    for m in (0, 3, 4, M - 1):
+        assert rel_err(y[m], hq.q3_matvec(_t(A[m]), dm, ds, dz).cpu().numpy()) <= 1e-3
+    if M <= 12:
+        tunable("HQ_Q3_ROW_BLOCKS", 0)
+        if _plan(K, N, M) == PLAN_BLOCK:
+            # the same digits and the same order of sums within a row: the same bits
+            assert np.array_equal(_run(hq, A, mat, scales, zeros), y)
+
+
 def test_block_kernel_plan_limits(hq, tunable):
-    """Beyond 8 rows, for 5 ... 8 rows beyond eight rounds of K or where the GEMM's 128-column tiles fill the device,
-    or with more partial sums than the fixed scratch of the entry point that allocates nothing holds, the batch
-    takes the GEMM; HQ_Q3_SMALL_BATCH lowers the limit.  (The counts below are for 256 compute units.)"""
+    """Beyond 32 rows, beyond four workgroups per compute unit as row blocks (5 and 6 rows: one), for 5 ... 8 rows
+    as passes beyond eight rounds of K or where the GEMM's 128-column tiles fill the device, or with more partial
+    sums than the fixed scratch of the entry point that allocates nothing holds, the batch takes the GEMM;
+    HQ_Q3_SMALL_BATCH lowers the limit.  (The counts below are for 256 compute units.)"""
     assert _plan(32768, 256, 8) == PLAN_BLOCK
-    assert _plan(32800, 256, 8) == PLAN_BLOCK         # nine rounds, four tiles: still one workgroup per round
+    assert _plan(32800, 256, 8) == PLAN_BLOCK         # nine rounds, four tiles: still one workgroup per round, two passes
     assert _plan(49152, 12288, 8) == PLAN_GEMM        # twelve rounds, 192 tiles: six rounds per workgroup, one pass only
     assert _plan(49152, 12288, 4) == PLAN_BLOCK
     assert _plan(4096, 4096, 8) == PLAN_BLOCK
-    assert _plan(4096, 4096, 12) == PLAN_BLOCK        # three passes: 64 workgroups
-    assert _plan(4096, 4096, 13) == PLAN_GEMM
-    assert _plan(4096, 16448, 12) == PLAN_GEMM        # 257 workgroups
-    assert _plan(8192, 8192, 12) == PLAN_BLOCK        # 128 tiles x 2 rounds
-    assert _plan(8192, 8256, 12) == PLAN_GEMM
+    assert _plan(4096, 4096, 13) == PLAN_BLOCK        # four row blocks: 256 workgroups
+    assert _plan(4096, 4096, 32) == PLAN_BLOCK        # eight row blocks: two workgroups per compute unit
+    assert _plan(4096, 4096, 33) == PLAN_GEMM
+    assert _plan(4096, 16448, 12) == PLAN_BLOCK       # 257 tiles x 3 row blocks
+    assert _plan(4096, 16448, 16) == PLAN_GEMM        # x 4 row blocks: more than four per compute unit
+    assert _plan(4096, 16448, 6) == PLAN_BLOCK        # six rows there: two passes of one workgroup per tile
+    assert _plan(8192, 8192, 12) == PLAN_BLOCK        # 128 tiles x 2 rounds x 3 row blocks
+    assert _plan(8192, 22016, 12) == PLAN_GEMM        # 344 x 2 x 3
     assert _plan(8192, 28672, 4) == PLAN_BLOCK        # one pass per workgroup: always
     assert _plan(8192, 28672, 5) == PLAN_GEMM         # two passes: not where the GEMM's 224 tiles fill the device
-    assert _plan(8192, 22016, 8) == PLAN_BLOCK        # 172 tiles of 128 columns
+    assert _plan(8192, 22016, 8) == PLAN_BLOCK        # 172 tiles of 128 columns: two passes
     assert _plan(28672, 8192, 8) == PLAN_BLOCK
     assert _plan(12288, 65536, 3) == PLAN_BLOCK       # 1024 tiles x 3 rounds x 3 rows would be 9216 partial rows: two ranges of K
     assert _plan(12288, 65536, 8) == PLAN_GEMM        # two passes: one round per workgroup only
-    tunable("HQ_Q3_SMALL_BATCH", 16)
+    tunable("HQ_Q3_ROW_BLOCKS", 0)                    # passes only: the limits of the passes
+    assert _plan(4096, 4096, 12) == PLAN_BLOCK        # three passes: 64 workgroups
     assert _plan(4096, 4096, 13) == PLAN_GEMM
+    assert _plan(4096, 16448, 12) == PLAN_GEMM        # 257 workgroups
+    assert _plan(8192, 8256, 12) == PLAN_GEMM
+    tunable("HQ_Q3_ROW_BLOCKS", -1)
+    tunable("HQ_Q3_SMALL_BATCH", 16)
+    assert _plan(4096, 4096, 16) == PLAN_BLOCK
+    assert _plan(4096, 4096, 17) == PLAN_GEMM
     tunable("HQ_Q3_SMALL_BATCH", 4)
     assert _plan(4096, 4096, 4) == PLAN_BLOCK
     assert _plan(4096, 4096, 5) == PLAN_GEMM
