@@ -132,19 +132,19 @@ extern "C" int hq_reserve_workspace(void* stream, int max_K, int max_N) {
   const size_t full_split = tiles * (rounds <= 8 ? rounds : 1);
   const size_t per_cu = tiles + 2 * (size_t)d->cus;
   size_t split_floats = (full_split > per_cu ? full_split : per_cu) * 64 * 2;
-  // batches 2 ... 32 on the matvec-like kernel: one partial row per tile, round of K and activation row, at most 8192
+  // batches 2 ... 64 on the matvec-like kernel: one partial row per tile, round of K and activation row, at most 8192
   size_t block_splits = rounds;
   if (rounds > 8) {  // longer K: two workgroups per compute unit
     block_splits = 2 * (size_t)d->cus / (tiles ? tiles : 1);
     if (block_splits < 1) block_splits = 1;
     if (block_splits > rounds) block_splits = rounds;
   }
-  // (up to 32 rows as row blocks of four: the same bound, and a counter per tile and row block)
-  const size_t block_rows = tiles * block_splits * 32 < 8192 ? tiles * block_splits * 32 : 8192;
+  // (up to 64 rows as row blocks of four: the same bound, and a counter per tile and row block)
+  const size_t block_rows = tiles * block_splits * 64 < 8192 ? tiles * block_splits * 64 : 8192;
   if (block_rows * 64 > split_floats) split_floats = block_rows * 64;
   HqWorkspace ws;
   return hq_get_workspace((hipStream_t)stream, gemm_floats > split_floats ? gemm_floats : split_floats,
-                          tiles > 1 ? tiles * 8 : 8, &ws);
+                          tiles > 1 ? tiles * 16 : 16, &ws);
 }
 
 extern "C" int hq_shutdown(void) {

@@ -503,7 +503,7 @@ void q3_block_split(const HqDevice* dev, int K, int N, int batch_M, int* nsplit,
   *nsplit = (rounds + *rpw - 1) / *rpw;
 }
 
-constexpr int kRowBlockBatchMax = 32;  // rows a batch may have as row blocks of four
+constexpr int kRowBlockBatchMax = 64;  // rows a batch may have as row blocks of four
 
 // Row blocks (workgroups per column tile, four rows each) of a batch of more than four rows; 1: passes inside
 // one workgroup; 0: the four-rows-per-pass kernel does not take this batch at all.

@@ -130,7 +130,7 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  * "mul +=" behaviour.  batch_M > 1 requires HQ_DTYPE_F16 and has no counterpart in
  * the reference; which kernel serves it (hq_q3_matvec_plan tells):
  *   - the matvec's kernel, four rows side by side: batches 2 ... 4 (at 0.1 ... 0.6 us more than
- *     batch 1); batches up to 32 as row blocks of four, one workgroup per column tile, 4096
+ *     batch 1); batches up to 64 as row blocks of four, one workgroup per column tile, 4096
  *     elements of K and row block, where that makes at most four workgroups per compute unit
  *     (5 and 6 rows: at most one) and K <= 32768; otherwise 5 ... 8 rows as two passes of one
  *     workgroup unless N / 128 is at least 7/8 of the compute units or K is longer than that;
@@ -151,7 +151,7 @@ int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float
  */
 #define HQ_Q3_PLAN_MATVEC 0 /* batch_M == 1 */
 #define HQ_Q3_PLAN_GEMM 2   /* batched MFMA GEMM */
-#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 2 ... 32: the matvec's kernel, four rows per pass or workgroup */
+#define HQ_Q3_PLAN_BLOCK 3  /* batch_M 2 ... 64: the matvec's kernel, four rows per pass or workgroup */
 int hq_q3_matvec_plan(int K, int N, int batch_M);
 
 /*
@@ -160,8 +160,8 @@ int hq_q3_matvec_plan(int K, int N, int batch_M);
  * scratch the kernels need (split-K partial sums and arrival counters of batches 1 and 2, the batched
  * path's re-ordered activations, row sums, row scales and K-split sums) is a fixed 10 MiB + 64 KiB array in device
  * memory that each GPU holds from library load to process end, instead of the stream's workspace.
- * The call runs no hipMalloc, hipFree or allocating library routine.  Limits: batch_M > 2 needs
- * K <= 16384; a split-K matvec needs tiles * splits * batch_M <= 8192 (the one-per-round split falls
+ * The call runs no hipMalloc, hipFree or allocating library routine.  Limits: a batch that the MFMA
+ * GEMM serves (hq_q3_matvec_plan) needs K <= 16384; a split-K matvec needs tiles * splits * batch_M <= 8192 (the one-per-round split falls
  * back to one workgroup per compute unit where it would not fit) and N <= 1032192; beyond them
  * HQ_ERR_TOO_LARGE.  All calls on one GPU
  * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race;

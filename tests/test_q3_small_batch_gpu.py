@@ -41,7 +41,7 @@ def _check(y, exact):
 # wide (N = 257 tiles, the last one 4 columns wide) and narrow (3 tiles, the last one 4 columns wide);
 # K = 4128 is not a multiple of a workgroup's round, so the kernel splits it in two;
 # the long-K shape is there for the smallest batches only
-_EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)] for M in range(2, 35)
+_EVERY_BATCH = [(M, K, N) for (K, N) in [(512, 16388), (4128, 8192), (1024, 132)] for M in list(range(2, 35)) + [47, 48, 61, 64, 65, 66]
                 if (K == 512 and M <= 15) or (K == 4128 and M <= 4) or K == 1024]
 
 
@@ -50,8 +50,8 @@ def test_every_batch_vs_oracle(hq, oracle, M, K, N):
     codes, scales, zeros, A = oa.make_q3_problem(1000 + 16 * M + (K % 7), K, N, x_dtype=np.float16, batch=M)
     mat = oracle.q3_pack(codes)
     # more than four rows: row blocks of four where that makes at most four workgroups per compute unit (the
-    # wide shape: up to three blocks of its 257 tiles), up to 32 rows
-    want_plan = PLAN_BLOCK if M <= (12 if N > 1000 else 32) else PLAN_GEMM
+    # wide shape: up to three blocks of its 257 tiles), up to 64 rows
+    want_plan = PLAN_BLOCK if M <= (12 if N > 1000 else 64) else PLAN_GEMM
     assert _plan(K, N, M) == want_plan
     y = _run(hq, A, mat, scales, zeros)
     _check(y, oracle.q3_gemm(A, mat, scales, zeros, mode=0))
@@ -253,7 +253,7 @@ def test_block_kernel_vs_oracle(hq, oracle, M, K, N):
 
 
 @pytest.mark.parametrize("M,K,N", [(5, 4128, 1028), (8, 512, 4100), (11, 4128, 1028), (12, 160, 16388), (13, 1024, 132),
-                                   (16, 8192, 260), (23, 4096, 516), (32, 32768, 68), (32, 160, 4100)])
+                                   (16, 8192, 260), (23, 4096, 516), (32, 32768, 68), (32, 160, 4100), (61, 4128, 260), (64, 512, 132)])
 def test_row_blocks_and_passes_agree(hq, oracle, tunable, M, K, N):
     """More than four rows as row blocks of four (one workgroup each; forced here whatever the launch size, with
     and without a K split, with a last block of one to four rows) against the oracle, against the same batch
@@ -278,7 +278,7 @@ def test_row_blocks_and_passes_agree(hq, oracle, tunable, M, K, N):
 
 
 def test_block_kernel_plan_limits(hq, tunable):
-    """Beyond 32 rows, beyond four workgroups per compute unit as row blocks (5 and 6 rows: one), for 5 ... 8 rows
+    """Beyond 64 rows, beyond four workgroups per compute unit as row blocks (5 and 6 rows: one), for 5 ... 8 rows
     as passes beyond eight rounds of K or where the GEMM's 128-column tiles fill the device, or with more partial
     sums than the fixed scratch of the entry point that allocates nothing holds, the batch takes the GEMM;
     HQ_Q3_SMALL_BATCH lowers the limit.  (The counts below are for 256 compute units.)"""
@@ -289,7 +289,9 @@ def test_block_kernel_plan_limits(hq, tunable):
     assert _plan(4096, 4096, 8) == PLAN_BLOCK
     assert _plan(4096, 4096, 13) == PLAN_BLOCK        # four row blocks: 256 workgroups
     assert _plan(4096, 4096, 32) == PLAN_BLOCK        # eight row blocks: two workgroups per compute unit
-    assert _plan(4096, 4096, 33) == PLAN_GEMM
+    assert _plan(4096, 4096, 64) == PLAN_BLOCK        # sixteen row blocks: four workgroups per compute unit
+    assert _plan(4096, 4096, 65) == PLAN_GEMM
+    assert _plan(4096, 8192, 64) == PLAN_GEMM         # 128 tiles x 16 row blocks
     assert _plan(4096, 16448, 12) == PLAN_BLOCK       # 257 tiles x 3 row blocks
     assert _plan(4096, 16448, 16) == PLAN_GEMM        # x 4 row blocks: more than four per compute unit
     assert _plan(4096, 16448, 6) == PLAN_BLOCK        # six rows there: two passes of one workgroup per tile

@@ -62,7 +62,7 @@ def test_noalloc_rejects_beyond_its_limits(hq):
     from hecbench_amd import _lib
     lib = _lib.load()
     dev = torch.device("cuda:0")
-    K, N, M = 32768, 64, 33                     # the batched GEMM's activations would need 4 MiB
+    K, N, M = 32768, 64, 65                     # the batched GEMM's activations would need 4 MiB
     A = torch.zeros((M, K), dtype=torch.float16, device=dev)
     w = torch.zeros((3 * K // 32, N), dtype=torch.int32, device=dev)
     s = torch.zeros(N, device=dev)
