@@ -239,7 +239,7 @@ def load_ref_hip():
 # ------------------------------------------------------------------ inputs
 
 def make_q3_problem(seed, K, N, x_dtype=np.float32, batch=None):
-    """BASELINE-style seeded GPTQ 3-bit problem."""
+    """Seeded GPTQ 3-bit problem in the shape of the benchmark's fixture: codes, scales, pre-multiplied zeros, activations."""
     rng = np.random.default_rng(seed)
     codes = rng.integers(0, 8, size=(K, N), dtype=np.uint8)
     scales = rng.uniform(0.005, 0.02, size=N).astype(np.float32)
