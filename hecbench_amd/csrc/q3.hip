@@ -38,6 +38,7 @@ namespace {
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u2v __attribute__((ext_vector_type(2)));
 typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 
 struct Q3Args {
@@ -118,7 +119,7 @@ __device__ __forceinline__ constexpr int step_off(int s) {
 // ROUNDS: 0 one round per workgroup, 1 several with a round's loads issued at once one round ahead, 2 several
 // with only the first step's loads at the top of a round and step s + 1 of the next round before the
 // arithmetic of step s.
-template <int WAVES, int STEPS, bool XF16, int ROUNDS>
+template <int WAVES, int STEPS, bool XF16, int ROUNDS, int CPL = 4>
 __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w_, const void* x_, int K_, int N_, int gpw_,
                                                               int nsplit_, int x_f16_, unsigned flags_,
                                                               const float* scales_, const float* zeros_, float* y_,
@@ -137,16 +138,23 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int c = lane & 15, kb = lane >> 4;
-  const int tile = blockIdx.x, split = blockIdx.y;
+  // A lane owns CPL adjacent columns, a workgroup TW = 16 * CPL.  Narrow tiles (CPL < 4) are dealt out so that
+  // the 4 / CPL tiles of a 64-column group (whose packed rows share 128-byte lines) run on one XCD, in
+  // neighbouring slots: workgroup b runs on XCD b mod 8.
+  constexpr int TW = 16 * CPL, SUB = 4 / CPL;
+  const int slot = blockIdx.x >> 3;
+  const int tile = CPL == 4 ? (int)blockIdx.x : ((slot / SUB) * 8 + (int)(blockIdx.x & 7)) * SUB + slot % SUB;
+  const int split = blockIdx.y;
+  if (CPL < 4 && tile * TW >= a.N) return;  // the last group of eight may be short
   const int G = a.K >> 5;
   const int g_begin = split * a.gpw;
   const int g_count = min(a.gpw, G - g_begin);
   const size_t row_stride = (size_t)a.N;
-  const int n = tile * 64 + tid;
+  const int n = tile * TW + tid;
 
   // ---- loads that do not depend on the round ------------------------------------------------
   float sc_n = 0.f, zr_n = 0.f, y_old = 0.f;
-  if (tid < 64) {
+  if (tid < TW) {
     const int nc = min(n, a.N - 1);
     sc_n = a.scales[nc];
     zr_n = a.zeros[nc];
@@ -160,10 +168,10 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
   const char* xbase = reinterpret_cast<const char*>(a.x) + (size_t)g_begin * 32 * (XF16 ? 2 : 4);
   // weights: out-of-range columns read the last valid quad (their results are never
   // stored), out-of-range k-groups read a valid group and get zero activations
-  const int tile_cols = min(64, a.N - tile * 64);           // multiple of 4
-  const uint32_t col_off = (uint32_t)min(4 * c, tile_cols - 4) * 4u;
+  const int tile_cols = min(TW, a.N - tile * TW);           // multiple of 4
+  const uint32_t col_off = (uint32_t)min(CPL * c, tile_cols - CPL) * 4u;
   const uint32_t row_bytes = (uint32_t)a.N * 4u;
-  const char* wbase = reinterpret_cast<const char*>(a.w) + ((size_t)(3 * g_begin) * row_stride + (size_t)tile * 64) * 4;
+  const char* wbase = reinterpret_cast<const char*>(a.w) + ((size_t)(3 * g_begin) * row_stride + (size_t)tile * TW) * 4;
   constexpr int GPR = WAVES * 4 * STEPS;  // k-groups per round
   constexpr bool MULTI = ROUNDS != 0;
   constexpr int kNextEarly = ROUNDS == 2 ? 1 : STEPS;  // steps of the next round loaded at the top of a round
@@ -177,7 +185,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
   // load while that queue is full, and a stalled wave stages nothing (K=4096, N=11008: 5.45 -> 5.38 us; one
   // step early 5.42, three 5.40).
   constexpr int kEarly = MULTI ? STEPS : (STEPS < 2 ? STEPS : 2);
-  auto load_steps = [&](int r, uint32_t (&wreg)[STEPS][3][4], int s0, int s1) {
+  auto load_steps = [&](int r, uint32_t (&wreg)[STEPS][3][CPL], int s0, int s1) {
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       if (s < s0 || s >= s1) continue;
@@ -185,12 +193,19 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
         const uint32_t off = (g * 3u + (uint32_t)j) * row_bytes + col_off;
-        u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wbase + off));
-        wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
+        if constexpr (CPL == 4) {
+          u4v v = __builtin_nontemporal_load(reinterpret_cast<const u4v*>(wbase + off));
+          wreg[s][j][0] = v.x; wreg[s][j][1] = v.y; wreg[s][j][2] = v.z; wreg[s][j][3] = v.w;
+        } else if constexpr (CPL == 2) {
+          u2v v = __builtin_nontemporal_load(reinterpret_cast<const u2v*>(wbase + off));
+          wreg[s][j][0] = v.x; wreg[s][j][1] = v.y;
+        } else {
+          wreg[s][j][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(wbase + off));
+        }
       }
     }
   };
-  auto load_round = [&](int r, float (&xr)[XP][8], uint32_t (&wreg)[STEPS][3][4]) {
+  auto load_round = [&](int r, float (&xr)[XP][8], uint32_t (&wreg)[STEPS][3][CPL]) {
 #pragma unroll
     for (int p = 0; p < XP; ++p) {
       const int s = min(4 * p + xs, STEPS - 1);
@@ -218,21 +233,21 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
     for (int s = 0; s < STEPS; ++s)
       *reinterpret_cast<uint32_t*>(dig_w + step_off(s) + 8 * kRowBytes + lane * 4) = 0x01010101u;
   }
-  float run[4][4];  // per-digit sums of all rounds (bias removed, divided by 2^E)
+  float run[CPL][4];  // per-digit sums of all rounds (bias removed, divided by 2^E)
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
+  for (int q = 0; q < CPL; ++q)
 #pragma unroll
     for (int i = 0; i < 4; ++i) run[q][i] = 0.f;
   float asum_total = 0.f;
   constexpr uint32_t M0 = low3_mask(0), M1 = low3_mask(1), M2 = low3_mask(2);
 
   float xr[XP][8];
-  uint32_t wreg[STEPS][3][4];
+  uint32_t wreg[STEPS][3][CPL];
   load_round(0, xr, wreg);
   if (!MULTI) __builtin_amdgcn_sched_barrier(0);
   for (int r = 0; r < rounds; ++r) {
     float xr_next[XP][8];
-    uint32_t wreg_next[STEPS][3][4];
+    uint32_t wreg_next[STEPS][3][CPL];
     if (MULTI && r + 1 < rounds) load_round(r + 1, xr_next, wreg_next);  // in flight during this round
 
     // ---- stage this wave's activation digits (wave-local) ---------------------------------
@@ -291,9 +306,9 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 
     // ---- mask + MFMA -----------------------------------------------------------------------
-    f4 acc[4];
+    f4 acc[CPL];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
+    for (int q = 0; q < CPL; ++q) acc[q] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
       if (!MULTI && s + kEarly < STEPS) {
@@ -310,7 +325,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
       const u4v b0 = bp[0], b1 = bp[1];
       const v8i B = {(int)b0.x, (int)b0.y, (int)b0.z, (int)b0.w, (int)b1.x, (int)b1.y, (int)b1.z, (int)b1.w};
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+      for (int q = 0; q < CPL; ++q) {
         const uint32_t w0 = wreg[s][0][q], w1 = wreg[s][1][q], w2 = wreg[s][2][q];
         const v8i A = {(int)(w0 & M0), (int)(w1 & M1), (int)(w2 & M2),
                        (int)(__builtin_amdgcn_alignbit(w1, w0, 3) & M0),
@@ -323,7 +338,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
     // while everything is still an exact integer, then leave the round's fixed-point scale.
     const float descale = pow2f(-E);
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
+    for (int q = 0; q < CPL; ++q)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float unbiased = fmaf(row_bcast8(acc[q][i]), -8.f, acc[q][i]);
@@ -342,17 +357,23 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
 #pragma unroll
         for (int j = 0; j < 3; ++j)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) wreg[s][j][q] = wreg_next[s][j][q];
+          for (int q = 0; q < CPL; ++q) wreg[s][j][q] = wreg_next[s][j][q];
     }
   }
 
   // ---- combine digits, waves, scale/zero --------------------------------------------------
-  // D[row = 4*kb + i][col = c]: row is the weight column 4*row + q of the tile, col the digit.
+  // D[row = 4*kb + i][col = c]: row is the weight column CPL*row + q of the tile, col the digit.
   if (c < 8) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const f4 v = {run[0][i], run[1][i], run[2][i], run[3][i]};
-      *reinterpret_cast<f4*>(red + (wv * 8 + c) * kRedStride + 4 * (4 * kb + i)) = v;
+      float* dst = red + (wv * 8 + c) * kRedStride + CPL * (4 * kb + i);
+      if constexpr (CPL == 4) {
+        const f4 v = {run[0][i], run[1][i], run[2][i], run[3][i]};
+        *reinterpret_cast<f4*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int q = 0; q < CPL; ++q) dst[q] = run[q][i];
+      }
     }
   }
   if (lane == 0) wsum[wv] = asum_total;
@@ -369,7 +390,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
   }
   __syncthreads();
   float val = 0.f;
-  if (tid < 64 && n < a.N) {
+  if (tid < TW && n < a.N) {
     float qx = 0.f, xsum = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
@@ -416,7 +437,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
     __syncthreads();
     if (s_last && strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     if (s_last) {
-      if (tid < 64 && n < a.N) {
+      if (tid < TW && n < a.N) {
         float sum = 0.f;
         for (int s = 0; s < a.nsplit; ++s)
           sum += __hip_atomic_load(&a.partial[((size_t)tile * a.nsplit + s) * 64 + tid],
@@ -429,21 +450,29 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
   }
 }
 
-template <int WAVES, int STEPS, bool XF16, int ROUNDS>
+template <int WAVES, int STEPS, bool XF16, int ROUNDS, int CPL = 4>
 int launch_matvec_t(const Q3Args& a, int ntiles, hipStream_t stream) {
   const size_t smem = (size_t)WAVES * STEPS * kStepBytes + (size_t)WAVES * 8 * kRedStride * 4 + (size_t)WAVES * 64 * 4 +
                       (size_t)WAVES * 4 + 16;
   static const hipError_t attr =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_matvec_kernel<WAVES, STEPS, XF16, ROUNDS>),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&q3_matvec_kernel<WAVES, STEPS, XF16, ROUNDS, CPL>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
   if (attr != hipSuccess) return (int)attr;
-  hipLaunchKernelGGL((q3_matvec_kernel<WAVES, STEPS, XF16, ROUNDS>), dim3(ntiles, a.nsplit), dim3(WAVES * 64), smem,
+  // narrow tiles: whole groups of eight 64-column tiles (the workgroups beyond N leave at once)
+  const int gx = CPL == 4 ? ntiles : ((a.N + 63) / 64 + 7) / 8 * 8 * (4 / CPL);
+  hipLaunchKernelGGL((q3_matvec_kernel<WAVES, STEPS, XF16, ROUNDS, CPL>), dim3(gx, a.nsplit), dim3(WAVES * 64), smem,
                      stream, a.w, a.x, a.K, a.N, a.gpw, a.nsplit, a.x_f16, a.flags, a.scales, a.zeros, a.y, a.partial,
                      a.counters);
   return hq_launch_status();
 }
 template <int WAVES, int STEPS>
-int launch_matvec(const Q3Args& a, int ntiles, int cus, hipStream_t stream) {
+int launch_matvec(const Q3Args& a, int ntiles, int cus, int cpl, hipStream_t stream) {
+  if constexpr (WAVES == 8 && STEPS == 4) {
+    if (cpl == 1)
+      return a.x_f16 ? launch_matvec_t<8, 4, true, 0, 1>(a, ntiles, stream) : launch_matvec_t<8, 4, false, 0, 1>(a, ntiles, stream);
+    if (cpl == 2)
+      return a.x_f16 ? launch_matvec_t<8, 4, true, 0, 2>(a, ntiles, stream) : launch_matvec_t<8, 4, false, 0, 2>(a, ntiles, stream);
+  }
   // Several rounds per workgroup: with a workgroup on every compute unit the next round's loads go out a
   // step at a time (K=36864, N=16384 41.0 -> 37.4 us, K=40960, N=8192 25.9 -> 23.6, K=65536, N=4096 22.6 -> 20.7);
   // with compute units to spare a whole round at once keeps more in flight (K=49152, N=12288, 192 tiles: 42.2
@@ -655,7 +684,7 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   }
 
   const int G = K / 32;
-  const int ntiles = (N + 63) / 64;
+  int ntiles = (N + 63) / 64;
   // Launch shape: a workgroup of WAVES waves covers WAVES*4*STEPS k-groups per round and
   // walks its K range in rounds (the next round's loads are in flight during the current
   // one), or K is split across workgroups whose partial sums the last one to arrive adds up.
@@ -668,8 +697,26 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
     while (steps > 1 && waves * 4 * (steps / 2) >= G) steps /= 2;  // short K: fewer steps
   }
   const int gpr = waves * 4 * steps;  // k-groups one workgroup covers per round
+  // Few column tiles (the default workgroup, one round of K per workgroup): narrower tiles, 32 or 16 columns,
+  // as long as every workgroup still has a CU of its own - the idle CUs' load queues join in.
+  // HQ_Q3_TILE: 4, 2 or 1 columns per lane, unset: by the launch size.
+  int cpl = 4;
+  {
+    const int rounds = (G + gpr - 1) / gpr;
+    const int want = hq_tune(HQ_TUNE_Q3_TILE, -1);
+    if (waves == 8 && steps == 4 && rounds <= 8 && hq_tune(HQ_TUNE_Q3_KSPLIT, -1) < 0) {
+      if (want == 1 || want == 2) cpl = want;
+      else if (want < 0) cpl = 4 * ntiles * rounds <= dev->cus ? 1 : (2 * ntiles * rounds <= dev->cus ? 2 : 4);
+    }
+    if (cpl < 4) ntiles = (N + 16 * cpl - 1) / (16 * cpl);
+  }
   Q3Split sp;
   rc = q3_split_k(dev, G, gpr, ntiles, 1, false, fixed, stream, &sp);
+  if (rc == HQ_OK && cpl < 4 && sp.gpw > gpr) {  // narrow tiles are for single-round workgroups only
+    cpl = 4;
+    ntiles = (N + 63) / 64;
+    rc = q3_split_k(dev, G, gpr, ntiles, 1, false, fixed, stream, &sp);
+  }
   if (rc != HQ_OK) return rc;
 
   Q3Args a;
@@ -677,7 +724,7 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   a.y = y; a.partial = sp.partial; a.counters = sp.counters; a.K = K; a.N = N; a.gpw = sp.gpw;
   a.nsplit = sp.nsplit; a.x_f16 = (x_dtype == HQ_DTYPE_F16); a.flags = flags;
 #define HQ_Q3_CASE(W, S) \
-  if (waves == W && steps == S) return launch_matvec<W, S>(a, ntiles, dev->cus, stream);
+  if (waves == W && steps == S) return launch_matvec<W, S>(a, ntiles, dev->cus, cpl, stream);
   HQ_Q3_CASE(16, 1)
   HQ_Q3_CASE(8, 1) HQ_Q3_CASE(8, 2) HQ_Q3_CASE(8, 4)
   HQ_Q3_CASE(4, 1) HQ_Q3_CASE(4, 2) HQ_Q3_CASE(4, 4) HQ_Q3_CASE(4, 8)

@@ -143,6 +143,29 @@ def test_launch_shapes_match(hq, oracle, tunable):
                 tunable("HQ_SPLITK_FENCES", 0)
 
 
+@pytest.mark.parametrize("x_dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 1028), (160, 132), (32, 4), (8192, 1024), (12320, 516), (4096, 11008),
+                                 (32768, 68)])
+def test_narrow_tiles_match(hq, oracle, tunable, K, N, x_dtype):
+    """Tiles of 32 and 16 columns (chosen by default where 64-column tiles would leave more than half of the
+    compute units without a workgroup) against the 64-column tiles, forced on shapes with ragged last tiles,
+    K splits and many tiles: the same bits (a column's arithmetic does not depend on its tile), accumulation
+    included, and the oracle's result."""
+    codes, scales, zeros, x = oa.make_q3_problem(K + N, K, N, x_dtype=x_dtype)
+    mat = oracle.q3_pack(codes)
+    exact = oracle.q3_matvec_f64(x, mat, scales, zeros)
+    y0 = np.linspace(-1.0, 1.0, N).astype(np.float32)
+    tunable("HQ_Q3_TILE", 4)
+    wide = _run(hq, x, mat, scales, zeros)
+    wide_acc = _run(hq, x, mat, scales, zeros, out=y0.copy(), accumulate=True)
+    assert rel_err(wide, exact, FLOOR_F16) <= 1e-3
+    for cpl in (2, 1):
+        tunable("HQ_Q3_TILE", cpl)
+        assert np.array_equal(_run(hq, x, mat, scales, zeros), wide), cpl
+        assert np.array_equal(_run(hq, x, mat, scales, zeros, out=y0.copy(), accumulate=True), wide_acc), cpl
+        assert np.array_equal(_run(hq, x, mat, scales, zeros), wide), cpl  # counters left ready
+
+
 @pytest.mark.parametrize("K,N", [(8192, 22016), (16384, 16644), (28672, 1028), (5120, 13824)])
 def test_default_k_split_on_long_k(hq, oracle, tunable, K, N):
     """Up to eight rounds of K run as one workgroup per round whatever the tile count (more column tiles than
