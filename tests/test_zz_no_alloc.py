@@ -40,10 +40,12 @@ def test_noalloc_matches_workspace_path(hq, oracle):
     lib = _lib.load()
     # 32 and 8 column tiles: far fewer than half the compute units, so both calls split K across
     # workgroups and use the partial sums and the arrival counters
-    big = _problem(oracle, 301, 8192, 2048, 40)
-    small = _problem(oracle, 302, 2048, 512, 20)
+    big = _problem(oracle, 301, 8192, 2048, 70)
+    small = _problem(oracle, 302, 2048, 512, 66)
     for p in (big, small):                      # two calls in a row, the second with a smaller input
-        for batch in (1, 2, 6, 11, p["M"]):     # the matvec, one, two and three passes of the small-batch kernel, the GEMM
+        # the matvec (narrow tiles), the small-batch kernel with one workgroup per tile and with two, three and
+        # ten row blocks, the GEMM (64 rows and the rest)
+        for batch in (1, 2, 6, 11, 40, p["M"]):
             want = _call(lib.hq_q3_matvec, p, batch)
             got = _call(lib.hq_q3_matvec_noalloc, p, batch)
             assert np.array_equal(got, want), (p["K"], p["N"], batch)
