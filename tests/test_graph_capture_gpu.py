@@ -23,7 +23,7 @@ def test_replays_match_eager(hq, oracle):
     K, N = 8192, 8256                       # two rounds of K: split over two workgroups per tile (workspace)
     codes, scales, zeros, x = oa.make_q3_problem(901, K, N)
     mat = oracle.q3_pack(codes)
-    Kg, Ng, M = 1024, 516, 24               # batched GEMM: pre-pass and main kernel meet in the workspace
+    Kg, Ng, M = 1024, 516, 72               # batched GEMM (more than 64 rows): pre-pass and main kernel meet in the workspace
     codes_g, scales_g, zeros_g, A = oa.make_q3_problem(902, Kg, Ng, x_dtype=np.float16, batch=M)
     mat_g = oracle.q3_pack(codes_g)
     dx, dm, ds, dz = _t(x), _t(mat), _t(scales), _t(zeros)
@@ -32,6 +32,8 @@ def test_replays_match_eager(hq, oracle):
     y_na = torch.zeros(N, device="cuda:0")
     yg = torch.zeros(M, Ng, device="cuda:0")
     A4 = torch.randn(4, K, device="cuda:0").half()          # batch 4 on the matvec's weights: partial sums of four rows
+    A24 = torch.randn(24, Kg, device="cuda:0").half()        # 24 rows on the small matrix: six row blocks per tile
+    y24 = torch.zeros(24, Ng, device="cuda:0")
     y4 = torch.zeros(4, N, device="cuda:0")
     stream = torch.cuda.Stream()
     vp = lambda t: ctypes.c_void_p(t.data_ptr())
@@ -46,9 +48,10 @@ def test_replays_match_eager(hq, oracle):
         hq.q3_matvec(dx, dm, ds, dz, out=y)
         hq.q3_gemm(dA, dmg, dsg, dzg, out=yg)
         hq.q3_gemm(A4, dm, ds, dz, out=y4)
+        hq.q3_gemm(A24, dmg, dsg, dzg, out=y24)
         noalloc(stream)
     stream.synchronize()
-    want, want_g, want_na, want_4 = y.clone(), yg.clone(), y_na.clone(), y4.clone()
+    want, want_g, want_na, want_4, want_24 = y.clone(), yg.clone(), y_na.clone(), y4.clone(), y24.clone()
     assert torch.equal(want, want_na)
 
     graph = torch.cuda.CUDAGraph()
@@ -56,9 +59,10 @@ def test_replays_match_eager(hq, oracle):
         hq.q3_matvec(dx, dm, ds, dz, out=y)
         hq.q3_gemm(dA, dmg, dsg, dzg, out=yg)
         hq.q3_gemm(A4, dm, ds, dz, out=y4)
+        hq.q3_gemm(A24, dmg, dsg, dzg, out=y24)
         noalloc(torch.cuda.current_stream())
     for rep in range(4):
-        y.fill_(float(rep)); yg.fill_(-1.0); y_na.fill_(7.0); y4.fill_(3.0)  # eager work between the replays
+        y.fill_(float(rep)); yg.fill_(-1.0); y_na.fill_(7.0); y4.fill_(3.0); y24.fill_(5.0)  # eager work between the replays
         other = hq.q3_matvec(dx, dm, ds, dz)                       # an eager call on another stream's workspace
         torch.cuda.synchronize()
         graph.replay()
@@ -66,5 +70,6 @@ def test_replays_match_eager(hq, oracle):
         assert torch.equal(y, want), rep
         assert torch.equal(yg, want_g), rep
         assert torch.equal(y4, want_4), rep
+        assert torch.equal(y24, want_24), rep
         assert torch.equal(y_na, want_na), rep
         assert torch.equal(other, want), rep
