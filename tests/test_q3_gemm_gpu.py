@@ -10,6 +10,13 @@ from tests.tol import FLOOR_F16, TOL_F16_ACC, rel_err
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _the_gemm_kernel_only(tunable):
+    """Small launches of up to 64 rows would take the matvec's four-rows-per-workgroup kernel by default
+    (tests/test_q3_small_batch_gpu.py covers that): this file is about the MFMA GEMM, so every batch takes it."""
+    tunable("HQ_Q3_SMALL_BATCH", 0)
+
+
 def _run(hq, A, mat, scales, zeros):
     import torch
     dev = torch.device("cuda:0")
