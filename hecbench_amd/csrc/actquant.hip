@@ -446,7 +446,10 @@ int launch_static(const T* in, int8_t* out, int64_t tokens, int hidden, float sc
   const int64_t total = tokens * hidden;
   const int64_t units = (total + kVec - 1) / kVec;
   int64_t blocks = (units + 256 * kStaticUnroll - 1) / (256 * kStaticUnroll);
-  const int64_t cap = (int64_t)dev->cus * 32;  // grid-stride beyond that
+  // six workgroups per CU, grid-stride beyond that (us per call at 32 / 6 per CU, fp16: 4096 x 5137 13.8 / 12.8,
+  // 4096 x 4096 11.3 / 10.7, 8192 x 5120 24.3 / 23.3, 16384 x 8192 72.4 / 71.6; four and eight per CU, and grids
+  // sized so that every workgroup makes the same number of trips, measured in between)
+  const int64_t cap = (int64_t)dev->cus * 6;
   if (blocks > cap) blocks = cap;
   if (has_azp)
     hipLaunchKernelGGL((static_quant_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, stream, in, out, scale, azp,
