@@ -137,6 +137,44 @@ def _summary(secs, steps):
     return med / steps * 1e6, secs[0] / steps * 1e6, secs[-1] / steps * 1e6
 
 
+def measure_device():
+    """What this box delivers to the simplest kernels (hq_probe_*): a pure read and a copy of 512 MiB (more
+    than the 256 MB Infinity Cache), and independent 16-byte reads at random entries of a 1 MB table (a
+    code-book lookup without the arithmetic: the rate of L2 requests)."""
+    import torch
+    from hecbench_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    n = 512 << 20
+    src = [torch.empty(n, dtype=torch.uint8, device=dev).random_() for _ in range(2)]
+    dst = torch.empty(n, dtype=torch.uint8, device=dev)
+    ps = [ctypes.c_void_p(t.data_ptr()) for t in src]
+    pd = ctypes.c_void_p(dst.data_ptr())
+
+    def check(rc):
+        if rc:
+            raise RuntimeError(lib.hq_strerror(rc).decode())
+
+    out = {}
+    secs = _time_windows(lambda i: check(lib.hq_probe_stream(0, ps[i], pd, n, stream)), 2, 10, 4, 11)
+    out["hbm_read_measured_GBps"] = round(n / (secs[len(secs) // 2] / 10) / 1e9, 1)
+    secs = _time_windows(lambda i: check(lib.hq_probe_stream(1, ps[i], pd, n, stream)), 2, 10, 4, 11)
+    out["hbm_copy_measured_GBps"] = round(2 * n / (secs[len(secs) // 2] / 10) / 1e9, 1)
+    out["hbm_probe"] = "hq_probe_stream over 512 MiB, two source buffers alternating; copy counts bytes read + written"
+    del src, dst
+    table = torch.empty(1 << 20, dtype=torch.uint8, device=dev).random_()
+    sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+    want = 1 << 24
+    cnt = lib.hq_probe_gather16_count(want)
+    pt, pk = ctypes.c_void_p(table.data_ptr()), ctypes.c_void_p(sink.data_ptr())
+    secs = _time_windows(lambda i: check(lib.hq_probe_gather16(pt, 1 << 20, want, pk, stream)), 1, 20, 5, 11)
+    out["l2_gather16_measured_Greq_s"] = round(cnt / (secs[len(secs) // 2] / 20) / 1e9, 1)
+    out["l2_gather_probe"] = ("hq_probe_gather16: %d independent 16-byte reads per launch at random entries of a "
+                              "1 MB table, eight in flight per lane" % cnt)
+    return out
+
+
 def bench_q3(steps, warmup, windows, hot=False):
     import torch
     from hecbench_amd import _lib
@@ -171,7 +209,7 @@ def _roofline_hbm(algo_bytes, us, profile):
             "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": profile_traffic(profile)}
 
 
-def bench_configs(steps, warmup, windows):
+def bench_configs(steps, warmup, windows, device=None):
     """Configurations 0, 2, 3 and 4 of the benchmark: microseconds per call (median window), algorithmic GB/s
     and the roofline object of each; inputs rotated over more than 512 MB so that every call reads HBM."""
     import torch
@@ -247,6 +285,13 @@ def bench_configs(steps, warmup, windows):
                Ma * Ka // 8 * 2 + 65536 * 16 + 3 * Ka * 2, secs, steps, "aqlm_matvec_4096x4096",
                dtype="f16 in, f32 sums, f16 out")
     out["3_aqlm_4096x4096"]["gather_GBps"] = round(Ma * Ka // 8 * 16 / us / 1e3, 1)   # 16-byte code-book gathers (L2)
+    # what bounds this kernel: one L2 request per 16-byte code-book entry; the peak is the rate the same box
+    # delivers to a kernel that does nothing but such reads from a table of the same size
+    peak = (device or {}).get("l2_gather16_measured_Greq_s")
+    greq = Ma * Ka // 8 / us / 1e3
+    out["3_aqlm_4096x4096"]["roofline_l2_requests"] = {
+        "bound": "l2_requests", "achieved": round(greq, 1), "peak": peak, "unit": "G 16-byte gathers/s",
+        "frac": None if not peak else round(greq / peak, 4), "traffic": None}
     del codes
     # config 4: batched GPTQ 3-bit GEMM M=64 K=8192 N=28672 (rotate 7 x 88 MB)
     Mg, Kg, Ng = 64, 8192, 28672
@@ -430,6 +475,47 @@ def bench_others(steps, warmup, windows):
     return out
 
 
+def cpu_configs():
+    """Serial and OpenMP times of the oracle's restatements for configurations 0, 2, 3 and 4 (bounded samples,
+    scaled to the full problem where a sample is used; about five seconds in all).  Reported next to the GPU
+    numbers, never a target."""
+    import numpy as np
+    from tests import oracle_api as oa
+    o = oa.load_oracle()
+    threads = max(1, min(o.max_threads(), os.cpu_count() or 1))
+
+    def timed(fn, reps):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return (time.perf_counter() - t0) / reps
+
+    jobs = {}
+    packed, absmax = oa.make_nf4_problem(0, 4096 * 4096, 64)
+    jobs["0_nf4_dequant_4096x4096"] = (lambda: o.dequant_4bit(packed, absmax, 4096 * 4096, 64), 2, 1, "2 full calls")
+    bW, alpha, qb, x = oa.make_lut_problem(0, 4096, 2048, 3, 128)
+    jobs["2_lut_gemv_4096x16384_q3"] = (lambda: o.lut_gemv_f64(bW, alpha, qb, x, 128), 2, 8,
+                                        "2048 of 16384 columns, scaled x8")
+    codes, cb, sc, xa = oa.make_aqlm_problem(0, 4096, 4096)
+    jobs["3_aqlm_4096x4096"] = (lambda: o.aqlm_matvec(codes, cb, sc, xa, (4096, 0, 0, 0), 65536), 2, 1, "2 full calls")
+    qc, scales, zeros, A = oa.make_q3_problem(0, 8192, 1024, np.float16, batch=4)
+    mat = o.q3_pack(qc)
+    jobs["4_q3_gemm_64x8192x28672"] = (lambda: o.q3_gemm(A, mat, scales, zeros), 2, 16 * 28,
+                                       "4 of 64 rows x 1024 of 28672 columns, scaled x448")
+    out = {}
+    for name, (fn, reps, scale, sample) in jobs.items():
+        o.set_threads(1)
+        serial = timed(fn, reps) * scale
+        o.set_threads(threads)
+        try:
+            par = timed(fn, reps) * scale
+        finally:
+            o.set_threads(1)
+        out[name] = {"cpu_serial": {"us": round(serial * 1e6, 1), "cores": 1, "kind": "port", "sample": sample},
+                     "cpu_openmp": {"us": round(par * 1e6, 1), "cores": threads, "kind": "port", "sample": sample}}
+    return out
+
+
 def cpu_others():
     """Serial CPU times of the oracle for the other configurations (one host core; bounded samples, scaled to
     the full problem where a sample is used).  Reported next to the GPU numbers, never a target."""
@@ -488,6 +574,28 @@ def cpu_others():
     if omp is not None:
         out["quantize_dynamic8_16777216"]["reference_omp"] = omp
     return out
+
+
+def quantbnb_host_only():
+    """The build's own quantBnB driver run host-only (its verification loops spread over the host cores with
+    OpenMP, no GPU call): what the benchmark's -omp variant measures with OMP_TARGET_OFFLOAD=DISABLED."""
+    import subprocess
+    exe = os.path.join(ROOT, "hecbench_amd", "bench", "quantBnB")
+    if not os.path.exists(exe):
+        return None
+    try:
+        r = subprocess.run([exe, "16777216", "3", "--host-only"], capture_output=True, text=True, timeout=120)
+    except (subprocess.TimeoutExpired, OSError):
+        return None
+    m = re.search(r"kQuantize kernel with block size \d+: ([0-9.]+) \(us\)\n(PASS|FAIL)\n\s+\(host only: OpenMP loop on "
+                  r"(\d+) threads; one thread: ([0-9.]+) us\)", r.stdout)
+    if not m:
+        return None
+    return {"cpu_openmp": {"us": round(float(m.group(1)), 1), "cores": int(m.group(3)), "kind": "port",
+                           "sample": "quantBnB 16777216 3 --host-only (the driver's own host loop)",
+                           "verdict": m.group(2)},
+            "cpu_serial": {"us": round(float(m.group(4)), 1), "cores": 1, "kind": "port",
+                           "sample": "the same loop on one thread, one pass"}}
 
 
 def reference_quantbnb_omp():
@@ -578,17 +686,26 @@ def main():
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": profile_traffic("q3_matvec_4096x11008")},
         "device": info,
     }
+    result["device"] = dict(info, **measure_device())
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_q3(state)
     del state
     if not args.no_configs:
         # the other four benchmark configurations: a few thousand calls each at most
         st = max(1, min(args.steps, 1000))
-        result["configs"] = bench_configs(st, min(args.warmup, 100), _windows_for(st, args.windows))
+        result["configs"] = bench_configs(st, min(args.warmup, 100), _windows_for(st, args.windows), result["device"])
+        if not args.no_cpu:
+            for name, legs in cpu_configs().items():
+                if name in result["configs"]:
+                    result["configs"][name].update(legs)
     if not args.no_others:
         # the kernels of the neighbouring benchmarks (gemv, mxfp4, quantVLLM, quantBnB), shorter loops
         st = max(20, min(args.steps // 4, 500))
         result["other_kernels"] = bench_others(st, 20, _windows_for(st, args.windows) if args.steps < 200 else 11)
+    if not args.no_others and not args.no_cpu:
+        legs = quantbnb_host_only()
+        if legs:
+            result["other_kernels"]["quantize_dynamic8_16777216"].update(legs)
     if args.all and not args.no_others:
         if not args.no_cpu:
             cpu = cpu_others()
@@ -598,8 +715,9 @@ def main():
                     tgt = next((v for k, v in result["configs"].items() if k[2:] == name), None)
                 if tgt is None:
                     continue
-                tgt["cpu_serial"] = {"us": round(c["cpu_us"], 1), "cores": 1, "kind": c.get("kind", "port"),
-                                     "sample": c["sample"]}
+                if "cpu_serial" not in tgt:
+                    tgt["cpu_serial"] = {"us": round(c["cpu_us"], 1), "cores": 1, "kind": c.get("kind", "port"),
+                                         "sample": c["sample"]}
                 if "reference_omp" in c:
                     tgt["cpu_reference_omp"] = c["reference_omp"]
     print(json.dumps(result))

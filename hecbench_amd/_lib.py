@@ -17,6 +17,9 @@ _SIGNATURES = {
     "hq_strerror": (_c.c_char_p, [_c.c_int]),
     "hq_init": (_c.c_int, []),
     "hq_reserve_workspace": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int]),
+    "hq_q3_workspace_need": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int, _c.c_int, _c.POINTER(_c.c_int64),
+                                        _c.POINTER(_c.c_int64)]),
+    "hq_reserve_need": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int, _c.POINTER(_c.c_int64), _c.POINTER(_c.c_int64)]),
     "hq_shutdown": (_c.c_int, []),
     "hq_set_tunable": (_c.c_int, [_c.c_char_p, _c.c_int, _c.c_int]),
     "hq_device_info": (_c.c_int, [_c.POINTER(_c.c_int)] * 5 + [_c.c_char_p, _c.c_int]),
@@ -48,6 +51,9 @@ _SIGNATURES = {
     "hq_gemv_int4": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int, _c.c_float,
                                 _c.c_float, _c.c_void_p]),
     "hq_mxfp4_qdq": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int, _c.c_void_p]),
+    "hq_probe_stream": (_c.c_int, [_c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p]),
+    "hq_probe_gather16": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_void_p]),
+    "hq_probe_gather16_count": (_c.c_int64, [_c.c_int64]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

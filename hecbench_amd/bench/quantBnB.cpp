@@ -1,12 +1,16 @@
 // quantBnB driver: same command line, inputs, verification and printed lines as the
 // HeCBench benchmark (src/quantBnB-hip/main.cu), on top of libhq.
 //
-//   quantBnB <number of elements> <repeat>
+//   quantBnB <number of elements> <repeat> [--host-only]
 //
 // Part 1 is the reference benchmark itself: bitsandbytes dynamic-map 8-bit
 // quantisation, device result compared bit for bit with the host function.
 // Part 2 runs the blockwise NF4 dequantisation of the same element count
 // (blocksize 64, fp16 output) against a host loop, also bit for bit.
+// Both host loops are timed as well, on one thread and spread over the host cores with OpenMP (what the
+// quantBnB-omp variant of the benchmark does when it runs without a device); --host-only runs nothing
+// else, needs no GPU and prints the OpenMP loop's time in the benchmark's own line.
+#include <omp.h>
 #include "bench_common.h"
 
 namespace {
@@ -56,14 +60,27 @@ const float kNf4[16] = {-1.0f, -0.6961928009986877f, -0.5250730514526367f, -0.39
 
 }  // namespace
 
+// Seconds per pass of a host loop over n elements on `threads` threads.
+template <class F>
+double time_host_loop(F&& body, size_t n, int threads, int passes) {
+  const auto t0 = std::chrono::steady_clock::now();
+  for (int p = 0; p < passes; ++p) {
+#pragma omp parallel for schedule(static) num_threads(threads)
+    for (long i = 0; i < (long)n; ++i) body((size_t)i);
+  }
+  return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / passes;
+}
+
 int main(int argc, char* argv[]) {
-  if (argc != 3) {
-    std::printf("Usage: %s <number of elements> <repeat>\n", argv[0]);
+  const bool host_only = argc == 4 && std::string(argv[3]) == "--host-only";
+  if (argc != 3 && !host_only) {
+    std::printf("Usage: %s <number of elements> <repeat> [--host-only]\n", argv[0]);
     return 1;
   }
   const size_t n = (size_t)std::atol(argv[1]);
   const int repeat = std::atoi(argv[2]);
-  HQ_OK_OR_DIE(hq_init());
+  const int block_size = 256;
+  const int cores = omp_get_max_threads();
 
   // ---- part 1: kQuantize contract --------------------------------------------------------
   const std::vector<float> code = dynamic_map();
@@ -71,15 +88,44 @@ int main(int argc, char* argv[]) {
   std::vector<uint8_t> out(n), ref(n);
   std::mt19937 gen{19937};
   std::normal_distribution<float> d{0.f, 1.f};
-  for (size_t i = 0; i < n; ++i) {
-    A[i] = d(gen);
-    ref[i] = dquantize_host(code.data(), A[i]);
+  for (size_t i = 0; i < n; ++i) A[i] = d(gen);
+  const double host1 = time_host_loop([&](size_t i) { ref[i] = dquantize_host(code.data(), A[i]); }, n, 1, 1);
+  const int host_passes = host_only ? (repeat > 0 ? repeat : 1) : 1;
+  const double hostN = time_host_loop([&](size_t i) { out[i] = dquantize_host(code.data(), A[i]); }, n, cores, host_passes);
+  if (host_only) {
+    std::printf("Average execution time of kQuantize kernel with block size %d: %f (us)\n", block_size, hostN * 1e6);
+    std::printf("%s\n", out == ref ? "PASS" : "FAIL");
+    std::printf("  (host only: OpenMP loop on %d threads; one thread: %f us)\n", cores, host1 * 1e6);
   }
+  // NF4 inputs and the host loop of part 2
+  const int blocksize = 64;
+  SeededRng rng(1234);
+  std::vector<uint8_t> packed((n + 1) / 2);
+  std::vector<float> absmax((n + blocksize - 1) / blocksize);
+  for (auto& b : packed) b = (uint8_t)(rng.u32() >> 24);
+  for (auto& a : absmax) a = (float)rng.uniform(0.5, 2.0);
+  std::vector<uint16_t> want(n), got(n);
+  auto nf4_host = [&](std::vector<uint16_t>& dst) {
+    return [&](size_t e) {
+      const uint8_t b = packed[e >> 1];
+      const unsigned c = (e & 1) ? (b & 15u) : (b >> 4);
+      volatile float prod = kNf4[c] * absmax[e / blocksize];  // fp32 product, then one rounding to fp16
+      dst[e] = f32_to_f16_bits(prod);
+    };
+  };
+  const double nf4_host1 = time_host_loop(nf4_host(want), n, 1, 1);
+  const double nf4_hostN = time_host_loop(nf4_host(got), n, cores, host_passes);
+  if (host_only) {
+    std::printf("Average execution time of NF4 dequantize kernel with block size %d: %f (us)\n", blocksize, nf4_hostN * 1e6);
+    std::printf("%s\n", got == want ? "PASS" : "FAIL");
+    std::printf("  (host only: OpenMP loop on %d threads; one thread: %f us)\n", cores, nf4_host1 * 1e6);
+    return out == ref && got == want ? 0 : 1;
+  }
+  HQ_OK_OR_DIE(hq_init());
   DevBuf<float> d_A(n), d_code(256);
   DevBuf<uint8_t> d_out(n);
   d_A.upload(A);
   d_code.upload(code);
-  const int block_size = 256;
   HIP_OK(hipDeviceSynchronize());
   auto start = std::chrono::steady_clock::now();
   for (int i = 0; i < repeat; ++i) HQ_OK_OR_DIE(hq_quantize_dynamic8(d_code.p, d_A.p, d_out.p, (int64_t)n, nullptr));
@@ -91,22 +137,10 @@ int main(int argc, char* argv[]) {
   d_out.download(out.data(), n);
   const bool ok1 = out == ref;
   std::printf("%s\n", ok1 ? "PASS" : "FAIL");
-  std::printf("  (%.1f GB/s of 5 B/element traffic)\n", 5.0 * n / ((t_ns * 1e-3) / repeat) * 1e-3);
+  std::printf("  (%.1f GB/s of 5 B/element traffic; host loop: %.0f us on one thread, %.0f us on %d OpenMP threads)\n",
+              5.0 * n / ((t_ns * 1e-3) / repeat) * 1e-3, host1 * 1e6, hostN * 1e6, cores);
 
   // ---- part 2: blockwise NF4 dequantisation ------------------------------------------------
-  const int blocksize = 64;
-  SeededRng rng(1234);
-  std::vector<uint8_t> packed((n + 1) / 2);
-  std::vector<float> absmax((n + blocksize - 1) / blocksize);
-  for (auto& b : packed) b = (uint8_t)(rng.u32() >> 24);
-  for (auto& a : absmax) a = (float)rng.uniform(0.5, 2.0);
-  std::vector<uint16_t> want(n), got(n);
-  for (size_t e = 0; e < n; ++e) {
-    const uint8_t b = packed[e >> 1];
-    const unsigned c = (e & 1) ? (b & 15u) : (b >> 4);
-    volatile float prod = kNf4[c] * absmax[e / blocksize];  // fp32 product, then one rounding to fp16
-    want[e] = f32_to_f16_bits(prod);
-  }
   // rotate over enough distinct buffers that no call is served from the 256 MB cache
   const size_t per_call = packed.size() + absmax.size() * 4 + n * 2;
   const int nbuf = (int)std::max<size_t>(2, (size_t)(600e6 / (double)per_call) + 1);
@@ -130,5 +164,6 @@ int main(int argc, char* argv[]) {
   std::printf("%s\n", ok2 ? "PASS" : "FAIL");
   std::printf("  (%.1f GB/s = %.1f%% of %.0f GB/s HBM peak, %zu bytes per call, %d rotated buffers)\n",
               per_call / us * 1e-3, per_call / us * 1e-3 / kHbmPeakGBs * 100, kHbmPeakGBs, per_call, nbuf);
+  std::printf("  (host loop: %.0f us on one thread, %.0f us on %d OpenMP threads)\n", nf4_host1 * 1e6, nf4_hostN * 1e6, cores);
   return ok1 && ok2 ? 0 : 1;
 }

@@ -112,39 +112,54 @@ int hq_get_workspace(hipStream_t stream, size_t need_floats, size_t need_counter
   return HQ_OK;
 }
 
+// Upper bound of what any hq_q3_matvec call with K <= max_K, N <= max_N (any batch) and any hq_lut_gemv call
+// of those sizes takes from its stream's workspace on a device of `cus` compute units, with the default launch
+// policy.  Host arithmetic only.  (tests/test_workspace_cpu.py checks it against the per-call need over a
+// sweep of shapes.)
+static void reserve_bound(int cus, int max_K, int max_N, size_t* floats, size_t* counters) {
+  // batched GEMM: re-ordered activations of 64 rows (128 bytes per input feature, K padded to 1024), the row
+  // sums and scales, and - whenever some N <= max_N leaves compute units without a 128-column tile and K has
+  // two or more ranges of four steps, i.e. always but for very short K - the raw sums of its K split, at most
+  // 256 blocks of 64 x 128
+  const size_t kpad = ((size_t)max_K + 1023) / 1024 * 1024;
+  const size_t gemm_floats = kpad * 32 + 128 + (kpad >= 2048 ? (size_t)256 * 64 * 128 : 0);
+  // split-K matvecs: a partial row of 64 floats per column tile and split - one split per 4096 elements of K
+  // up to eight whatever the tile count (a shorter K than max_K may split where max_K itself does not), beyond
+  // that only as many as give every compute unit a workgroup; narrow tiles (16 or 32 columns) only while
+  // tiles x splits stay within the compute units.  The LUT kernels: two workgroups per compute unit, 128
+  // floats each.
+  const size_t tiles = ((size_t)max_N + 63) / 64;
+  const size_t rounds = ((size_t)max_K + 4095) / 4096;
+  const size_t full_split = tiles * (rounds <= 8 ? rounds : 8);
+  const size_t per_cu = tiles + 2 * (size_t)cus;
+  size_t split_floats = (full_split > per_cu ? full_split : per_cu) * 64 * 2;
+  // batches 2 ... 64 on the matvec-like kernel: one partial row per tile, range of K and activation row, at most
+  // 8192 of them whatever the shape
+  if ((size_t)8192 * 64 > split_floats) split_floats = (size_t)8192 * 64;
+  *floats = gemm_floats > split_floats ? gemm_floats : split_floats;
+  // arrival counters: one per column tile, narrow tiles four per 64 columns, row blocks sixteen per tile
+  *counters = tiles > 1 ? tiles * 16 : 16;
+}
+
+extern "C" int hq_reserve_need(int compute_units, int max_K, int max_N, int64_t* floats, int64_t* counters) {
+  if (!floats || !counters) return HQ_ERR_NULL_POINTER;
+  if (max_K < 0 || max_N < 0 || compute_units <= 0) return HQ_ERR_BAD_SHAPE;
+  size_t f = 0, c = 0;
+  reserve_bound(compute_units, max_K, max_N, &f, &c);
+  *floats = (int64_t)f;
+  *counters = (int64_t)c;
+  return HQ_OK;
+}
+
 extern "C" int hq_reserve_workspace(void* stream, int max_K, int max_N) {
   if (max_K < 0 || max_N < 0) return HQ_ERR_BAD_SHAPE;
   const HqDevice* d = nullptr;
   int rc = hq_current_device(&d);
   if (rc != HQ_OK) return rc;
-  // batched GEMM: re-ordered activations of 64 rows (128 bytes per input feature, K padded to 1024) plus
-  // the row sums and scales; split-K matvecs: a partial row of 64 floats per column tile and split (two rows
-  // for a batch of 2) - up to eight splits (one per 4096 elements of K) whatever the tile count, beyond that
-  // only as many as give every compute unit a workgroup (the LUT table kernel: two per compute unit, 128
-  // floats each)
-  const size_t kpad = ((size_t)max_K + 1023) / 1024 * 1024;
-  // (plus, when the 128-column tiles do not fill the device, the raw sums of its K split: at most 256
-  // blocks of 64 x 128)
-  const size_t tiles128 = ((size_t)max_N + 127) / 128;
-  const size_t gemm_floats = kpad * 32 + 128 + (2 * tiles128 <= (size_t)d->cus ? (size_t)256 * 64 * 128 : 0);
-  const size_t tiles = ((size_t)max_N + 63) / 64;
-  const size_t rounds = ((size_t)max_K + 4095) / 4096;
-  const size_t full_split = tiles * (rounds <= 8 ? rounds : 1);
-  const size_t per_cu = tiles + 2 * (size_t)d->cus;
-  size_t split_floats = (full_split > per_cu ? full_split : per_cu) * 64 * 2;
-  // batches 2 ... 64 on the matvec-like kernel: one partial row per tile, round of K and activation row, at most 8192
-  size_t block_splits = rounds;
-  if (rounds > 8) {  // longer K: two workgroups per compute unit
-    block_splits = 2 * (size_t)d->cus / (tiles ? tiles : 1);
-    if (block_splits < 1) block_splits = 1;
-    if (block_splits > rounds) block_splits = rounds;
-  }
-  // (up to 64 rows as row blocks of four: the same bound, and a counter per tile and row block)
-  const size_t block_rows = tiles * block_splits * 64 < 8192 ? tiles * block_splits * 64 : 8192;
-  if (block_rows * 64 > split_floats) split_floats = block_rows * 64;
+  size_t floats = 0, counters = 0;
+  reserve_bound(d->cus, max_K, max_N, &floats, &counters);
   HqWorkspace ws;
-  return hq_get_workspace((hipStream_t)stream, gemm_floats > split_floats ? gemm_floats : split_floats,
-                          tiles > 1 ? tiles * 16 : 16, &ws);
+  return hq_get_workspace((hipStream_t)stream, floats, counters, &ws);
 }
 
 extern "C" int hq_shutdown(void) {

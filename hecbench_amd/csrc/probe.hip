@@ -1,0 +1,104 @@
+// Memory-system probes: what this device delivers to the simplest possible kernels, so that a benchmark
+// line can set a kernel's rate beside a rate measured on the same box instead of a data-sheet figure only.
+//   hq_probe_stream: a plain streaming read (mode 0) or copy (mode 1) of `bytes` bytes;
+//   hq_probe_gather16: independent 16-byte reads at pseudo-random entries of a table (the access
+//                      pattern of a code-book lookup), the rate of which is bounded by cache requests per
+//                      second, not by bytes.
+// There is no counterpart in the HeCBench tree; the benchmark drivers call them for their report.
+#include "hq_internal.h"
+
+namespace {
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+
+// units = 16-byte pieces; every thread keeps four loads in flight and walks the range grid-stride
+template <bool COPY>
+__global__ __launch_bounds__(256) void probe_stream_kernel(const u4v* __restrict__ src, u4v* __restrict__ dst,
+                                                          long units, u4v* __restrict__ sink) {
+  const long stride = (long)gridDim.x * 256;
+  long i = (long)blockIdx.x * 256 + threadIdx.x;
+  u4v acc = {0u, 0u, 0u, 0u};
+  for (; i + 3 * stride < units; i += 4 * stride) {
+    u4v v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (COPY) __builtin_nontemporal_store(v[u], dst + i + u * stride);
+      else acc ^= v[u];
+    }
+  }
+  for (; i < units; i += stride) {
+    const u4v v = __builtin_nontemporal_load(src + i);
+    if (COPY) __builtin_nontemporal_store(v, dst + i);
+    else acc ^= v;
+  }
+  // keeps the loads alive; the condition is false for any realistic data
+  if (!COPY && (acc.x & acc.y & acc.z & acc.w) == 0xffffffffu && acc.x + acc.y == 12345u) *sink = acc;
+}
+
+// every lane performs `per_lane` independent 16-byte reads, eight in flight at a time
+__global__ __launch_bounds__(256) void probe_gather_kernel(const u4v* __restrict__ table, uint32_t mask, int per_lane,
+                                                          u4v* __restrict__ sink) {
+  uint32_t s = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
+  u4v acc = {0u, 0u, 0u, 0u};
+  for (int i = 0; i < per_lane; i += 8) {
+    u4v v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      s ^= s << 13; s ^= s >> 17; s ^= s << 5;  // xorshift32
+      v[u] = table[s & mask];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc ^= v[u];
+  }
+  if ((acc.x & acc.y & acc.z & acc.w) == 0xffffffffu && acc.x + acc.y == 12345u) *sink = acc;
+}
+}  // namespace
+
+extern "C" int hq_probe_stream(int mode, const void* src, void* dst, int64_t bytes, void* stream) {
+  if (!src || !dst) return HQ_ERR_NULL_POINTER;
+  if (mode != 0 && mode != 1) return HQ_ERR_BAD_ENUM;
+  if (bytes < 16 || (bytes & 15)) return HQ_ERR_BAD_SHAPE;
+  if (((uintptr_t)src & 15) || ((uintptr_t)dst & 15)) return HQ_ERR_MISALIGNED;
+  const HqDevice* dev = nullptr;
+  const int rc = hq_current_device(&dev);
+  if (rc != HQ_OK) return rc;
+  const long units = bytes / 16;
+  long wgs = (units + 1023) / 1024;  // at most one trip of four loads per thread ...
+  const long cap = (long)dev->cus * 16;  // ... but no more than sixteen workgroups per compute unit
+  if (wgs > cap) wgs = cap;
+  if (mode == 1)
+    hipLaunchKernelGGL(probe_stream_kernel<true>, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream,
+                       (const u4v*)src, (u4v*)dst, units, (u4v*)dst);
+  else  // mode 0 writes nothing (dst is only the never-taken sink)
+    hipLaunchKernelGGL(probe_stream_kernel<false>, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream,
+                       (const u4v*)src, (u4v*)dst, units, (u4v*)dst);
+  return hq_launch_status();
+}
+
+extern "C" int hq_probe_gather16(const void* table, int64_t table_bytes, int64_t gathers, void* sink16, void* stream) {
+  if (!table || !sink16) return HQ_ERR_NULL_POINTER;
+  if (table_bytes < 16 || (table_bytes & (table_bytes - 1)) || table_bytes > ((int64_t)1 << 32)) return HQ_ERR_BAD_SHAPE;
+  if (gathers <= 0) return HQ_ERR_BAD_SHAPE;
+  if (((uintptr_t)table & 15) || ((uintptr_t)sink16 & 15)) return HQ_ERR_MISALIGNED;
+  const HqDevice* dev = nullptr;
+  const int rc = hq_current_device(&dev);
+  if (rc != HQ_OK) return rc;
+  // eight workgroups per compute unit; the number of reads is rounded up to a whole trip of every lane
+  const long lanes = (long)dev->cus * 8 * 256;
+  long per_lane = (gathers + lanes - 1) / lanes;
+  per_lane = (per_lane + 7) / 8 * 8;
+  if (per_lane > (1 << 24)) return HQ_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(probe_gather_kernel, dim3((unsigned)(dev->cus * 8)), dim3(256), 0, (hipStream_t)stream,
+                     (const u4v*)table, (uint32_t)(table_bytes / 16 - 1), (int)per_lane, (u4v*)sink16);
+  return hq_launch_status();
+}
+
+extern "C" int64_t hq_probe_gather16_count(int64_t gathers) {
+  const HqDevice* dev = nullptr;
+  if (gathers <= 0 || hq_current_device(&dev) != HQ_OK) return -1;
+  const long lanes = (long)dev->cus * 8 * 256;
+  long per_lane = (gathers + lanes - 1) / lanes;
+  per_lane = (per_lane + 7) / 8 * 8;
+  return per_lane * lanes;
+}

@@ -497,6 +497,7 @@ int hq_q3_block_launch(const void* x, const int32_t* qweight, const float* scale
                        int K, int N, int M, int nsplit, int rpw, int mblocks, float* partial, unsigned* counters,
                        unsigned flags, hipStream_t stream);
 int hq_q3_block_groups_per_round(void);
+int hq_q3_gemm_need(int cus, int K, int N, size_t* floats, size_t* counters);
 
 namespace {
 // Zeroes n words with a kernel (a memset node inside a captured graph is not an option for callers
@@ -516,13 +517,13 @@ constexpr size_t kBlockPartialRows = 8192;
 // How the kernel for 2 ... 8 rows cuts K: up to eight rounds of 4096 elements, one workgroup per round (as the
 // batch-1 kernel); beyond that as many workgroups per column tile as give every compute unit two, each taking
 // several rounds one after the other.
-void q3_block_split(const HqDevice* dev, int K, int N, int batch_M, int* nsplit, int* rpw) {
+void q3_block_split(int cus, int K, int N, int batch_M, int* nsplit, int* rpw) {
   const int gpr = hq_q3_block_groups_per_round();
   const int rounds = (K / 32 + gpr - 1) / gpr;
   const int ntiles = (N + 63) / 64;
   int ns = rounds;
   if (rounds > 8) {
-    ns = 2 * dev->cus / ntiles;
+    ns = 2 * cus / ntiles;
     if (ns < 1) ns = 1;
     if (ns > rounds) ns = rounds;
   }
@@ -536,7 +537,7 @@ constexpr int kRowBlockBatchMax = 64;  // rows a batch may have as row blocks of
 
 // Row blocks (workgroups per column tile, four rows each) of a batch of more than four rows; 1: passes inside
 // one workgroup; 0: the four-rows-per-pass kernel does not take this batch at all.
-int q3_block_row_blocks(const HqDevice* dev, int K, int N, int batch_M, int nsplit, int rpw) {
+int q3_block_row_blocks(int cus, int K, int N, int batch_M, int nsplit, int rpw) {
   (void)K;
   // Measured (us per call, passes in one workgroup or the GEMM -> row blocks): with a CU for every workgroup,
   // K=4096, N=4096: 5 rows 7.2 -> 5.2, 8 rows 8.4 -> 5.3, 12 rows 11.7 -> 5.3, 16 rows 12.7 -> 5.6; with up to
@@ -553,18 +554,18 @@ int q3_block_row_blocks(const HqDevice* dev, int K, int N, int batch_M, int nspl
                         (nsplit == 1 || groups * mb * 4 <= kBlockPartialRows);
   if (possible) {
     const size_t wgs = groups * mb;
-    if (mode == 1 || wgs <= (size_t)dev->cus || (batch_M >= 7 && wgs <= 4 * (size_t)dev->cus)) return mb;
+    if (mode == 1 || wgs <= (size_t)cus || (batch_M >= 7 && wgs <= 4 * (size_t)cus)) return mb;
   }
   return batch_M <= 12 ? 1 : 0;
 }
 
-int q3_plan(const HqDevice* dev, int K, int N, int batch_M) {
+int q3_plan(int cus, int K, int N, int batch_M) {
   if (batch_M == 1) return HQ_Q3_PLAN_MATVEC;
   const int limit = hq_tune(HQ_TUNE_Q3_SMALL_BATCH, kRowBlockBatchMax);  // 0: every batch takes the GEMM
   int nsplit, rpw;
-  q3_block_split(dev, K, N, batch_M, &nsplit, &rpw);
+  q3_block_split(cus, K, N, batch_M, &nsplit, &rpw);
   if (batch_M > limit) return HQ_Q3_PLAN_GEMM;
-  const int mb = q3_block_row_blocks(dev, K, N, batch_M, nsplit, rpw);
+  const int mb = q3_block_row_blocks(cus, K, N, batch_M, nsplit, rpw);
   if (mb > 1) return HQ_Q3_PLAN_BLOCK;
   if (mb == 0) return HQ_Q3_PLAN_GEMM;
   // 2 ... 8 rows in one workgroup per tile and K range.  Five to eight rows take
@@ -574,25 +575,30 @@ int q3_plan(const HqDevice* dev, int K, int N, int batch_M) {
   const size_t groups = (size_t)((N + 63) / 64) * nsplit;
   const size_t tiles128 = (size_t)(N + 127) / 128;
   if (batch_M <= 8 && (nsplit == 1 || groups * batch_M <= kBlockPartialRows) &&
-      (batch_M <= 4 || (rpw == 1 && 8 * tiles128 < 7 * (size_t)dev->cus)))
+      (batch_M <= 4 || (rpw == 1 && 8 * tiles128 < 7 * (size_t)cus)))
     return HQ_Q3_PLAN_BLOCK;
   // 9 ... 12 rows, three passes: where the launch has at most one workgroup per compute unit (it is a matter
   // of latency there, and the GEMM needs three launches)
-  if (batch_M <= 12 && rpw == 1 && groups <= (size_t)dev->cus) return HQ_Q3_PLAN_BLOCK;
+  if (batch_M <= 12 && rpw == 1 && groups <= (size_t)cus) return HQ_Q3_PLAN_BLOCK;
   return HQ_Q3_PLAN_GEMM;
 }
 
-// How the digit kernels (batch 1 and batch 2) divide K: a workgroup covers gpr k-groups per round and walks
-// its K range in rounds (the next round's loads are in flight during the current one), or K is split across
-// workgroups whose partial sums (rows_out rows of 64 floats per workgroup) the last one to arrive adds up.
-struct Q3Split {
-  int gpw;     // k-groups per workgroup, whole rounds
-  int nsplit;  // workgroups per column tile
-  float* partial;
-  unsigned* counters;
+// How the digit kernels divide K: a workgroup covers gpr k-groups per round and walks its K range in rounds
+// (the next round's loads are in flight during the current one), or K is split across workgroups whose
+// partial sums (rows_out rows of 64 floats per workgroup) the last one to arrive adds up.
+// Planning is pure arithmetic (the launch, the workspace reservation and the size query share it);
+// q3_split_acquire then takes the scratch, once, when the plan is final.
+struct Q3SplitPlan {
+  int gpw;          // k-groups per workgroup, whole rounds
+  int nsplit;       // workgroups per column tile
+  int ntiles;       // column tiles (times row blocks) = arrival counters
+  size_t floats;    // partial sums: 0 without a split
+  bool too_large;   // the fixed scratch cannot hold this plan
 };
-int q3_split_k(const HqDevice* dev, int G, int gpr, int ntiles, int rows_out, bool single_round,
-               const HqQ3Scratch* fixed, hipStream_t stream, Q3Split* out) {
+struct Q3Limits {  // what a fixed scratch holds; null pointer = the stream's workspace (grows on demand)
+  size_t partial_floats, ncounters;
+};
+Q3SplitPlan q3_split_plan(int cus, int G, int gpr, int ntiles, int rows_out, bool single_round, const Q3Limits* fixed) {
   const int max_split = (G + gpr - 1) / gpr;
   const size_t tile_floats = (size_t)ntiles * rows_out * 64;
   int nsplit = single_round ? max_split : hq_tune(HQ_TUNE_Q3_KSPLIT, 0);
@@ -603,33 +609,107 @@ int q3_split_k(const HqDevice* dev, int G, int gpr, int ntiles, int rows_out, bo
     // 20.4 -> 15.1 us; N=28672, 448 tiles, 21.4 -> 18.6 us; K=28672, N=8192 21.7 -> 19.6 us).  Longer K: only
     // as many splits as it takes to give every CU a workgroup - each split adds a partial-sum row per tile
     // and a device-scope round trip (K=49152, N=12288: 43 us unsplit, 51-58 us split).
-    nsplit = max_split <= 8 ? max_split : dev->cus / ntiles;
+    nsplit = max_split <= 8 ? max_split : cus / ntiles;
     if (fixed && nsplit > 1 && (tile_floats * nsplit > fixed->partial_floats || (size_t)ntiles > fixed->ncounters))
-      nsplit = dev->cus / ntiles;  // the fixed scratch is too small for the full split
+      nsplit = cus / ntiles;  // the fixed scratch is too small for the full split
   }
   if (nsplit > max_split) nsplit = max_split;
   if (nsplit < 1) nsplit = 1;
-  int gpw = (G + nsplit - 1) / nsplit;
-  gpw = (gpw + gpr - 1) / gpr * gpr;  // whole rounds
-  nsplit = (G + gpw - 1) / gpw;
-  out->gpw = gpw; out->nsplit = nsplit; out->partial = nullptr; out->counters = nullptr;
-  if (nsplit > 1 && fixed) {
+  Q3SplitPlan p;
+  p.gpw = (G + nsplit - 1) / nsplit;
+  p.gpw = (p.gpw + gpr - 1) / gpr * gpr;  // whole rounds
+  p.nsplit = (G + p.gpw - 1) / p.gpw;
+  p.ntiles = ntiles;
+  p.floats = p.nsplit > 1 ? tile_floats * p.nsplit : 0;
+  p.too_large = p.nsplit > 1 && fixed && (p.floats > fixed->partial_floats || (size_t)ntiles > fixed->ncounters);
+  return p;
+}
+
+struct Q3Split {
+  float* partial;
+  unsigned* counters;
+};
+int q3_split_acquire(const Q3SplitPlan& p, const HqQ3Scratch* fixed, hipStream_t stream, Q3Split* out) {
+  out->partial = nullptr;
+  out->counters = nullptr;
+  if (p.nsplit <= 1) return HQ_OK;
+  if (fixed) {
     // fixed scratch shared by every call on this device: the counters start from zero by a fill kernel
     // on the same stream (they also reset themselves, but an earlier call may have been cut short)
-    if (tile_floats * nsplit > fixed->partial_floats || (size_t)ntiles > fixed->ncounters) return HQ_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((ntiles + 255) / 256), dim3(256), 0, stream, fixed->counters, ntiles);
+    if (p.too_large) return HQ_ERR_TOO_LARGE;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((p.ntiles + 255) / 256), dim3(256), 0, stream, fixed->counters, p.ntiles);
     const int rc = hq_launch_status();
     if (rc != HQ_OK) return rc;
     out->partial = fixed->partial;
     out->counters = fixed->counters;
-  } else if (nsplit > 1) {
-    HqWorkspace ws;
-    const int rc = hq_get_workspace(stream, tile_floats * nsplit, (size_t)ntiles, &ws);
-    if (rc != HQ_OK) return rc;
-    out->partial = ws.partial;
-    out->counters = ws.counters;
+    return HQ_OK;
   }
+  HqWorkspace ws;
+  const int rc = hq_get_workspace(stream, p.floats, (size_t)p.ntiles, &ws);
+  if (rc != HQ_OK) return rc;
+  out->partial = ws.partial;
+  out->counters = ws.counters;
   return HQ_OK;
+}
+
+// Launch shape of the batch-1 kernel (pure arithmetic).
+struct Q3MatvecPlan {
+  int waves, steps, cpl, ntiles;
+  Q3SplitPlan split;
+};
+Q3MatvecPlan q3_matvec_shape(int cus, int K, int N, const Q3Limits* fixed) {
+  const int G = K / 32;
+  Q3MatvecPlan m;
+  m.ntiles = (N + 63) / 64;
+  // A workgroup of WAVES waves covers WAVES*4*STEPS k-groups per round and walks its K range in rounds
+  // (the next round's loads are in flight during the current one), or K is split across workgroups whose
+  // partial sums the last one to arrive adds up.
+  m.waves = hq_tune(HQ_TUNE_Q3_WAVES, 8);
+  m.steps = hq_tune(HQ_TUNE_Q3_STEPS, 0);
+  if (m.waves != 4 && m.waves != 8 && m.waves != 16) m.waves = 8;
+  if (m.waves == 16) m.steps = 1;  // register budget of 16-wave workgroups
+  if (m.steps != 1 && m.steps != 2 && m.steps != 4 && (m.steps != 8 || m.waves != 4)) {
+    m.steps = 4;
+    while (m.steps > 1 && m.waves * 4 * (m.steps / 2) >= G) m.steps /= 2;  // short K: fewer steps
+  }
+  const int gpr = m.waves * 4 * m.steps;  // k-groups one workgroup covers per round
+  // Few column tiles (the default workgroup, one round of K per workgroup): narrower tiles, 32 or 16 columns,
+  // as long as every workgroup still has a CU of its own - the idle CUs' load queues join in.
+  // HQ_Q3_TILE: 4, 2 or 1 columns per lane, unset: by the launch size.
+  m.cpl = 4;
+  {
+    const int rounds = (G + gpr - 1) / gpr;
+    const int want = hq_tune(HQ_TUNE_Q3_TILE, -1);
+    if (m.waves == 8 && m.steps == 4 && rounds <= 8 && hq_tune(HQ_TUNE_Q3_KSPLIT, -1) < 0) {
+      if (want == 1 || want == 2) m.cpl = want;
+      else if (want < 0) m.cpl = 4 * m.ntiles * rounds <= cus ? 1 : (2 * m.ntiles * rounds <= cus ? 2 : 4);
+    }
+    if (m.cpl < 4) m.ntiles = (N + 16 * m.cpl - 1) / (16 * m.cpl);
+  }
+  m.split = q3_split_plan(cus, G, gpr, m.ntiles, 1, false, fixed);
+  if (m.cpl < 4 && (m.split.gpw > gpr || m.split.too_large)) {  // narrow tiles are for single-round workgroups only
+    m.cpl = 4;
+    m.ntiles = (N + 63) / 64;
+    m.split = q3_split_plan(cus, G, gpr, m.ntiles, 1, false, fixed);
+  }
+  return m;
+}
+
+// Split of the kernel for batches 2 ... 64 (pure arithmetic): row blocks or passes.
+struct Q3BlockPlan {
+  int nsplit, rpw, mblocks;
+  Q3SplitPlan split;
+};
+Q3BlockPlan q3_block_shape(int cus, int K, int N, int batch_M, const Q3Limits* fixed) {
+  Q3BlockPlan b;
+  q3_block_split(cus, K, N, batch_M, &b.nsplit, &b.rpw);
+  b.mblocks = q3_block_row_blocks(cus, K, N, batch_M, b.nsplit, b.rpw);
+  if (b.mblocks < 1) b.mblocks = 1;
+  if (b.mblocks > 1)
+    b.split = q3_split_plan(cus, K / 32, hq_q3_block_groups_per_round(), (N + 63) / 64 * b.mblocks, 4, true, fixed);
+  else
+    b.split = q3_split_plan(cus, K / 32, b.rpw * hq_q3_block_groups_per_round(), (N + 63) / 64, batch_M, true, fixed);
+  return b;
 }
 }  // namespace
 
@@ -637,7 +717,37 @@ extern "C" int hq_q3_matvec_plan(int K, int N, int batch_M) {
   if (K <= 0 || N <= 0 || batch_M <= 0 || (K & 31) || (N & 3)) return HQ_ERR_BAD_SHAPE;
   const HqDevice* dev = nullptr;
   const int rc = hq_current_device(&dev);
-  return rc != HQ_OK ? rc : q3_plan(dev, K, N, batch_M);
+  return rc != HQ_OK ? rc : q3_plan(dev->cus, K, N, batch_M);
+}
+
+// Workspace one hq_q3_matvec call takes from its stream on a device of `cus` compute units: the same plan
+// functions as the launch (host arithmetic only, no device is touched).
+int hq_q3_workspace_need_impl(int cus, int K, int N, int batch_M, size_t* floats, size_t* counters) {
+  if (K <= 0 || N <= 0 || batch_M <= 0 || (K & 31) || (N & 3) || cus <= 0) return HQ_ERR_BAD_SHAPE;
+  *floats = 0;
+  *counters = 0;
+  if (batch_M == 1) {
+    const Q3MatvecPlan m = q3_matvec_shape(cus, K, N, nullptr);
+    *floats = m.split.floats;
+    *counters = m.split.nsplit > 1 ? (size_t)m.split.ntiles : 0;
+    return HQ_OK;
+  }
+  if (q3_plan(cus, K, N, batch_M) == HQ_Q3_PLAN_BLOCK) {
+    const Q3BlockPlan b = q3_block_shape(cus, K, N, batch_M, nullptr);
+    *floats = b.split.floats;
+    *counters = b.split.nsplit > 1 ? (size_t)b.split.ntiles : 0;
+    return HQ_OK;
+  }
+  return hq_q3_gemm_need(cus, K, N, floats, counters);
+}
+
+extern "C" int hq_q3_workspace_need(int compute_units, int K, int N, int batch_M, int64_t* floats, int64_t* counters) {
+  if (!floats || !counters) return HQ_ERR_NULL_POINTER;
+  size_t f = 0, c = 0;
+  const int rc = hq_q3_workspace_need_impl(compute_units, K, N, batch_M, &f, &c);
+  *floats = (int64_t)f;
+  *counters = (int64_t)c;
+  return rc;
 }
 
 extern "C" int hq_q3_matvec(const void* x, int x_dtype, const int32_t* qweight, const float* scales,
@@ -657,72 +767,43 @@ int hq_q3_matvec_impl(const void* x, int x_dtype, const int32_t* qweight, const 
   if (((uintptr_t)qweight & 15) || ((uintptr_t)x & 15) ||  // activations are read with 128-bit loads
       ((uintptr_t)y & 3) || ((uintptr_t)scales & 3) || ((uintptr_t)zeros & 3))
     return HQ_ERR_MISALIGNED;
+  // batches share one alignment contract whichever kernel the plan picks: the GEMM reads scale / zero and
+  // writes y four columns at a time
+  if (batch_M > 1 && (((uintptr_t)scales & 15) || ((uintptr_t)zeros & 15) || ((uintptr_t)y & 15))) return HQ_ERR_MISALIGNED;
   const HqDevice* dev = nullptr;
   int rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
+  Q3Limits lim_s, *lim = nullptr;
+  if (fixed) {
+    lim_s.partial_floats = fixed->partial_floats;
+    lim_s.ncounters = fixed->ncounters;
+    lim = &lim_s;
+  }
+  Q3Split sp;
   if (batch_M > 1) {
     if (x_dtype != HQ_DTYPE_F16) return HQ_ERR_BAD_ENUM;
     // Small batches ride on the matvec's digit kernels (one pass over the weights, one launch); everything
     // else takes the batched GEMM.
-    const int plan = q3_plan(dev, K, N, batch_M);
-    if (plan == HQ_Q3_PLAN_BLOCK) {
-      Q3Split sp;
-      int nsplit, rpw;
-      q3_block_split(dev, K, N, batch_M, &nsplit, &rpw);
-      int mblocks = q3_block_row_blocks(dev, K, N, batch_M, nsplit, rpw);
-      if (mblocks < 1) mblocks = 1;
-      if (mblocks > 1)
-        rc = q3_split_k(dev, K / 32, hq_q3_block_groups_per_round(), (N + 63) / 64 * mblocks, 4, true, fixed, stream, &sp);
-      else
-        rc = q3_split_k(dev, K / 32, rpw * hq_q3_block_groups_per_round(), (N + 63) / 64, batch_M, true, fixed, stream, &sp);
+    if (q3_plan(dev->cus, K, N, batch_M) == HQ_Q3_PLAN_BLOCK) {
+      const Q3BlockPlan b = q3_block_shape(dev->cus, K, N, batch_M, lim);
+      if (b.split.nsplit != b.nsplit) return HQ_ERR_BAD_SHAPE;
+      rc = q3_split_acquire(b.split, fixed, stream, &sp);
       if (rc != HQ_OK) return rc;
-      if (sp.nsplit != nsplit) return HQ_ERR_BAD_SHAPE;
-      return hq_q3_block_launch(x, qweight, scales, zeros, y, K, N, batch_M, nsplit, rpw, mblocks, sp.partial, sp.counters,
-                                flags, stream);
+      return hq_q3_block_launch(x, qweight, scales, zeros, y, K, N, batch_M, b.nsplit, b.rpw, b.mblocks, sp.partial,
+                                sp.counters, flags, stream);
     }
     return hq_q3_gemm_launch(x, qweight, scales, zeros, y, K, N, batch_M, flags, stream, fixed);
   }
 
-  const int G = K / 32;
-  int ntiles = (N + 63) / 64;
-  // Launch shape: a workgroup of WAVES waves covers WAVES*4*STEPS k-groups per round and
-  // walks its K range in rounds (the next round's loads are in flight during the current
-  // one), or K is split across workgroups whose partial sums the last one to arrive adds up.
-  int waves = hq_tune(HQ_TUNE_Q3_WAVES, 8);
-  int steps = hq_tune(HQ_TUNE_Q3_STEPS, 0);
-  if (waves != 4 && waves != 8 && waves != 16) waves = 8;
-  if (waves == 16) steps = 1;  // register budget of 16-wave workgroups
-  if (steps != 1 && steps != 2 && steps != 4 && (steps != 8 || waves != 4)) {
-    steps = 4;
-    while (steps > 1 && waves * 4 * (steps / 2) >= G) steps /= 2;  // short K: fewer steps
-  }
-  const int gpr = waves * 4 * steps;  // k-groups one workgroup covers per round
-  // Few column tiles (the default workgroup, one round of K per workgroup): narrower tiles, 32 or 16 columns,
-  // as long as every workgroup still has a CU of its own - the idle CUs' load queues join in.
-  // HQ_Q3_TILE: 4, 2 or 1 columns per lane, unset: by the launch size.
-  int cpl = 4;
-  {
-    const int rounds = (G + gpr - 1) / gpr;
-    const int want = hq_tune(HQ_TUNE_Q3_TILE, -1);
-    if (waves == 8 && steps == 4 && rounds <= 8 && hq_tune(HQ_TUNE_Q3_KSPLIT, -1) < 0) {
-      if (want == 1 || want == 2) cpl = want;
-      else if (want < 0) cpl = 4 * ntiles * rounds <= dev->cus ? 1 : (2 * ntiles * rounds <= dev->cus ? 2 : 4);
-    }
-    if (cpl < 4) ntiles = (N + 16 * cpl - 1) / (16 * cpl);
-  }
-  Q3Split sp;
-  rc = q3_split_k(dev, G, gpr, ntiles, 1, false, fixed, stream, &sp);
-  if (rc == HQ_OK && cpl < 4 && sp.gpw > gpr) {  // narrow tiles are for single-round workgroups only
-    cpl = 4;
-    ntiles = (N + 63) / 64;
-    rc = q3_split_k(dev, G, gpr, ntiles, 1, false, fixed, stream, &sp);
-  }
+  const Q3MatvecPlan m = q3_matvec_shape(dev->cus, K, N, lim);
+  rc = q3_split_acquire(m.split, fixed, stream, &sp);
   if (rc != HQ_OK) return rc;
+  const int waves = m.waves, steps = m.steps, cpl = m.cpl, ntiles = m.ntiles;
 
   Q3Args a;
   a.x = x; a.w = reinterpret_cast<const uint32_t*>(qweight); a.scales = scales; a.zeros = zeros;
-  a.y = y; a.partial = sp.partial; a.counters = sp.counters; a.K = K; a.N = N; a.gpw = sp.gpw;
-  a.nsplit = sp.nsplit; a.x_f16 = (x_dtype == HQ_DTYPE_F16); a.flags = flags;
+  a.y = y; a.partial = sp.partial; a.counters = sp.counters; a.K = K; a.N = N; a.gpw = m.split.gpw;
+  a.nsplit = m.split.nsplit; a.x_f16 = (x_dtype == HQ_DTYPE_F16); a.flags = flags;
 #define HQ_Q3_CASE(W, S) \
   if (waves == W && steps == S) return launch_matvec<W, S>(a, ntiles, dev->cus, cpl, stream);
   HQ_Q3_CASE(16, 1)

@@ -1,4 +1,6 @@
-// GPTQ 3-bit product for small batches (2 ... 12 activation rows) on the matvec's matrix-core kernel, gfx950.
+// GPTQ 3-bit product for batches of 2 ... 64 activation rows on the matvec's matrix-core kernel, gfx950: four
+// rows per pass over the weights; up to twelve rows as passes of one workgroup, up to 64 as row blocks of four
+// rows in workgroups of their own (q3_block_rows_kernel below).
 //
 // q3.hip (batch 1) carries the activations as fixed point relative to the largest magnitude a wave sees in a
 // round, eight 4-bit digits per activation, so one matrix-core pass over the weights serves one row (a

@@ -331,29 +331,51 @@ int launch_gemm(const GemmArgs& a, hipStream_t stream) {
 
 }  // namespace
 
+// Launch plan of the batched GEMM (host arithmetic only; the launch, the workspace reservation and the size
+// query share it).  K split: column tiles alone leave most CUs idle when N is small (N = 4096: 32 tiles), so K
+// is cut into as many ranges as give every CU a workgroup (at most kMaxSplitGroups of them, which is what the
+// fixed scratch of the entry point that allocates nothing holds), each range a multiple of kBufs steps; the
+// workgroups leave raw sums in the workspace and a second kernel adds them in split order (deterministic).
+namespace {
+struct GemmPlan {
+  int Gpad, nsplit, spp;
+  size_t ap_halves, partial_floats;
+};
+GemmPlan gemm_plan(int cus, int K, int N) {
+  GemmPlan p;
+  const int G = K / 32;
+  p.Gpad = (G + kChunk - 1) / kChunk * kChunk;
+  p.ap_halves = (size_t)p.Gpad * 4 * 64 * 8;
+  const int ntiles = (N + kTileN - 1) / kTileN;
+  const int nsteps = p.Gpad / kStepGroups;
+  p.nsplit = (cus < kMaxSplitGroups ? cus : kMaxSplitGroups) / ntiles;
+  if (p.nsplit > nsteps / kBufs) p.nsplit = nsteps / kBufs;
+  if (p.nsplit < 1) p.nsplit = 1;
+  p.spp = (nsteps + p.nsplit - 1) / p.nsplit;
+  p.spp = (p.spp + kBufs - 1) / kBufs * kBufs;
+  p.nsplit = (nsteps + p.spp - 1) / p.spp;
+  p.partial_floats = p.nsplit > 1 ? (size_t)ntiles * p.nsplit * 64 * kTileN : 0;
+  return p;
+}
+}  // namespace
+
+int hq_q3_gemm_need(int cus, int K, int N, size_t* floats, size_t* counters) {
+  const GemmPlan p = gemm_plan(cus, K, N);
+  *floats = p.ap_halves / 2 + 128 + p.partial_floats;
+  *counters = 1;
+  return HQ_OK;
+}
+
 int hq_q3_gemm_launch(const void* x, const int32_t* qweight, const float* scales, const float* zeros, float* y,
                       int K, int N, int M, unsigned flags, hipStream_t stream, const HqQ3Scratch* fixed) {
   if (((uintptr_t)x & 15) || (K & 7)) return HQ_ERR_MISALIGNED;
   if (((uintptr_t)scales & 15) || ((uintptr_t)zeros & 15) || ((uintptr_t)y & 15)) return HQ_ERR_MISALIGNED;
-  const int G = K / 32;
-  const int Gpad = (G + kChunk - 1) / kChunk * kChunk;
-  const size_t ap_halves = (size_t)Gpad * 4 * 64 * 8;
-  // K split: column tiles alone leave most CUs idle when N is small (N = 4096: 32 tiles), so K is cut into as
-  // many ranges as give every CU a workgroup (at most kMaxSplitGroups of them, which is what the fixed
-  // scratch of the entry point that allocates nothing holds), each range a multiple of kBufs steps; the
-  // workgroups leave raw sums in the workspace and a second kernel adds them in split order (deterministic).
   const HqDevice* dev = nullptr;
   int rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
-  const int ntiles = (N + kTileN - 1) / kTileN;
-  const int nsteps = Gpad / kStepGroups;
-  int nsplit = (dev->cus < kMaxSplitGroups ? dev->cus : kMaxSplitGroups) / ntiles;
-  if (nsplit > nsteps / kBufs) nsplit = nsteps / kBufs;
-  if (nsplit < 1) nsplit = 1;
-  int spp = (nsteps + nsplit - 1) / nsplit;
-  spp = (spp + kBufs - 1) / kBufs * kBufs;
-  nsplit = (nsteps + spp - 1) / spp;
-  const size_t partial_floats = nsplit > 1 ? (size_t)ntiles * nsplit * 64 * kTileN : 0;
+  const GemmPlan plan = gemm_plan(dev->cus, K, N);
+  const int Gpad = plan.Gpad, nsplit = plan.nsplit, spp = plan.spp;
+  const size_t ap_halves = plan.ap_halves, partial_floats = plan.partial_floats;
   _Float16* Ap;
   float *rowsum, *rowinv, *partial = nullptr;
   if (fixed) {

@@ -76,6 +76,16 @@ int hq_init(void);
  * (needed before stream capture).  No counterpart in the reference. */
 int hq_reserve_workspace(void* stream, int max_K, int max_N);
 
+/* Host-only size queries behind hq_reserve_workspace (plain arithmetic: no device is touched, so they also
+ * answer for a device that is not present).  hq_q3_workspace_need: floats and arrival counters one
+ * hq_q3_matvec(K, N, batch_M) call takes from its stream's workspace on a device of compute_units compute
+ * units, computed by the very plan functions of the launch.  hq_reserve_need: what
+ * hq_reserve_workspace(stream, max_K, max_N) makes sure of - at least the need of every call with K <= max_K
+ * and N <= max_N, whatever the batch.  Counterpart of the compute-unit query that sizes the launch in
+ * src/quantAQLM-hip/main.cu:108-121. */
+int hq_q3_workspace_need(int compute_units, int K, int N, int batch_M, int64_t* floats, int64_t* counters);
+int hq_reserve_need(int compute_units, int max_K, int max_N, int64_t* floats, int64_t* counters);
+
 /* Waits for the current device, then frees every workspace the library holds on any device.
  * Optional; the library can be used again afterwards (workspaces are re-created on demand). */
 int hq_shutdown(void);
@@ -122,7 +132,9 @@ int hq_quantize_dynamic8(const float* code, const float* A, uint8_t* out, int64_
  * the pre-multiplied scale*zero_point.
  *   x        : [batch_M][K] row-major, fp32 (HQ_DTYPE_F32) or fp16 (HQ_DTYPE_F16)
  *   y        : fp32 [batch_M][N]
- *   K % 32 == 0, N % 4 == 0, batch_M >= 1; qweight and x 16-byte aligned.
+ *   K % 32 == 0, N % 4 == 0, batch_M >= 1; qweight and x 16-byte aligned; for batch_M > 1 scales, zeros
+ *   and y 16-byte aligned as well (whichever kernel the plan picks, so that a pointer that works at one
+ *   batch size or on one device works at every other), for batch_M == 1 4-byte aligned.
  * Products are accumulated in fp32 for both dtypes (the reference's fp16
  * variant accumulates 16 terms in fp16).
  * batch_M == 1 replaces vecquant3matmul / vecquant3matmul_faster
@@ -282,6 +294,21 @@ int hq_gemv_int4(const uint8_t* mat_packed, const void* vec_fp16, void* res_fp16
  * (kernel main.cu:109-142), without its timing loop and printing.
  */
 int hq_mxfp4_qdq(const void* in, void* out, int64_t n_elems, int dtype, void* stream);
+
+/*
+ * Memory-system probes for the benchmark report (no counterpart in the reference): the rate this device
+ * delivers to the simplest kernels, measured next to the library kernels instead of quoted from a data sheet.
+ *   hq_probe_stream(mode, src, dst, bytes, stream): mode 0 reads `bytes` bytes of src and writes nothing
+ *     (dst must still be a valid 16-byte buffer), mode 1 copies them to dst.  bytes a multiple of 16.
+ *   hq_probe_gather16(table, table_bytes, gathers, sink16, stream): at least `gathers` independent 16-byte
+ *     reads at pseudo-random entries of a table of table_bytes bytes (a power of two) - the access pattern
+ *     of a code-book lookup, bounded by cache requests per second; sink16 is a 16-byte buffer that is
+ *     never written in practice.  hq_probe_gather16_count(gathers) returns the exact number of reads that
+ *     call performs on the current device (the request rounded up to whole trips of every lane).
+ */
+int hq_probe_stream(int mode, const void* src, void* dst, int64_t bytes, void* stream);
+int hq_probe_gather16(const void* table, int64_t table_bytes, int64_t gathers, void* sink16, void* stream);
+int64_t hq_probe_gather16_count(int64_t gathers);
 
 #ifdef __cplusplus
 }

@@ -33,6 +33,12 @@ static double round_to_f16_grid(double d) {
   return d < 0 ? -r : r;
 }
 
+/* Threads the loops over independent outputs use (1 = serial, the default): the timed CPU baseline
+ * runs them serially and again over the host cores; results do not depend on it. */
+static int g_threads = 1;
+void hqo_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
+int hqo_max_threads(void) { return omp_get_max_threads(); }
+
 uint16_t hqo_f64_to_f16(double d) {
   if (d != d) return 0x7e00;
   double r = round_to_f16_grid(d);
@@ -232,8 +238,9 @@ void hqo_q3_gemm(const uint16_t* A, const int32_t* mat, double* out,
   int G = K / 32;
   double* Ad = (double*)malloc(sizeof(double) * (size_t)M * K);
   for (size_t i = 0; i < (size_t)M * K; ++i) Ad[i] = hqo_f16_to_f32(A[i]);
-  double* wcol = (double*)malloc(sizeof(double) * (size_t)K);
+#pragma omp parallel for schedule(static) num_threads(g_threads)
   for (int n = 0; n < N; ++n) {
+    double* wcol = (double*)malloc(sizeof(double) * (size_t)K);
     for (int g = 0; g < G; ++g) {
       uint32_t w[3];
       for (int j = 0; j < 3; ++j) w[j] = (uint32_t)mat[(size_t)(3 * g + j) * N + n];
@@ -249,8 +256,8 @@ void hqo_q3_gemm(const uint16_t* A, const int32_t* mat, double* out,
       for (int k = 0; k < K; ++k) acc += a[k] * wcol[k];
       out[(size_t)m * N + n] = acc;
     }
+    free(wcol);
   }
-  free(wcol);
   free(Ad);
 }
 
@@ -274,6 +281,7 @@ const float hqo_fp4_table[16] = {
 void hqo_dequant_4bit(const uint8_t* packed, const float* absmax, uint16_t* out,
                       int64_t n, int blocksize, int table) {
   const float* T = table ? hqo_fp4_table : hqo_nf4_table;
+#pragma omp parallel for schedule(static) num_threads(g_threads)
   for (int64_t e = 0; e < n; ++e) {
     uint8_t b = packed[e >> 1];
     unsigned c = (e & 1) ? (b & 15u) : (b >> 4); /* high nibble first */
@@ -486,6 +494,7 @@ void hqo_lut_gemv_f64(const uint32_t* bW, const uint16_t* alpha, const uint16_t*
       for (int kw = g * group / 32; kw < (g + 1) * group / 32; ++kw) {
         const uint32_t* row = bW + ((size_t)kw * nb + b) * N;
         const uint16_t* al = alpha + ((size_t)g * nb + b) * N;
+#pragma omp parallel for schedule(static) num_threads(g_threads)
         for (int n = 0; n < N; ++n) {
           uint32_t w = row[n];
           double s = 0.0;
@@ -545,6 +554,7 @@ void hqo_aqlm_matvec(const int16_t* codes, const uint16_t* codebooks,
                      double* y64, int M, int K, const int cb_a_sizes[4],
                      int cb_stride_int4, int mode) {
   int ncodes = K / 8;
+#pragma omp parallel for schedule(static) num_threads(g_threads)
   for (int m = 0; m < M; ++m) {
     const uint16_t* cb = codebooks;
     for (int j = 0; j < 4 && m >= cb_a_sizes[j]; ++j)

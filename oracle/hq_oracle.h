@@ -61,6 +61,12 @@ uint16_t hqo_hmul(uint16_t a, uint16_t b);
 void hqo_q3_pack(const uint8_t* codes, int K, int N, int32_t* mat);
 void hqo_q3_unpack(const int32_t* mat, int K, int N, uint8_t* codes);
 
+/* Threads for the loops over independent outputs of hqo_dequant_4bit, hqo_lut_gemv_f64,
+ * hqo_aqlm_matvec and hqo_q3_gemm (1 = serial, the default; results do not depend on it): the
+ * benchmark times the restatements serially and again over the host cores. */
+void hqo_set_threads(int n);
+int hqo_max_threads(void);
+
 /* fp32 kernel, src/quant3MatMul-hip/kernels.h:12-90: per 256-row block
  * res += (scale*float(q) - zero) * x  sequentially in fp32 (no FMA
  * contraction), block partials added to mul[] in block order.  mul is

@@ -34,6 +34,13 @@ class Oracle:
         self.nf4_table = np.ctypeslib.as_array((ctypes.c_float * 16).in_dll(lib, "hqo_nf4_table")).copy()
         self.fp4_table = np.ctypeslib.as_array((ctypes.c_float * 16).in_dll(lib, "hqo_fp4_table")).copy()
 
+    def set_threads(self, n):
+        """Threads for the loops over independent outputs (1 = serial); results do not depend on it."""
+        self.lib.hqo_set_threads(int(n))
+
+    def max_threads(self):
+        return int(self.lib.hqo_max_threads())
+
     # ---- q3
     def q3_pack(self, codes):
         K, N = codes.shape

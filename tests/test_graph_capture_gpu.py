@@ -73,3 +73,48 @@ def test_replays_match_eager(hq, oracle):
         assert torch.equal(y24, want_24), rep
         assert torch.equal(y_na, want_na), rep
         assert torch.equal(other, want), rep
+
+
+def test_capture_after_reserve_only(hq):
+    """A fresh stream sees nothing but hq_reserve_workspace before the capture: every recorded call with a
+    smaller K or N - among them a batched GEMM whose few column tiles split K, the largest workspace user -
+    must find its workspace there (an allocation during capture would fail the call)."""
+    import torch
+    from hecbench_amd import _lib
+    lib = _lib.load()
+    dev = "cuda:0"
+    g = torch.Generator(device=dev)
+    g.manual_seed(77)
+    maxK, maxN = 8192, 8256
+    shapes = [(1, 8192, 8256), (72, 8192, 4096), (4, 8192, 8256), (24, 1024, 516), (1, 4096, 1024), (16, 4096, 4096)]
+    probs = []
+    for M, K, N in shapes:
+        mat = torch.randint(-2 ** 31, 2 ** 31 - 1, (3 * K // 32, N), dtype=torch.int32, device=dev, generator=g)
+        s = torch.empty(N, device=dev).uniform_(0.005, 0.02, generator=g)
+        z = s * torch.randint(3, 5, (N,), device=dev, generator=g).float()
+        x = torch.randn(M, K, device=dev, generator=g)
+        x = x[0].contiguous() if M == 1 else x.half()
+        probs.append((M, x, mat, s, z))
+
+    def run(p, out):
+        M, x, mat, s, z = p
+        return hq.q3_matvec(x, mat, s, z, out=out) if M == 1 else hq.q3_gemm(x, mat, s, z, out=out)
+
+    # eager results on the default stream (this also sets the kernels' one-time function attributes)
+    want = [run(p, None).clone() for p in probs]
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    outs = [torch.zeros_like(w) for w in want]
+    assert lib.hq_reserve_workspace(ctypes.c_void_p(stream.cuda_stream), maxK, maxN) == 0
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        for p, o in zip(probs, outs):
+            run(p, o)
+    for rep in range(3):
+        for o in outs:
+            o.fill_(float(rep))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for (M, *_), o, w in zip(probs, outs, want):
+            assert torch.equal(o, w), (rep, M, tuple(o.shape))
