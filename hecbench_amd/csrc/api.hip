@@ -25,7 +25,7 @@ std::vector<std::pair<int, void*>> g_retired;  // outgrown buffers, freed by hq_
 namespace {
 const char* const kTunableNames[HQ_TUNE_COUNT] = {
     "HQ_Q3_WAVES", "HQ_Q3_STEPS", "HQ_Q3_KSPLIT", "HQ_Q3_TILE", "HQ_Q3_SMALL_BATCH", "HQ_Q3_ROW_BLOCKS", "HQ_LUT_PATH", "HQ_LUT_KSPLIT", "HQ_NF4_PIPE",
-    "HQ_AQLM_ROWS", "HQ_Q8_WGS", "HQ_Q8_FAST", "HQ_GEMV_LDS", "HQ_SPLITK_FENCES"};
+    "HQ_AQLM_ROWS", "HQ_Q8_WGS", "HQ_Q8_FAST", "HQ_GEMV_LDS", "HQ_GEMV_SPLIT", "HQ_SPLITK_FENCES"};
 constexpr int kUnset = INT_MIN;
 std::atomic<int> g_tunables[HQ_TUNE_COUNT];
 std::once_flag g_tunables_once;

@@ -183,6 +183,71 @@ __global__ __launch_bounds__(256) void gemv_kernel(const char* mat_, const u4v* 
   gemv_finish<MODE, R>(a, row0, acc, acc16, MODE == kF16 ? 0.f : wave_sum(vsum));
 }
 
+// Rows cut across the waves of a workgroup.  On this part a stream moves fastest when every wave issues a
+// few loads and ends - the wave launcher refills the compute units better than any loop (a plain read of 537 MB
+// runs at 7.0 TB/s with one 128-bit load per thread and at 5.6 TB/s as a grid-stride loop) - so for long rows a
+// workgroup of SPLIT waves shares R rows, every wave takes every SPLIT-th two-step piece of the columns,
+// and the waves' sums meet in LDS in wave order (deterministic).
+template <int MODE, int R, int SPLIT>
+__global__ __launch_bounds__(SPLIT * 64) void gemv_split_kernel(const char* mat_, const u4v* vec_, _Float16* res_, int rows_,
+                                                                int n_, float scale_, float zp_) {
+  GemvArgs a;
+  a.mat = mat_; a.vec = vec_; a.res = res_; a.rows = rows_; a.n = n_; a.scale = scale_; a.zp = zp_;
+  using G = Geom<MODE>;
+  __shared__ float part[SPLIT][R + 1];
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int row0 = blockIdx.x * R;
+  const int units = a.n / G::kPerUnit;  // 16-byte units per matrix row
+  const size_t row_bytes = (size_t)units * 16;
+  const u4v* rowp[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    rowp[r] = reinterpret_cast<const u4v*>(a.mat + (size_t)min(row0 + r, a.rows - 1) * row_bytes);
+  float acc[R], acc16[R], vsum = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = acc16[r] = 0.f;
+  // pieces of two steps (2 KB per row) dealt to the waves in turn: neighbouring waves start 2 KB apart
+  // whatever the row length (waves 4 KB apart measured 97 against 76 us at 16384 x 16384)
+  for (int u0 = wv * 128; u0 < units; u0 += SPLIT * 128) {
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const int u = u0 + st * 64 + lane;
+      if (u < units) {
+        u4v m[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) m[r] = __builtin_nontemporal_load(rowp[r] + u);
+        u4v v[G::kVecUnits];
+#pragma unroll
+        for (int i = 0; i < G::kVecUnits; ++i) v[i] = a.vec[(size_t)u * G::kVecUnits + i];
+        gemv_step<MODE, R, true>(m, v, acc, acc16, vsum);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const float s = wave_sum(MODE == kI4 ? fmaf(acc16[r], 0.0625f, acc[r]) : acc[r]);
+    if (lane == 0) part[wv][r] = s;
+  }
+  if (MODE != kF16) {
+    const float vs = wave_sum(vsum);
+    if (lane == 0) part[wv][R] = vs;
+  }
+  __syncthreads();
+  if (threadIdx.x < R && row0 + (int)threadIdx.x < a.rows) {
+    const int r = threadIdx.x;
+    float s = 0.f, vs = 0.f;
+#pragma unroll
+    for (int w = 0; w < SPLIT; ++w) {
+      s += part[w][r];
+      if (MODE != kF16) vs += part[w][R];
+    }
+    if (MODE == kI8) s = a.scale * (s - a.zp * vs);
+    if (MODE == kI4) s = a.scale * (s * 16777216.f - a.zp * vs);  // codes were fp16 subnormals code * 2^-24
+    a.res[row0 + r] = (_Float16)s;
+  }
+}
+
 // The vector in LDS, the workgroups persistent.  A CU returns its loads in issue order and holds about
 // 64 KB of them, whichever cache serves them: every piece of the vector a wave loads next to its matrix
 // rows (as many bytes as the rows themselves for int8 with two rows per wave and int4 with four) takes a
@@ -286,6 +351,25 @@ int launch_gemv(const void* mat, const void* vec, void* res, int rows, int n, fl
   // 16384 x 28672 41.7 -> 38.8, 16384 x 16384 25.8 -> 25.5); fp16 and int8 gain on some shapes and lose on
   // others (fp16 16384 x 16384 88.7 -> 83.0 us but 28672 x 8192 70.6 -> 79.0), fewer rows lose throughout.
   // HQ_GEMV_LDS: 0 never, 1 wherever the vector fits, unset: the rule above.
+  // Rows cut across the waves of a workgroup: fp16 rows of 8192 elements or more, two steps of two rows per
+  // wave (16384 x 16384: 88.7 -> 75.7 us = 7.1 TB/s; 28672 x 8192 70.5 -> 64.3; 8192 x 28672 73.8 -> 66.8;
+  // 4096 x 16384 23.0 -> 21.0).  Other step counts per wave are worse, some much (four steps, i.e. waves that
+  // start 4 KB apart: 97.5 us at 16384 x 16384), and int8 / int4 rows gain little or lose: they keep whole
+  // rows per wave.  HQ_GEMV_SPLIT: 0 never, 4 / 8 / 16 that many waves per pair of rows, unset: this rule.
+  {
+    int split = hq_tune(HQ_TUNE_GEMV_SPLIT, -1);
+    const int units = n / Geom<MODE>::kPerUnit;
+    if (split < 0)  // (a forced choice between the two whole-row kernels below stands)
+      split = (MODE == kF16 && units >= 1024 && hq_tune(HQ_TUNE_GEMV_LDS, -1) < 0) ? (units >= 2048 ? 16 : 8) : 0;
+    const int groups = (rows + 1) / 2;
+#define HQ_GEMV_SPLIT_CASE(S) \
+    if (split == S) { \
+      hipLaunchKernelGGL((gemv_split_kernel<MODE, 2, S>), dim3(groups), dim3(S * 64), 0, stream, a.mat, a.vec, a.res, a.rows, a.n, a.scale, a.zp); \
+      return hq_launch_status(); \
+    }
+    HQ_GEMV_SPLIT_CASE(4) HQ_GEMV_SPLIT_CASE(8) HQ_GEMV_SPLIT_CASE(16)
+#undef HQ_GEMV_SPLIT_CASE
+  }
   const int lds = hq_tune(HQ_TUNE_GEMV_LDS, -1);
   const int full = dev->cus * 16;  // waves of a full launch of the LDS kernel
   if ((size_t)n * 2 <= kMaxVectorLds && (lds == 1 || (lds < 0 && MODE == kI4 && rows >= full * 4))) {

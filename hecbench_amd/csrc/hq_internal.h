@@ -65,7 +65,7 @@ int hq_noalloc_setup(void);
 // one relaxed atomic load.
 enum HqTunable {
   HQ_TUNE_Q3_WAVES, HQ_TUNE_Q3_STEPS, HQ_TUNE_Q3_KSPLIT, HQ_TUNE_Q3_TILE, HQ_TUNE_Q3_SMALL_BATCH, HQ_TUNE_Q3_ROW_BLOCKS, HQ_TUNE_LUT_PATH, HQ_TUNE_LUT_KSPLIT,
-  HQ_TUNE_NF4_PIPE, HQ_TUNE_AQLM_ROWS, HQ_TUNE_Q8_WGS, HQ_TUNE_Q8_FAST, HQ_TUNE_GEMV_LDS, HQ_TUNE_SPLITK_FENCES, HQ_TUNE_COUNT
+  HQ_TUNE_NF4_PIPE, HQ_TUNE_AQLM_ROWS, HQ_TUNE_Q8_WGS, HQ_TUNE_Q8_FAST, HQ_TUNE_GEMV_LDS, HQ_TUNE_GEMV_SPLIT, HQ_TUNE_SPLITK_FENCES, HQ_TUNE_COUNT
 };
 int hq_tune(HqTunable id, int dflt);
 

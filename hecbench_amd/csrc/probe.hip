@@ -10,30 +10,19 @@
 namespace {
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 
-// units = 16-byte pieces; every thread keeps four loads in flight and walks the range grid-stride
+// units = 16-byte pieces, ONE per thread: on this part the plain grid - a workgroup's worth of loads per
+// workgroup, 131072 workgroups for 512 MiB - streams faster than any grid-stride loop (512 MiB read: 6.98 TB/s
+// against 5.6 TB/s with sixteen workgroups per compute unit and four loads in flight per thread, 6.76 TB/s with
+// one trip of four loads per thread; copy 6.5 against 4.7 TB/s): the wave launcher is the better load scheduler.
 template <bool COPY>
 __global__ __launch_bounds__(256) void probe_stream_kernel(const u4v* __restrict__ src, u4v* __restrict__ dst,
                                                           long units, u4v* __restrict__ sink) {
-  const long stride = (long)gridDim.x * 256;
-  long i = (long)blockIdx.x * 256 + threadIdx.x;
-  u4v acc = {0u, 0u, 0u, 0u};
-  for (; i + 3 * stride < units; i += 4 * stride) {
-    u4v v[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(src + i + u * stride);
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      if (COPY) __builtin_nontemporal_store(v[u], dst + i + u * stride);
-      else acc ^= v[u];
-    }
-  }
-  for (; i < units; i += stride) {
-    const u4v v = __builtin_nontemporal_load(src + i);
-    if (COPY) __builtin_nontemporal_store(v, dst + i);
-    else acc ^= v;
-  }
-  // keeps the loads alive; the condition is false for any realistic data
-  if (!COPY && (acc.x & acc.y & acc.z & acc.w) == 0xffffffffu && acc.x + acc.y == 12345u) *sink = acc;
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= units) return;
+  const u4v v = __builtin_nontemporal_load(src + i);
+  if (COPY) __builtin_nontemporal_store(v, dst + i);
+  // keeps the load alive; the condition is false for any realistic data
+  else if ((v.x & v.y & v.z & v.w) == 0xffffffffu && v.x + v.y == 12345u) *sink = v;
 }
 
 // every lane performs `per_lane` independent 16-byte reads, eight in flight at a time
@@ -64,9 +53,8 @@ extern "C" int hq_probe_stream(int mode, const void* src, void* dst, int64_t byt
   const int rc = hq_current_device(&dev);
   if (rc != HQ_OK) return rc;
   const long units = bytes / 16;
-  long wgs = (units + 1023) / 1024;  // at most one trip of four loads per thread ...
-  const long cap = (long)dev->cus * 16;  // ... but no more than sixteen workgroups per compute unit
-  if (wgs > cap) wgs = cap;
+  const long wgs = (units + 255) / 256;
+  if (wgs > 0x7fffffffL) return HQ_ERR_TOO_LARGE;
   if (mode == 1)
     hipLaunchKernelGGL(probe_stream_kernel<true>, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream,
                        (const u4v*)src, (u4v*)dst, units, (u4v*)dst);

@@ -92,7 +92,7 @@ int hq_shutdown(void);
 
 /* Launch-shape override for tests and sweeps, not part of the stable interface: name is one of
  * HQ_Q3_WAVES, HQ_Q3_STEPS, HQ_Q3_KSPLIT, HQ_Q3_TILE, HQ_Q3_SMALL_BATCH, HQ_Q3_ROW_BLOCKS, HQ_LUT_PATH, HQ_LUT_KSPLIT, HQ_NF4_PIPE,
- * HQ_AQLM_ROWS, HQ_Q8_WGS, HQ_Q8_FAST, HQ_GEMV_LDS, HQ_SPLITK_FENCES (an environment variable of the same name seeds
+ * HQ_AQLM_ROWS, HQ_Q8_WGS, HQ_Q8_FAST, HQ_GEMV_LDS, HQ_GEMV_SPLIT, HQ_SPLITK_FENCES (an environment variable of the same name seeds
  * the knob once per process); clear != 0 returns the knob to the library's own choice.  Results
  * never depend on a knob beyond the documented tolerances. */
 int hq_set_tunable(const char* name, int value, int clear);

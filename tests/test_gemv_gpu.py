@@ -64,6 +64,29 @@ def test_vector_in_lds_kernel(hq, oracle, tunable, rows, n, mode):
     assert np.array_equal(lds.view(np.uint16), plain.view(np.uint16))
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("split", [4, 8, 16])
+@pytest.mark.parametrize("rows,n", [(37, 1024), (1, 32), (513, 8192), (16, 16384), (131, 11008), (7, 65536 + 64)])
+def test_rows_cut_across_waves(hq, oracle, tunable, rows, n, mode, split):
+    """The kernel whose workgroups share a pair of rows, every wave a piece of the columns: forced with 4, 8
+    and 16 waves on odd row counts, rows shorter than one step per wave (idle waves) and rows that do not
+    divide into whole steps."""
+    mat, vec = gemv_problem(rows * 7 + n + mode + split, rows, n, mode)
+    _, r64 = oracle.gemv(mat, mode, vec, SCALE, ZP)
+    tunable("HQ_GEMV_SPLIT", split)
+    got, _, _ = _run(hq, mat, vec, mode)
+    _check(got, r64)
+
+
+@pytest.mark.parametrize("rows,n", [(130, 8192), (33, 16384), (66, 28672), (5, 32768)])
+def test_long_fp16_rows_default_rule(hq, oracle, rows, n):
+    """fp16 rows of 8192 elements or more take the split kernel by default."""
+    mat, vec = gemv_problem(rows + n, rows, n, 0)
+    _, r64 = oracle.gemv(mat, 0, vec, SCALE, ZP)
+    got, _, _ = _run(hq, mat, vec, 0)
+    _check(got, r64)
+
+
 def test_vector_too_long_for_lds(hq, oracle, tunable):
     """Beyond 65536 elements the vector does not fit: the ordinary kernel runs even when the other is asked for."""
     mat, vec = gemv_problem(5, 24, 65536 + 32, 2)
