@@ -296,7 +296,7 @@ __device__ __forceinline__ f4 mfma_fp8_fp4(v8i a, v8i b, f4 c) {
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 4, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
 }
 
-constexpr int kDigQuad = 4 * 4 * 32 + 32;  // digits of one quad [k-word][digit][32 operand bytes], then 32 zero bytes
+constexpr int kDigQuad = 4 * 4 * 32 + 16;  // digits of one quad [k-word][digit][32 operand bytes], then 16 zero bytes
 constexpr int planes_of_set(int nb, int s) { return nb - 3 * s < 3 ? nb - 3 * s : 3; }
 
 template <int NB, int QUADS, int WAVES, bool BIAS, bool RAGGED, bool ONE_ROUND>
@@ -415,9 +415,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(
       for (int h = 0; h < 2; ++h) {
         const int jj = 4 * m + 2 * h + (kb >> 1);
         const int b = jj % P, kw = jj / P;
-        // rows of other planes read zeros; of the two zero pieces the one whose LDS banks the quarter's
-        // digit rows (all at half_off) do not use
-        doff[s][m][h] = (m < P && (c >> 2) == b) ? (kw * 4 + (c & 3)) * 32 + half_off : 512 + (16 - half_off);
+        doff[s][m][h] = (m < P && (c >> 2) == b) ? (kw * 4 + (c & 3)) * 32 + half_off : 512;
       }
   }
   // plain operand (every row r holds digit r & 3 of all four k-words): one MFMA with all-ones weights
@@ -426,7 +424,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(
   v8i ones;
 #pragma unroll
   for (int r = 0; r < 8; ++r) ones[r] = r < 4 ? 0x11111111 : 0;
-  if (lane < 8 * QUADS) *reinterpret_cast<uint32_t*>(xs_w + (lane >> 3) * kDigQuad + 512 + (lane & 7) * 4) = 0u;
+  if (lane < 4 * QUADS) *reinterpret_cast<uint32_t*>(xs_w + (lane >> 2) * kDigQuad + 512 + (lane & 3) * 4) = 0u;
 
   constexpr int STRIDE = WAVES * QUADS;
   auto compute_round = [&](int q0, Round& r, Round& next) {
