@@ -520,34 +520,40 @@ def cpu_configs():
     threads = max(1, min(o.max_threads(), os.cpu_count() or 1))
 
     def timed(fn, reps):
-        t0 = time.perf_counter()
+        """(median, best) seconds of `reps` single calls"""
+        t = []
         for _ in range(reps):
+            t0 = time.perf_counter()
             fn()
-        return (time.perf_counter() - t0) / reps
+            t.append(time.perf_counter() - t0)
+        t.sort()
+        return t[len(t) // 2], t[0]
 
     jobs = {}
     packed, absmax = oa.make_nf4_problem(0, 4096 * 4096, 64)
-    jobs["0_nf4_dequant_4096x4096"] = (lambda: o.dequant_4bit(packed, absmax, 4096 * 4096, 64), 2, 1, "2 full calls")
+    jobs["0_nf4_dequant_4096x4096"] = (lambda: o.dequant_4bit(packed, absmax, 4096 * 4096, 64), 3, 1, "3 full calls")
     bW, alpha, qb, x = oa.make_lut_problem(0, 4096, 2048, 3, 128)
-    jobs["2_lut_gemv_4096x16384_q3"] = (lambda: o.lut_gemv_f64(bW, alpha, qb, x, 128), 2, 8,
-                                        "2048 of 16384 columns, scaled x8")
+    jobs["2_lut_gemv_4096x16384_q3"] = (lambda: o.lut_gemv_f64(bW, alpha, qb, x, 128), 3, 8,
+                                        "3 calls on 2048 of 16384 columns, scaled x8")
     codes, cb, sc, xa = oa.make_aqlm_problem(0, 4096, 4096)
-    jobs["3_aqlm_4096x4096"] = (lambda: o.aqlm_matvec(codes, cb, sc, xa, (4096, 0, 0, 0), 65536), 2, 1, "2 full calls")
+    jobs["3_aqlm_4096x4096"] = (lambda: o.aqlm_matvec(codes, cb, sc, xa, (4096, 0, 0, 0), 65536), 3, 1, "3 full calls")
     qc, scales, zeros, A = oa.make_q3_problem(0, 8192, 1024, np.float16, batch=4)
     mat = o.q3_pack(qc)
-    jobs["4_q3_gemm_64x8192x28672"] = (lambda: o.q3_gemm(A, mat, scales, zeros), 2, 16 * 28,
-                                       "4 of 64 rows x 1024 of 28672 columns, scaled x448")
+    jobs["4_q3_gemm_64x8192x28672"] = (lambda: o.q3_gemm(A, mat, scales, zeros), 3, 16 * 28,
+                                       "3 calls on 4 of 64 rows x 1024 of 28672 columns, scaled x448")
     out = {}
     for name, (fn, reps, scale, sample) in jobs.items():
         o.set_threads(1)
-        serial = timed(fn, reps) * scale
+        s_med, s_best = timed(fn, reps)
         o.set_threads(threads)
         try:
-            par = timed(fn, reps) * scale
+            p_med, p_best = timed(fn, reps)
         finally:
             o.set_threads(1)
-        out[name] = {"cpu_serial": {"us": round(serial * 1e6, 1), "cores": 1, "kind": "port", "sample": sample},
-                     "cpu_openmp": {"us": round(par * 1e6, 1), "cores": threads, "kind": "port", "sample": sample}}
+        out[name] = {"cpu_serial": {"us": round(s_med * scale * 1e6, 1), "us_best": round(s_best * scale * 1e6, 1), "cores": 1,
+                                    "kind": "port", "sample": sample + " (median; best beside it)"},
+                     "cpu_openmp": {"us": round(p_med * scale * 1e6, 1), "us_best": round(p_best * scale * 1e6, 1),
+                                    "cores": threads, "kind": "port", "sample": sample + " (median; best beside it)"}}
     return out
 
 
