@@ -124,13 +124,11 @@ static void reserve_bound(int cus, int max_K, int max_N, size_t* floats, size_t*
   const size_t kpad = ((size_t)max_K + 1023) / 1024 * 1024;
   const size_t gemm_floats = kpad * 32 + 128 + (kpad >= 2048 ? (size_t)256 * 64 * 128 : 0);
   // split-K matvecs: a partial row of 64 floats per column tile and split - one split per 4096 elements of K
-  // up to eight whatever the tile count (a shorter K than max_K may split where max_K itself does not), beyond
-  // that only as many as give every compute unit a workgroup; narrow tiles (16 or 32 columns) only while
-  // tiles x splits stay within the compute units.  The LUT kernels: two workgroups per compute unit, 128
-  // floats each.
+  // (a shorter K than max_K splits no further); narrow tiles (16 or 32 columns) only while tiles x splits stay
+  // within the compute units.  The LUT kernels: two workgroups per compute unit, 128 floats each.
   const size_t tiles = ((size_t)max_N + 63) / 64;
   const size_t rounds = ((size_t)max_K + 4095) / 4096;
-  const size_t full_split = tiles * (rounds <= 8 ? rounds : 8);
+  const size_t full_split = tiles * rounds;
   const size_t per_cu = tiles + 2 * (size_t)cus;
   size_t split_floats = (full_split > per_cu ? full_split : per_cu) * 64 * 2;
   // batches 2 ... 64 on the matvec-like kernel: one partial row per tile, range of K and activation row, at most

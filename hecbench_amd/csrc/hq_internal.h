@@ -69,6 +69,25 @@ enum HqTunable {
 };
 int hq_tune(HqTunable id, int dflt);
 
+// Sum of the nsplit partial sums p[s * stride] of a K split, added in split order (the result does not depend
+// on which workgroup arrived last).  The loads are device-scope atomic loads, which bypass the non-coherent
+// cache levels; eight of them are in flight at a time - one after the other each costs a trip to memory, and
+// the last workgroup of a tile is the last thing a kernel does.
+__device__ __forceinline__ float hq_sum_partials(const float* p, size_t stride, int nsplit) {
+  float sum = 0.f;
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int s = s0 + j < nsplit ? s0 + j : nsplit - 1;
+      v[j] = __hip_atomic_load(p + (size_t)s * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sum += s0 + j < nsplit ? v[j] : 0.f;
+  }
+  return sum;
+}
+
 // Streaming stores: write-through (sc1) and nontemporal (nt), i.e. the data is on its way to memory at once
 // and is not kept in the L2.  For a 33.5 MB write stream on MI355X: 5.80 us against 6.46 us with nt alone
 // and 7.04 us with plain stores.  The compiler cannot see that the assembly is a store, so the wait states it

@@ -178,10 +178,7 @@ __global__ __launch_bounds__(256) void lut_gemv_kernel(LutArgs a) {
     if (*s_last && a.strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     if (*s_last) {
       if (tid < 64 * CPL && n < a.N) {
-        float sum = 0.f;
-        for (int s = 0; s < a.nsplit; ++s)
-          sum += __hip_atomic_load(&a.partial[((size_t)tile * a.nsplit + s) * (64 * CPL) + tid],
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const float sum = hq_sum_partials(&a.partial[(size_t)tile * a.nsplit * (64 * CPL) + tid], 64 * CPL, a.nsplit);
         a.y[n] = (_Float16)sum;
       }
       if (tid == 0) __hip_atomic_store(&a.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -575,10 +572,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(
     if (last && a.strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     if (last) {
       if (tid < 64 && n < a.N) {
-        float sum = 0.f;
-        for (int s = 0; s < a.nsplit; ++s)
-          sum += __hip_atomic_load(&a.partial[((size_t)tile * a.nsplit + s) * 64 + tid], __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
+        const float sum = hq_sum_partials(&a.partial[(size_t)tile * a.nsplit * 64 + tid], 64, a.nsplit);
         a.y[n] = (_Float16)(sum * 2048.f);
       }
       if (tid == 0)  // ready for the next call

@@ -438,10 +438,7 @@ __global__ __launch_bounds__(WAVES * 64) void q3_matvec_kernel(const uint32_t* w
     if (s_last && strict) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     if (s_last) {
       if (tid < TW && n < a.N) {
-        float sum = 0.f;
-        for (int s = 0; s < a.nsplit; ++s)
-          sum += __hip_atomic_load(&a.partial[((size_t)tile * a.nsplit + s) * 64 + tid],
-                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const float sum = hq_sum_partials(&a.partial[(size_t)tile * a.nsplit * 64 + tid], 64, a.nsplit);
         a.y[n] = (a.flags & HQ_FLAG_ACCUMULATE) ? a.y[n] + sum : sum;
       }
       if (tid == 0)  // ready for the next call
@@ -603,13 +600,17 @@ Q3SplitPlan q3_split_plan(int cus, int G, int gpr, int ntiles, int rows_out, boo
   const size_t tile_floats = (size_t)ntiles * rows_out * 64;
   int nsplit = single_round ? max_split : hq_tune(HQ_TUNE_Q3_KSPLIT, 0);
   if (nsplit <= 0) {
-    // Up to eight rounds of K: one workgroup per round.  Single-round workgroups need half the registers,
-    // so two share a CU and one's reduction tail runs under the other's loads, and 2-8 times as many
-    // workgroups spread evenly over the CUs whatever the tile count (batch 1 at K=8192: N=22016, 344 tiles,
-    // 20.4 -> 15.1 us; N=28672, 448 tiles, 21.4 -> 18.6 us; K=28672, N=8192 21.7 -> 19.6 us).  Longer K: only
-    // as many splits as it takes to give every CU a workgroup - each split adds a partial-sum row per tile
-    // and a device-scope round trip (K=49152, N=12288: 43 us unsplit, 51-58 us split).
-    nsplit = max_split <= 8 ? max_split : cus / ntiles;
+    // One workgroup per round of K.  Single-round workgroups need half the registers, so two share a CU and
+    // one's reduction tail runs under the other's loads, and the workgroups spread evenly over the CUs
+    // whatever the tile count (batch 1 at K=8192: N=22016, 344 tiles, 20.4 -> 15.1 us; N=28672, 448 tiles,
+    // 21.4 -> 18.6 us; K=28672, N=8192 21.7 -> 19.6 us).  A plain grid of short workgroups also streams faster
+    // than workgroups that walk K (K=49152, N=12288, 192 tiles: 40.2 against 43.0 us; K=40960, N=22016,
+    // 344 tiles: 57.4 against 70.7; K=36864, N=20480: 49.3 against 62.6), except beyond eight rounds where the
+    // unsplit workgroups would fill the CUs evenly anyway and the exchange is all a split adds (K=36864,
+    // N=16384, 256 tiles: 37.8 unsplit, 39.4 split).
+    const int per_cu = (ntiles + cus - 1) / cus;
+    const bool even = (size_t)ntiles * 20 >= (size_t)per_cu * cus * 19;
+    nsplit = (max_split <= 8 || !even) ? max_split : 1;
     if (fixed && nsplit > 1 && (tile_floats * nsplit > fixed->partial_floats || (size_t)ntiles > fixed->ncounters))
       nsplit = cus / ntiles;  // the fixed scratch is too small for the full split
   }

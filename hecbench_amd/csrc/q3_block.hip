@@ -347,10 +347,8 @@ __device__ __forceinline__ void q3_block_body(const BlockArgs& a, const int tile
     if (s_last) {
       if (ncol < a.N) {
         for (int m = tid >> 6; m < M; m += kWaves) {
-          float sum = 0.f;
-          for (int s = 0; s < a.nsplit; ++s)
-            sum += __hip_atomic_load(&a.partial[(((size_t)vtile * a.nsplit + s) * a.prow + m) * 64 + col], __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_AGENT);
+          const float sum = hq_sum_partials(&a.partial[((size_t)vtile * a.nsplit * a.prow + m) * 64 + col],
+                                            (size_t)a.prow * 64, a.nsplit);
           float* yp = &a.y[(size_t)m * a.N + ncol];
           *yp = (a.flags & HQ_FLAG_ACCUMULATE) ? *yp + sum : sum;
         }
