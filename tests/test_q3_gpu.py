@@ -187,10 +187,11 @@ def test_default_k_split_on_long_k(hq, oracle, tunable, K, N):
 
 @pytest.mark.parametrize("K,N,x_dtype", [(36864, 16384, np.float32), (33792, 16388, np.float16), (36864, 4096, np.float32)])
 def test_more_than_eight_rounds_of_k(hq, oracle, tunable, K, N, x_dtype):
-    """Workgroups that walk several rounds of K: a workgroup on every compute unit (256 and 257 tiles, the last
-    one 4 columns wide: the next round's loads go out a step at a time), a K the rounds do not divide, and
-    64 tiles with K split four ways.  Sampled columns against the oracle, every column against a different
-    split, the same bits on a second call."""
+    """More than eight rounds of K.  256 tiles fill the compute units evenly: unsplit workgroups walk the
+    rounds, the next round's loads going out a step at a time.  257 tiles (the last one 4 columns wide, a K the
+    rounds do not divide) and 64 tiles do not: one workgroup per round, nine partial sums per tile, added up
+    in two batches of loads.  Sampled columns against the oracle, every column against a three-way split whose
+    workgroups walk several rounds, the same bits on a second call."""
     rng = np.random.default_rng(K + N)
     mat = rng.integers(-2 ** 31, 2 ** 31, size=(3 * K // 32, N), dtype=np.int64).astype(np.int32)
     scales = rng.uniform(0.005, 0.02, size=N).astype(np.float32)
