@@ -303,7 +303,17 @@ __global__ __launch_bounds__(256) void q3_gemm_reduce(GemmArgs a, int Mpad) {
   for (int m = blockIdx.y * 8 + (threadIdx.x >> 5); m < a.M; m += gridDim.y * 8) {
     const float* p = a.partial + (((size_t)tile * a.nsplit) * Mpad + m) * kTileN + 4 * nl;
     f4v v = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < a.nsplit; ++s) v += __builtin_nontemporal_load(reinterpret_cast<const f4v*>(p + (size_t)s * Mpad * kTileN));
+    for (int s0 = 0; s0 < a.nsplit; s0 += 8) {  // eight loads in flight, added in split order
+      f4v t[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int s = s0 + j < a.nsplit ? s0 + j : a.nsplit - 1;
+        t[j] = __builtin_nontemporal_load(reinterpret_cast<const f4v*>(p + (size_t)s * Mpad * kTileN));
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (s0 + j < a.nsplit) v += t[j];
+    }
     const float ri = a.rowinv[m] * 16777216.f, rs = a.rowsum[m];
     f4v o;
 #pragma unroll
