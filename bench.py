@@ -175,6 +175,62 @@ def measure_device():
     return out
 
 
+def lds_patterns():
+    """(name, width in bits, write, byte offset per lane) of the LDS access patterns hq_probe_lds is run on:
+    patterns whose conflicts are known, and the operand layouts of the matvec kernels (lane = 16 * quarter + c)."""
+    lanes = range(64)
+    c = lambda l: l & 15
+    kb = lambda l: l >> 4
+    piece = lambda row, quarter, half: 16 * row + 512 * quarter + 176 * half   # q3.hip dig_piece
+    xs = lambda l: (l >> 3) & 3
+    xkb = lambda l: ((l >> 2) & 1) * 2 + (l >> 5)
+    pats = [
+        ("read b32, consecutive words", 32, 0, [4 * l for l in lanes]),
+        ("read b64, consecutive", 64, 0, [8 * l for l in lanes]),
+        ("read b128, consecutive", 128, 0, [16 * l for l in lanes]),
+        ("read b32, 8 bytes apart (two lanes of a pass per bank)", 32, 0, [8 * l for l in lanes]),
+        ("read b32, 128 bytes apart (a pass in one bank)", 32, 0, [(128 * l) % 8192 for l in lanes]),
+        ("read b128, 256 bytes apart (a pass in one bank group)", 128, 0, [(256 * l) % 8192 for l in lanes]),
+        ("write b32, consecutive words", 32, 1, [4 * l for l in lanes]),
+        ("write b128, consecutive", 128, 1, [16 * l for l in lanes]),
+        ("read b128, 3-bit matvec digit operand in rows of 144 bytes (the former layout)", 128, 0,
+         [min(c(l), 8) * 144 + kb(l) * 32 for l in lanes]),
+        ("read b128, 3-bit matvec digit operand, first half (q3.hip)", 128, 0,
+         [piece(c(l) if c(l) < 8 else 8 + (kb(l) & 1), kb(l), 0) for l in lanes]),
+        ("read b128, 3-bit matvec digit operand, second half, step 3", 128, 0,
+         [3 * 1888 + piece(c(l) if c(l) < 8 else 8 + (kb(l) & 1), kb(l), 1) for l in lanes]),
+        ("write b32, 3-bit matvec digit staging, row 0 even elements", 32, 1,
+         [xs(l) * 1888 + piece(0, 2 * (xkb(l) & 1), xkb(l) >> 1) + 4 * (l & 3) for l in lanes]),
+        ("write b32, 3-bit matvec digit staging, row 1 odd elements", 32, 1,
+         [xs(l) * 1888 + piece(1, 2 * (xkb(l) & 1) + 1, xkb(l) >> 1) + 4 * (l & 3) for l in lanes]),
+    ]
+    return pats
+
+
+def lds_probe(repeats=4096, launches=20):
+    """hq_probe_lds on every pattern of lds_patterns(), `launches` launches each, in that order (a profiler's
+    dispatches can be matched by order); microseconds per launch."""
+    import torch
+    from hecbench_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {"repeats_per_lane": repeats, "launches": launches, "patterns": []}
+    for name, width, write, offs in lds_patterns():
+        table = torch.tensor(offs, dtype=torch.int32, device=dev)
+
+        def call(_i):
+            rc = lib.hq_probe_lds(ctypes.c_void_p(table.data_ptr()), width, write, repeats,
+                                  ctypes.c_void_p(sink.data_ptr()), stream)
+            if rc:
+                raise RuntimeError("hq_probe_lds: " + lib.hq_strerror(rc).decode())
+        secs = _time_windows(call, 1, launches, 2, 3)
+        out["patterns"].append({"name": name, "width": width, "write": write,
+                                "us_per_launch": round(_summary(secs, launches)[0], 2)})
+    return out
+
+
 def bench_q3(steps, warmup, windows, hot=False):
     import torch
     from hecbench_amd import _lib
@@ -681,6 +737,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 20 plain device copies of 256 MiB (reference point for rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--lds-probe", action="store_true",
+                    help="run only hq_probe_lds, every pattern 20 times (LDS accesses whose bank conflicts are "
+                         "known, for reading rocprofv3's SQ_LDS_BANK_CONFLICT against them), and print their times")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this path has no collective and every box here has one GPU; "
@@ -697,6 +756,10 @@ def main():
     hq.init()
     info = hq.device_info()
     windows = _windows_for(args.steps, args.windows)
+
+    if args.lds_probe:
+        print(json.dumps(lds_probe()))
+        return
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_()

@@ -54,6 +54,7 @@ _SIGNATURES = {
     "hq_probe_stream": (_c.c_int, [_c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p]),
     "hq_probe_gather16": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_void_p]),
     "hq_probe_gather16_count": (_c.c_int64, [_c.c_int64]),
+    "hq_probe_lds": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_int, _c.c_int, _c.c_void_p, _c.c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

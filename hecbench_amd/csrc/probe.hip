@@ -4,6 +4,9 @@
 //   hq_probe_gather16: independent 16-byte reads at pseudo-random entries of a table (the access
 //                      pattern of a code-book lookup), the rate of which is bounded by cache requests per
 //                      second, not by bytes.
+//   hq_probe_lds: LDS reads or writes of 32, 64 or 128 bits per lane at byte offsets the caller gives per
+//                 lane, so that the hardware's bank-conflict counter can be read against patterns whose
+//                 conflicts are known (and the operand layouts of the library's kernels checked with it).
 // There is no counterpart in the HeCBench tree; the benchmark drivers call them for their report.
 #include "hq_internal.h"
 
@@ -39,6 +42,41 @@ __global__ __launch_bounds__(256) void probe_gather_kernel(const u4v* __restrict
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) acc ^= v[u];
+  }
+  if ((acc.x & acc.y & acc.z & acc.w) == 0xffffffffu && acc.x + acc.y == 12345u) *sink = acc;
+}
+
+// Every lane repeats one LDS access of WIDTH bits at its own byte offset (taken from a table of 64 offsets,
+// the same for every wave) inside its wave's 8 KB.
+template <int WIDTH, bool WRITE>
+__global__ __launch_bounds__(256) void probe_lds_kernel(const uint32_t* __restrict__ offsets, int repeats,
+                                                       u4v* __restrict__ sink) {
+  __shared__ u4v buf[2048 + 256];  // 32 KB and a margin for the widest access at the last offset
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  for (int i = tid; i < 2048 + 256; i += 256) buf[i] = u4v{(uint32_t)i, 1u, 2u, 3u};
+  __syncthreads();
+  const uint32_t base = (uint32_t)(uintptr_t)buf + (uint32_t)wv * 8192u + (offsets[lane] & 8191u & ~(uint32_t)(WIDTH / 8 - 1));
+  u4v acc = {0u, 0u, 0u, 0u};
+  for (int r = 0; r < repeats; ++r) {
+    const uint32_t p = base;
+    if (WRITE) {
+      const u4v v = {acc.x + (uint32_t)r, 1u, 2u, 3u};
+      if (WIDTH == 32) asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(p), "v"(v.x) : "memory");
+      else if (WIDTH == 64) asm volatile("ds_write_b64 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(p), "v"(((uint64_t)v.y << 32) | v.x) : "memory");
+      else asm volatile("ds_write_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(p), "v"(v) : "memory");
+    } else if (WIDTH == 32) {
+      uint32_t v;
+      asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+      acc.x ^= v;
+    } else if (WIDTH == 64) {
+      uint64_t v;
+      asm volatile("ds_read_b64 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+      acc.x ^= (uint32_t)v; acc.y ^= (uint32_t)(v >> 32);
+    } else {
+      u4v v;
+      asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+      acc ^= v;
+    }
   }
   if ((acc.x & acc.y & acc.z & acc.w) == 0xffffffffu && acc.x + acc.y == 12345u) *sink = acc;
 }
@@ -89,4 +127,25 @@ extern "C" int64_t hq_probe_gather16_count(int64_t gathers) {
   long per_lane = (gathers + lanes - 1) / lanes;
   per_lane = (per_lane + 7) / 8 * 8;
   return per_lane * lanes;
+}
+
+extern "C" int hq_probe_lds(const uint32_t* offsets64, int width_bits, int write, int repeats, void* sink16,
+                            void* stream) {
+  if (!offsets64 || !sink16) return HQ_ERR_NULL_POINTER;
+  if (width_bits != 32 && width_bits != 64 && width_bits != 128) return HQ_ERR_BAD_ENUM;
+  if (repeats <= 0 || repeats > (1 << 20)) return HQ_ERR_BAD_SHAPE;
+  if (((uintptr_t)sink16 & 15) || ((uintptr_t)offsets64 & 3)) return HQ_ERR_MISALIGNED;
+  const HqDevice* dev = nullptr;
+  const int rc = hq_current_device(&dev);
+  if (rc != HQ_OK) return rc;
+  const dim3 grid((unsigned)dev->cus), block(256);
+#define HQ_PROBE_LDS(W, WR) \
+  hipLaunchKernelGGL((probe_lds_kernel<W, WR>), grid, block, 0, (hipStream_t)stream, offsets64, repeats, (u4v*)sink16)
+  if (write) {
+    if (width_bits == 32) HQ_PROBE_LDS(32, true); else if (width_bits == 64) HQ_PROBE_LDS(64, true); else HQ_PROBE_LDS(128, true);
+  } else {
+    if (width_bits == 32) HQ_PROBE_LDS(32, false); else if (width_bits == 64) HQ_PROBE_LDS(64, false); else HQ_PROBE_LDS(128, false);
+  }
+#undef HQ_PROBE_LDS
+  return hq_launch_status();
 }

@@ -305,10 +305,16 @@ int hq_mxfp4_qdq(const void* in, void* out, int64_t n_elems, int dtype, void* st
  *     of a code-book lookup, bounded by cache requests per second; sink16 is a 16-byte buffer that is
  *     never written in practice.  hq_probe_gather16_count(gathers) returns the exact number of reads that
  *     call performs on the current device (the request rounded up to whole trips of every lane).
+ *   hq_probe_lds(offsets64, width_bits, write, repeats, sink16, stream): one workgroup of four waves per compute
+ *     unit; lane l of every wave repeats one LDS access of width_bits (32, 64 or 128) bits, a read or (write != 0)
+ *     a write, at byte offset offsets64[l] (device array of 64 offsets below 8192 - 16, multiples of the access size)
+ *     inside its wave's own LDS region - the lane pattern of any kernel's LDS operand can be put under a
+ *     profiler's bank-conflict counter next to patterns whose conflicts are known.
  */
 int hq_probe_stream(int mode, const void* src, void* dst, int64_t bytes, void* stream);
 int hq_probe_gather16(const void* table, int64_t table_bytes, int64_t gathers, void* sink16, void* stream);
 int64_t hq_probe_gather16_count(int64_t gathers);
+int hq_probe_lds(const uint32_t* offsets64, int width_bits, int write, int repeats, void* sink16, void* stream);
 
 #ifdef __cplusplus
 }

@@ -49,3 +49,26 @@ def test_gather_probe(hq):
     assert lib.hq_probe_gather16(_vp(table), (1 << 20) - 16, want, _vp(sink), st) < 0   # not a power of two
     assert lib.hq_probe_gather16(_vp(table), 1 << 20, 0, _vp(sink), st) < 0
     assert lib.hq_probe_gather16(None, 1 << 20, want, _vp(sink), st) < 0
+
+
+def test_lds_probe(hq):
+    """Every pattern the benchmark runs is valid for the probe and leaves the sink alone; a conflict-free
+    pattern is faster than the one that puts a whole pass into one bank; bad arguments are rejected."""
+    import torch
+    import bench
+    from hecbench_amd import _lib
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sink = torch.full((16,), 5, dtype=torch.uint8, device="cuda:0")
+    for name, width, write, offs in bench.lds_patterns():
+        table = torch.tensor(offs, dtype=torch.int32, device="cuda:0")
+        assert lib.hq_probe_lds(_vp(table), width, write, 64, _vp(sink), st) == 0, name
+    torch.cuda.synchronize()
+    assert bool((sink == 5).all())
+    res = {p["name"]: p["us_per_launch"] for p in bench.lds_probe(repeats=2048, launches=5)["patterns"]}
+    assert res["read b32, 128 bytes apart (a pass in one bank)"] > 1.5 * res["read b32, consecutive words"], res
+    table = torch.zeros(64, dtype=torch.int32, device="cuda:0")
+    assert lib.hq_probe_lds(_vp(table), 48, 0, 64, _vp(sink), st) < 0        # no such width
+    assert lib.hq_probe_lds(_vp(table), 32, 0, 0, _vp(sink), st) < 0         # no repeats
+    assert lib.hq_probe_lds(None, 32, 0, 64, _vp(sink), st) < 0
+    assert lib.hq_probe_lds(_vp(table), 32, 0, 64, None, st) < 0
