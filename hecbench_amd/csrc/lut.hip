@@ -293,7 +293,18 @@ __device__ __forceinline__ f4 mfma_fp8_fp4(v8i a, v8i b, f4 c) {
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 4, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
 }
 
-constexpr int kDigQuad = 4 * 4 * 32 + 16;  // digits of one quad [k-word][digit][32 operand bytes], then 16 zero bytes
+// LDS layout of a quad's digits: 32 operand bytes per (k-word, digit) as two 16-byte pieces, and a piece of
+// zeros.  Placed by the bank rules measured on this part (a 128-bit read is served in passes of 16 lanes - lanes
+// 0-3, 12-15, 20-27 / 4-11, 16-19, 28-31 of each half wave - over 256 bytes of banks; narrower stores in passes
+// of 32 lanes over 128 bytes): k-words 80 bytes apart, digits 16, the second pieces 336 bytes behind the first,
+// the zeros at byte 144, quads 704 bytes apart.  Neither an operand read (one, two or three planes per set) nor
+// a staging store meets another in a bank (with rows of 32 bytes, 128 bytes per k-word, the stores of the four
+// k-words fell into one bank and a quarter of the LDS cycles were conflicts).
+constexpr int kDigQuad = 704;
+constexpr int kDigZero = 144;
+__device__ __forceinline__ constexpr int dig_piece(int kword, int digit, int half) {
+  return 80 * kword + 16 * digit + 336 * half;
+}
 constexpr int planes_of_set(int nb, int s) { return nb - 3 * s < 3 ? nb - 3 * s : 3; }
 
 template <int NB, int QUADS, int WAVES, bool BIAS, bool RAGGED, bool ONE_ROUND>
@@ -325,7 +336,7 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(
   // 4*(e & 7) + (e >> 3) of the word, so activation 8*(sm & 3) + i of k-word sm >> 2 is element
   // 8*(i & 3) + 2*(sm & 3) + (i >> 2): activations i and i + 4 are neighbours in a digit row.
   const int st = lane >> 4, sm = lane & 15;
-  const int stage_off = (sm >> 2) * 128 + 2 * (sm & 3);
+  const int stage_off = dig_piece(sm >> 2, 0, 0) + 2 * (sm & 3);
 
   // what a lane multiplies its combined digits with, per set: alpha of plane 3s + kb, the bias (quarter 3
   // of set 0) or nothing (then its sums are zero)
@@ -401,7 +412,6 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(
   // Digit operand reads.  The fp8 operand of lane quarter kb holds MFMA K indices 16kb .. 16kb+15 in its
   // first 16 bytes and 64+16kb .. 64+16kb+15 in its last 16: halves h = 0, 1 lie in block 2h + (kb >> 1),
   // elements 16*(kb & 1) .. +15 of it.  Row c = 4b + d takes digit d there if the block's plane is b.
-  const int half_off = 16 * (kb & 1);
   int doff[SETS][3][2];
 #pragma unroll
   for (int s = 0; s < SETS; ++s) {
@@ -412,16 +422,16 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(
       for (int h = 0; h < 2; ++h) {
         const int jj = 4 * m + 2 * h + (kb >> 1);
         const int b = jj % P, kw = jj / P;
-        doff[s][m][h] = (m < P && (c >> 2) == b) ? (kw * 4 + (c & 3)) * 32 + half_off : 512;
+        doff[s][m][h] = (m < P && (c >> 2) == b) ? dig_piece(kw, c & 3, kb & 1) : kDigZero;
       }
   }
   // plain operand (every row r holds digit r & 3 of all four k-words): one MFMA with all-ones weights
   // gives the digit sums of the quad in every lane
-  const int poff0 = ((kb >> 1) * 4 + (c & 3)) * 32 + half_off, poff1 = poff0 + 2 * 128;
+  const int poff0 = dig_piece(kb >> 1, c & 3, kb & 1), poff1 = dig_piece((kb >> 1) + 2, c & 3, kb & 1);
   v8i ones;
 #pragma unroll
   for (int r = 0; r < 8; ++r) ones[r] = r < 4 ? 0x11111111 : 0;
-  if (lane < 4 * QUADS) *reinterpret_cast<uint32_t*>(xs_w + (lane >> 2) * kDigQuad + 512 + (lane & 3) * 4) = 0u;
+  if (lane < 4 * QUADS) *reinterpret_cast<uint32_t*>(xs_w + (lane >> 2) * kDigQuad + kDigZero + (lane & 3) * 4) = 0u;
 
   constexpr int STRIDE = WAVES * QUADS;
   auto compute_round = [&](int q0, Round& r, Round& next) {
@@ -459,10 +469,11 @@ __global__ __launch_bounds__(WAVES * 64) void bcq_planes_kernel(
           // digits of activations i and i + 4 side by side: bytes (d0, d0', d2, d2') and (d1, d1', d3, d3')
           const uint32_t pe = __builtin_amdgcn_perm(ev[i + 4], ev[i], 0x05010400u);
           const uint32_t po = __builtin_amdgcn_perm(od[i + 4], od[i], 0x05010400u);
-          *reinterpret_cast<uint16_t*>(dst + 0 * 32 + 8 * i) = (uint16_t)pe;
-          *reinterpret_cast<uint16_t*>(dst + 1 * 32 + 8 * i) = (uint16_t)po;
-          *reinterpret_cast<uint16_t*>(dst + 2 * 32 + 8 * i) = (uint16_t)(pe >> 16);
-          *reinterpret_cast<uint16_t*>(dst + 3 * 32 + 8 * i) = (uint16_t)(po >> 16);
+          const int at = dig_piece(0, 0, i >> 1) + 8 * (i & 1);  // byte 8 * i of the row's 32
+          *reinterpret_cast<uint16_t*>(dst + dig_piece(0, 0, 0) + at) = (uint16_t)pe;
+          *reinterpret_cast<uint16_t*>(dst + dig_piece(0, 1, 0) + at) = (uint16_t)po;
+          *reinterpret_cast<uint16_t*>(dst + dig_piece(0, 2, 0) + at) = (uint16_t)(pe >> 16);
+          *reinterpret_cast<uint16_t*>(dst + dig_piece(0, 3, 0) + at) = (uint16_t)(po >> 16);
         }
       }
     }
