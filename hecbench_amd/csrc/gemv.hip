@@ -254,6 +254,15 @@ __global__ __launch_bounds__(SPLIT * 64) void gemv_split_kernel(const char* mat_
 // place in that queue from the matrix.  Here a workgroup of sixteen waves copies the vector into LDS once
 // (piece i of matrix unit u at [i][u], so that a wave's reads of one piece are contiguous) and then walks
 // over groups of R rows, one group per wave and trip, with nothing but the matrix in the load queue.
+// Units between the pieces of the vector in LDS: the row length rounded up to 8 / kVecUnits past a multiple of
+// eight units.  The copy writes piece i of unit u from consecutive lanes (u = t / kVecUnits, i = t % kVecUnits);
+// a 128-bit LDS store is served eight lanes at a time over 128 bytes of banks, and with the pieces a multiple
+// of 128 bytes apart the pieces of one unit met in a bank.
+template <int MODE>
+__host__ __device__ constexpr int gemv_lds_stride(int units) {
+  return (units + 7) / 8 * 8 + 8 / Geom<MODE>::kVecUnits % 8;
+}
+
 template <int MODE, int R>
 __global__ __launch_bounds__(1024) void gemv_lds_kernel(const char* mat_, const u4v* vec_, _Float16* res_, int rows_, int n_, float scale_,
                                                        float zp_, int groups) {
@@ -264,6 +273,7 @@ __global__ __launch_bounds__(1024) void gemv_lds_kernel(const char* mat_, const 
   extern __shared__ u4v vl[];
   const int lane = threadIdx.x & 63;
   const int units = a.n / G::kPerUnit;  // 16-byte units per matrix row
+  const int vstride = gemv_lds_stride<MODE>(units);
   const size_t row_bytes = (size_t)units * 16;
   const int waves = gridDim.x * 16;
   int grp = blockIdx.x * 16 + (threadIdx.x >> 6);
@@ -281,7 +291,7 @@ __global__ __launch_bounds__(1024) void gemv_lds_kernel(const char* mat_, const 
   for (int r = 0; r < R; ++r) m[r] = __builtin_nontemporal_load(rowp[r] + min(lane, units - 1));
   for (int t = threadIdx.x; t < units * G::kVecUnits; t += 1024) {
     const int u = t / G::kVecUnits, i = t % G::kVecUnits;
-    vl[i * units + u] = a.vec[t];
+    vl[i * vstride + u] = a.vec[t];
   }
   __syncthreads();
 
@@ -301,7 +311,7 @@ __global__ __launch_bounds__(1024) void gemv_lds_kernel(const char* mat_, const 
 #pragma unroll
       for (int r = 0; r < R; ++r) m[r] = __builtin_nontemporal_load(rowp[r] + un);
 #pragma unroll
-      for (int i = 0; i < G::kVecUnits; ++i) v[i] = vl[i * units + u];
+      for (int i = 0; i < G::kVecUnits; ++i) v[i] = vl[i * vstride + u];
       if (first) gemv_step<MODE, R, true>(cur, v, acc, acc16, vsum);
       else gemv_step<MODE, R, false>(cur, v, acc, acc16, vsum);
     }
@@ -315,9 +325,9 @@ constexpr size_t kMaxVectorLds = 128 * 1024;  // bytes of the vector the LDS ker
 
 template <int MODE, int R>
 int launch_gemv_lds(const GemvArgs& a, int cus, hipStream_t stream) {
-  const size_t smem = (size_t)a.n * 2;
+  const size_t smem = (size_t)gemv_lds_stride<MODE>(a.n / Geom<MODE>::kPerUnit) * Geom<MODE>::kVecUnits * 16;
   static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemv_lds_kernel<MODE, R>),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxVectorLds);
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxVectorLds + 1024);
   if (attr != hipSuccess) return (int)attr;
   const int groups = (a.rows + R - 1) / R;
   const int wgs = (groups + 15) / 16;
