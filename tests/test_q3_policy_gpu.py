@@ -13,6 +13,7 @@ WINDOWS = 5
 # candidates: name -> knobs; "default" (no knob) is what the library does by itself
 MATVEC = {"default": {}, "unsplit": {"HQ_Q3_KSPLIT": 1}, "tiles32": {"HQ_Q3_TILE": 2}, "waves4": {"HQ_Q3_WAVES": 4},
           "steps2": {"HQ_Q3_STEPS": 2}}
+LONG_K = {"default": {}, "unsplit": {"HQ_Q3_KSPLIT": 1}, "three_ranges": {"HQ_Q3_KSPLIT": 3}}
 BATCH = {"default": {}, "gemm": {"HQ_Q3_SMALL_BATCH": 0}, "passes": {"HQ_Q3_ROW_BLOCKS": 0},
          "row_blocks": {"HQ_Q3_ROW_BLOCKS": 1}}
 CASES = [
@@ -24,6 +25,8 @@ CASES = [
     (4096, 4096, 12, BATCH),
     (8192, 28672, 16, BATCH),
     (8192, 28672, 64, BATCH),
+    (36864, 11008, 1, LONG_K),     # nine rounds of K, 172 column tiles: one workgroup per round
+    (36864, 16384, 1, LONG_K),     # 256 tiles fill the compute units evenly: unsplit workgroups walk the rounds
 ]
 
 
